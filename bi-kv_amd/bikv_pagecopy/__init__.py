@@ -1,0 +1,15 @@
+"""bikv_pagecopy — host side of the MI355X KV page-copy path (gather / scatter / host staging).
+
+Thin Python over libbikv_pagecopy.so (HIP, gfx950). PyTorch supplies device memory and streams only.
+"""
+from . import _lib
+from ._lib import load, set_tuning
+from .offsets import build_run_offsets
+from .pool import LAYER_MAJOR, PAGE_MAJOR, PageBatch, PagedKVPool, build_index
+from .runs import copy_runs
+from .staging import HostStager, measure_d2h, pinned_empty, plan_chunks
+
+__all__ = [
+    "load", "set_tuning", "build_run_offsets", "LAYER_MAJOR", "PAGE_MAJOR", "PageBatch", "PagedKVPool",
+    "build_index", "copy_runs", "HostStager", "measure_d2h", "pinned_empty", "plan_chunks",
+]

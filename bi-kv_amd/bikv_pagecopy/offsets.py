@@ -1,0 +1,52 @@
+"""Offset tables for the run copy, built from the coordinator's page lists.
+
+Mirror of the index stage of KVCache.shared_data_batch_pages
+(Bi-KV/DistributedStorage/kvcache.py:161-196): `cache_pages_list[k]` holds the page ids of item k
+and `id_token_pair[k][1]` its token count; every page becomes one run whose source offset is
+`page * page_size` and whose destination offset is the running sum of the page sizes, where the
+last page of an item counts only `tokens % page_size` tokens when that is non-zero.
+
+The reference computes these offsets in TOKENS and hands them to a kernel that reads them as
+ELEMENTS (copy_kernel.cu:22-33), so as shipped it copies from the wrong place; the two reference
+scripts that exercise the kernel pass element offsets (test_page_ipc.py:58-65). `unit="elements"`
+(default) multiplies by elements_per_token and is what a correct caller needs; `unit="tokens"`
+reproduces the reference's literal numbers.
+
+The reference builds the lists with two nested Python loops and two `torch.tensor(list)` uploads;
+this builder is vectorised numpy and produces one [2, n] array for a single upload.
+"""
+from typing import Sequence, Tuple
+
+import numpy as np
+
+
+def build_run_offsets(cache_pages_list: Sequence[Sequence[int]], item_tokens: Sequence[int],
+                      page_size: int, elements_per_token: int = 1,
+                      unit: str = "elements") -> Tuple[np.ndarray, int]:
+    """Returns (offsets, total_tokens): offsets[0] = source offsets, offsets[1] = destination offsets,
+    both int64, one entry per page in list order; total_tokens = sum of the copied page sizes."""
+    if unit not in ("elements", "tokens"):
+        raise ValueError("unit must be 'elements' or 'tokens'")
+    if page_size <= 0:
+        raise ValueError("page_size must be positive")
+    if len(cache_pages_list) != len(item_tokens):
+        raise ValueError("cache_pages_list and item_tokens differ in length")
+    counts = np.fromiter((len(p) for p in cache_pages_list), dtype=np.int64, count=len(cache_pages_list))
+    n = int(counts.sum())
+    out = np.empty((2, n), dtype=np.int64)
+    if n == 0:
+        return out, 0
+    pages = np.concatenate([np.asarray(p, dtype=np.int64).reshape(-1) for p in cache_pages_list if len(p)])
+    tokens = np.asarray(item_tokens, dtype=np.int64)
+    sizes = np.full(n, page_size, dtype=np.int64)
+    last = np.cumsum(counts) - 1                      # index of each item's last page
+    has = counts > 0
+    tail = tokens % page_size
+    partial = has & (tail != 0)
+    sizes[last[partial]] = tail[partial]
+    dst = np.zeros(n, dtype=np.int64)
+    np.cumsum(sizes[:-1], out=dst[1:])
+    scale = elements_per_token if unit == "elements" else 1
+    out[0] = pages * page_size * scale
+    out[1] = dst * scale
+    return out, int(sizes.sum())

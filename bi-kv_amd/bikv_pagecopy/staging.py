@@ -1,0 +1,87 @@
+"""Device -> pinned-host staging of gathered pages.
+
+The reference stages outgoing KV in host tensors allocated per call (Bi-KV/DistributedStorage/
+kvcache.py:105-108, Bi-KV/Worker/Worker.py:203-206) which the RDMA endpoint then sends from a
+pinned region (Bi-KV/NetworkTransport/onesided_rdma.h:301-337). HostStager fills such a pinned
+region straight from the paged pool: chunked gather on one HIP stream overlapped with
+hipMemcpyAsync on another (mode "pipelined"), or kernel stores directly into the mapped pinned
+buffer (mode "direct").
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import _lib
+from .pool import PagedKVPool, PageBatch, _LAYOUT_CODE
+
+_MODES = {"pipelined": _lib.STAGE_PIPELINED, "direct": _lib.STAGE_DIRECT}
+
+
+def pinned_empty(nbytes: int) -> torch.Tensor:
+    """A pinned host byte buffer (torch allocates it with hipHostMalloc)."""
+    return torch.empty(int(nbytes), dtype=torch.uint8, pin_memory=True)
+
+
+class HostStager:
+    def __init__(self, device, chunk_bytes: int = 8 << 20, n_buffers: int = 3):
+        self.device = torch.device(device)
+        self.chunk_bytes = int(chunk_bytes)
+        self.n_buffers = int(n_buffers)
+        idx = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        self._device_index = idx
+        h = C.c_void_p()
+        _lib.check(_lib.load().bikv_stager_create(idx, self.chunk_bytes, self.n_buffers, C.byref(h)))
+        self._h = h
+
+    def gather_to_host(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "pipelined"):
+        """Fills `host` (pinned) with the staging image of `batch`; returns (bytes, chunks, seconds)."""
+        if mode not in _MODES:
+            raise ValueError(f"unknown mode {mode!r}")
+        if host.is_cuda or not host.is_pinned():
+            raise RuntimeError("CPU data must be pinned memory")  # message of copy_kernel.cu:142
+        if not host.is_contiguous():
+            raise RuntimeError("host staging buffer must be contiguous")
+        # work queued on the caller's stream (e.g. the upload of the index arrays) must be visible
+        torch.cuda.current_stream(self.device).synchronize()
+        d = batch.desc()
+        stats = _lib.StageStats()
+        rp = batch.req_pages.ctypes.data_as(C.POINTER(C.c_int64))
+        _lib.check(_lib.load().bikv_gather_to_host(
+            self._h, pool._h, C.byref(d), rp, len(batch.req_pages), _LAYOUT_CODE[batch.layout],
+            host.data_ptr(), host.numel() * host.element_size(), _MODES[mode], C.byref(stats)))
+        return stats.bytes, stats.n_chunks, stats.wall_seconds
+
+    def close(self):
+        if getattr(self, "_h", None):
+            _lib.load().bikv_stager_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def plan_chunks(req_pages, n_planes: int, layout: str, max_slots: int) -> np.ndarray:
+    """The chunk plan of the pipelined mode as an [n_chunks, 6] int64 array:
+    (first_page, n_pages, plane_begin, plane_count, first_slot, n_slots). Pure host logic."""
+    lib = _lib.load()
+    rp = np.ascontiguousarray(req_pages, dtype=np.int64)
+    ptr = rp.ctypes.data_as(C.POINTER(C.c_int64))
+    n = _lib.check(lib.bikv_plan_chunks(ptr, len(rp), n_planes, _LAYOUT_CODE[layout], max_slots, None, 0))
+    out = np.zeros((max(n, 1), 6), dtype=np.int64)
+    _lib.check(lib.bikv_plan_chunks(ptr, len(rp), n_planes, _LAYOUT_CODE[layout], max_slots,
+                                    out.ctypes.data_as(C.POINTER(C.c_int64)), n))
+    return out[:n]
+
+
+def measure_d2h(device, host: torch.Tensor, dev: torch.Tensor, chunk_bytes: int = 0) -> float:
+    """Seconds for a plain hipMemcpyAsync of dev -> host (pinned): the host-link yardstick."""
+    idx = torch.device(device).index or 0
+    nbytes = min(host.numel() * host.element_size(), dev.numel() * dev.element_size())
+    sec = C.c_double()
+    torch.cuda.synchronize(device)
+    _lib.check(_lib.load().bikv_d2h_copy(idx, host.data_ptr(), dev.data_ptr(), nbytes, chunk_bytes, C.byref(sec)))
+    return sec.value

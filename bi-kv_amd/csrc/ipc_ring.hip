@@ -1,0 +1,297 @@
+// Producer/consumer ring of the `ipc_service` operator: a control block in POSIX shared memory,
+// a device ring buffer owned by the consumer, and the producer-side bookkeeping that follows every
+// copy. Behaviour follows Bi-KV/SharedMemory/CUDA_Shared/ipc_service.cpp:20-202 (init, send,
+// receive, cleanup) and copy_kernel.cu:84-89,115-128 (ring advance and shape publishing).
+//
+// Deliberate differences from the reference, all on error paths or internal:
+//   - sizes are 64-bit and use the real element size (reference: int, sizeof(half));
+//   - a batch larger than the whole ring is refused (reference: wraps to 0 and overruns);
+//   - the copy is awaited with a stream synchronise (reference: cudaDeviceSynchronize);
+//   - a producer in the consumer's own process uses the consumer's pointer instead of opening an
+//     IPC handle (a process cannot open its own handle);
+//   - consumer_receive can time out.
+#include "../../include/bikv_pagecopy.h"
+#include "pagecopy_internal.h"
+#include "pagecopy_kernels.h"
+
+#include <cerrno>
+#include <cstring>
+#include <ctime>
+#include <fcntl.h>
+#include <semaphore.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+using namespace bikv;
+
+static_assert(sizeof(sem_t) == 32, "sem_t is 32 bytes on x86-64 glibc; SharedControl depends on it");
+static_assert(sizeof(hipIpcMemHandle_t) <= BIKV_IPC_HANDLE_SIZE, "IPC handle must fit the control block");
+
+namespace {
+
+struct Role {
+  int fd = -1;
+  bikv_shared_control* ctrl = nullptr;
+  void* mem = nullptr;
+  int device = 0;
+  bool ipc_mapped = false;  // producer only: mem came from hipIpcOpenMemHandle
+  char shm_name[256] = "";
+};
+
+Role g_producer, g_consumer;
+
+sem_t* sem_of(unsigned char* raw) { return reinterpret_cast<sem_t*>(raw); }
+
+void unmap_role(Role& r) {
+  if (r.ctrl) {
+    munmap(r.ctrl, sizeof(bikv_shared_control));
+    r.ctrl = nullptr;
+  }
+  if (r.fd != -1) {
+    close(r.fd);
+    r.fd = -1;
+  }
+}
+
+// The reference's ring advance (copy_kernel.cu:87-89): a batch that does not fit behind the
+// current offset restarts at 0. Returns the write offset.
+size_t ring_reserve(bikv_shared_control* c, size_t data_size) {
+  if (c->current_offset + data_size > c->buffer_size) c->current_offset = 0;
+  return c->current_offset;
+}
+
+// The reference's publish step (copy_kernel.cu:116-128, ipc_service.cpp:130-142).
+void ring_publish(bikv_shared_control* c, size_t data_size, const int64_t* shape, size_t ndim,
+                  int32_t dtype_code) {
+  c->last_valid_offset = c->current_offset;
+  c->current_offset += data_size;
+  c->tensor_dim = ndim;
+  for (size_t i = 0; i < ndim && i < BIKV_MAX_DIM; ++i) c->tensor_shape[i] = shape[i];
+  c->data_size = data_size;
+  c->dtype_code = dtype_code;
+  sem_post(sem_of(c->sem_start));
+}
+
+}  // namespace
+
+extern "C" int bikv_consumer_init(int device, const char* shm_name, size_t buffer_bytes) {
+  if (!shm_name || !*shm_name) return fail(BIKV_EINVAL, "shm_name is empty");
+  if (strlen(shm_name) >= sizeof(g_consumer.shm_name)) return fail(BIKV_EINVAL, "shm_name too long");
+  if (buffer_bytes == 0) return fail(BIKV_EINVAL, "buffer_size must be positive");
+  if (g_consumer.ctrl) return fail(BIKV_ESTATE, "consumer already initialised (call consumer_cleanup first)");
+  BIKV_HIP(hipSetDevice(device));
+  Role r;
+  r.device = device;
+  strncpy(r.shm_name, shm_name, sizeof(r.shm_name) - 1);
+
+  shm_unlink(shm_name);  // make sure no stale object is left, as the reference does
+  r.fd = shm_open(shm_name, O_CREAT | O_RDWR | O_EXCL, 0666);
+  if (r.fd == -1) return fail(BIKV_ESYS, "consumer_init shm_open failed: %s", strerror(errno));
+  if (ftruncate(r.fd, sizeof(bikv_shared_control)) == -1) {
+    const int e = errno;
+    close(r.fd);
+    shm_unlink(shm_name);
+    return fail(BIKV_ESYS, "consumer_init ftruncate failed: %s", strerror(e));
+  }
+  void* m = mmap(nullptr, sizeof(bikv_shared_control), PROT_READ | PROT_WRITE, MAP_SHARED, r.fd, 0);
+  if (m == MAP_FAILED) {
+    const int e = errno;
+    close(r.fd);
+    shm_unlink(shm_name);
+    return fail(BIKV_ESYS, "consumer_init mmap failed: %s", strerror(e));
+  }
+  r.ctrl = static_cast<bikv_shared_control*>(m);
+  memset(r.ctrl, 0, sizeof(bikv_shared_control));
+  sem_init(sem_of(r.ctrl->sem_start), 1, 0);
+  sem_init(sem_of(r.ctrl->sem_complete), 1, 0);
+  gethostname(r.ctrl->hostname, sizeof(r.ctrl->hostname));
+  r.ctrl->current_offset = 0;
+  r.ctrl->last_valid_offset = 0;
+  r.ctrl->device_id = device;
+  r.ctrl->buffer_size = buffer_bytes;
+
+  hipError_t e = hipMalloc(&r.mem, buffer_bytes);
+  if (e != hipSuccess) {
+    unmap_role(r);
+    shm_unlink(shm_name);
+    return fail(BIKV_EHIP, "consumer_init hipMalloc failed: %s", hipGetErrorString(e));
+  }
+  hipIpcMemHandle_t handle;
+  memset(&handle, 0, sizeof(handle));
+  e = hipIpcGetMemHandle(&handle, r.mem);
+  if (e != hipSuccess) {
+    (void)hipFree(r.mem);
+    unmap_role(r);
+    shm_unlink(shm_name);
+    return fail(BIKV_EHIP, "consumer_init hipIpcGetMemHandle failed: %s", hipGetErrorString(e));
+  }
+  memcpy(r.ctrl->ipc_handle, &handle, sizeof(handle));
+  g_consumer = r;
+  return BIKV_OK;
+}
+
+extern "C" int bikv_producer_init(int device, const char* shm_name) {
+  if (!shm_name || !*shm_name) return fail(BIKV_EINVAL, "shm_name is empty");
+  if (g_producer.ctrl) return fail(BIKV_ESTATE, "producer already initialised (call producer_cleanup first)");
+  // The control block is opened and checked before the GPU is touched, so that a missing object
+  // or a foreign host is reported as such whatever the state of the device.
+  Role r;
+  r.device = device;
+  strncpy(r.shm_name, shm_name, sizeof(r.shm_name) - 1);
+  r.fd = shm_open(shm_name, O_RDWR, 0666);
+  if (r.fd == -1) return fail(BIKV_ESYS, "producer_init shm_open failed: %s", strerror(errno));
+  struct stat sb;
+  if (fstat(r.fd, &sb) == -1 || (size_t)sb.st_size < sizeof(bikv_shared_control)) {
+    close(r.fd);
+    return fail(BIKV_ESYS, "producer_init: shared object is smaller than the control block");
+  }
+  void* m = mmap(nullptr, sizeof(bikv_shared_control), PROT_READ | PROT_WRITE, MAP_SHARED, r.fd, 0);
+  if (m == MAP_FAILED) {
+    const int e = errno;
+    close(r.fd);
+    return fail(BIKV_ESYS, "producer_init mmap failed: %s", strerror(e));
+  }
+  r.ctrl = static_cast<bikv_shared_control*>(m);
+  char host[256];
+  memset(host, 0, sizeof(host));
+  gethostname(host, sizeof(host));
+  if (strncmp(host, r.ctrl->hostname, sizeof(host)) != 0) {
+    unmap_role(r);
+    return fail(BIKV_ESTATE, "Processes must run on the same host");
+  }
+  {
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) {
+      unmap_role(r);
+      return fail_hip(e, "hipSetDevice");
+    }
+  }
+  if (g_consumer.ctrl && strcmp(g_consumer.shm_name, shm_name) == 0) {
+    r.mem = g_consumer.mem;  // same process: no IPC mapping needed (or possible)
+    r.ipc_mapped = false;
+  } else {
+    hipIpcMemHandle_t handle;
+    memcpy(&handle, r.ctrl->ipc_handle, sizeof(handle));
+    hipError_t e = hipIpcOpenMemHandle(&r.mem, handle, hipIpcMemLazyEnablePeerAccess);
+    if (e != hipSuccess) {
+      unmap_role(r);
+      return fail(BIKV_EHIP, "producer_init hipIpcOpenMemHandle failed: %s", hipGetErrorString(e));
+    }
+    r.ipc_mapped = true;
+  }
+  g_producer = r;
+  return BIKV_OK;
+}
+
+extern "C" void bikv_producer_cleanup(void) {
+  if (g_producer.mem && g_producer.ipc_mapped) (void)hipIpcCloseMemHandle(g_producer.mem);
+  g_producer.mem = nullptr;
+  unmap_role(g_producer);
+  g_producer = Role();
+}
+
+extern "C" void bikv_consumer_cleanup(void) {
+  if (g_producer.ctrl && !g_producer.ipc_mapped && g_producer.mem == g_consumer.mem) {
+    // a same-process producer borrows the consumer's buffer: retire it first
+    bikv_producer_cleanup();
+  }
+  if (g_consumer.mem) {
+    (void)hipSetDevice(g_consumer.device);
+    (void)hipFree(g_consumer.mem);
+    g_consumer.mem = nullptr;
+  }
+  if (g_consumer.ctrl) {
+    sem_destroy(sem_of(g_consumer.ctrl->sem_start));
+    sem_destroy(sem_of(g_consumer.ctrl->sem_complete));
+  }
+  const bool had = g_consumer.fd != -1;
+  unmap_role(g_consumer);
+  if (had) shm_unlink(g_consumer.shm_name);
+  g_consumer = Role();
+}
+
+extern "C" int bikv_producer_copy_pages(const void* src, int64_t src_bytes, const int64_t* src_off,
+                                        const int64_t* dst_off, int64_t n_runs, int64_t page_size,
+                                        const bikv_tensor_dims* dims, int64_t elem_bytes,
+                                        int32_t dtype_code, void* stream) {
+  if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
+  if (!dims) return fail(BIKV_EINVAL, "dims is null");
+  if (n_runs < 0 || page_size <= 0 || elem_bytes <= 0) return fail(BIKV_EINVAL, "bad n_runs, page_size or elem_bytes");
+  if (dims->head_size <= 0 || dims->num_kv_heads <= 0 || dims->num_layers <= 0 || dims->kv_pair <= 0)
+    return fail(BIKV_EINVAL, "TensorDims fields must be positive");
+  bikv_shared_control* c = g_producer.ctrl;
+  const int64_t elems_per_token = dims->head_size * dims->num_kv_heads * dims->num_layers * dims->kv_pair;
+  const int64_t run_bytes = page_size * elems_per_token * elem_bytes;
+  const int64_t data_size = n_runs * run_bytes;
+  if ((size_t)data_size > c->buffer_size)
+    return fail(BIKV_ERANGE, "batch of %lld bytes does not fit the %zu-byte ring", (long long)data_size, c->buffer_size);
+  BIKV_HIP(hipSetDevice(g_producer.device));
+  const size_t at = ring_reserve(c, (size_t)data_size);
+  if (n_runs > 0) {
+    int rc = bikv_copy_runs(src, src_bytes, static_cast<char*>(g_producer.mem) + at,
+                            (int64_t)(c->buffer_size - at), src_off, dst_off, n_runs, run_bytes,
+                            elem_bytes, stream);
+    if (rc) return rc;
+    rc = sync_and_check(g_producer.device, static_cast<hipStream_t>(stream));
+    if (rc) return rc;
+  }
+  const int64_t shape[5] = {n_runs * page_size, dims->head_size, dims->num_kv_heads, dims->num_layers, dims->kv_pair};
+  ring_publish(c, (size_t)data_size, shape, 5, dtype_code);
+  return BIKV_OK;
+}
+
+extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64_t* shape,
+                                  size_t ndim, int32_t dtype_code, void* stream) {
+  if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
+  if (ndim > BIKV_MAX_DIM) return fail(BIKV_EINVAL, "at most %d dimensions can be published", BIKV_MAX_DIM);
+  if ((bytes > 0 && !dev_src) || (ndim > 0 && !shape)) return fail(BIKV_EINVAL, "null pointer argument");
+  bikv_shared_control* c = g_producer.ctrl;
+  if (bytes > c->buffer_size)
+    return fail(BIKV_ERANGE, "tensor of %zu bytes does not fit the %zu-byte ring", bytes, c->buffer_size);
+  BIKV_HIP(hipSetDevice(g_producer.device));
+  const size_t at = ring_reserve(c, bytes);
+  if (bytes > 0) {
+    BIKV_HIP(hipMemcpyAsync(static_cast<char*>(g_producer.mem) + at, dev_src, bytes,
+                            hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
+    BIKV_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  }
+  ring_publish(c, bytes, shape, ndim, dtype_code);
+  return BIKV_OK;
+}
+
+extern "C" int bikv_consumer_receive(int64_t timeout_ms, void** ptr, int64_t shape[BIKV_MAX_DIM],
+                                     size_t* ndim, size_t* data_bytes, int32_t* device_id,
+                                     int32_t* dtype_code) {
+  if (!g_consumer.ctrl || !g_consumer.mem) return fail(BIKV_ESTATE, "consumer is not initialised");
+  if (!ptr || !shape || !ndim) return fail(BIKV_EINVAL, "null pointer argument");
+  bikv_shared_control* c = g_consumer.ctrl;
+  sem_t* s = sem_of(c->sem_start);
+  int rc;
+  if (timeout_ms < 0) {
+    do { rc = sem_wait(s); } while (rc == -1 && errno == EINTR);
+  } else {
+    struct timespec ts;
+    clock_gettime(CLOCK_REALTIME, &ts);
+    ts.tv_sec += timeout_ms / 1000;
+    ts.tv_nsec += (timeout_ms % 1000) * 1000000L;
+    if (ts.tv_nsec >= 1000000000L) { ts.tv_sec += 1; ts.tv_nsec -= 1000000000L; }
+    do { rc = sem_timedwait(s, &ts); } while (rc == -1 && errno == EINTR);
+  }
+  if (rc == -1) {
+    if (errno == ETIMEDOUT) return fail(BIKV_ESTATE, "consumer_receive timed out after %lld ms", (long long)timeout_ms);
+    return fail(BIKV_ESYS, "consumer_receive sem_wait failed: %s", strerror(errno));
+  }
+  if (c->tensor_dim > BIKV_MAX_DIM) return fail(BIKV_ESTATE, "control block holds %zu dimensions", c->tensor_dim);
+  *ptr = static_cast<char*>(g_consumer.mem) + c->last_valid_offset;
+  *ndim = c->tensor_dim;
+  for (size_t i = 0; i < c->tensor_dim; ++i) shape[i] = c->tensor_shape[i];
+  if (data_bytes) *data_bytes = c->data_size;
+  if (device_id) *device_id = c->device_id;
+  if (dtype_code) *dtype_code = c->dtype_code;
+  return BIKV_OK;
+}
+
+extern "C" const bikv_shared_control* bikv_producer_control(void) { return g_producer.ctrl; }
+extern "C" const bikv_shared_control* bikv_consumer_control(void) { return g_consumer.ctrl; }
+extern "C" void* bikv_consumer_buffer(void) { return g_consumer.mem; }

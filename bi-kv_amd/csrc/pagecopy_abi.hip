@@ -1,0 +1,581 @@
+// C ABI of libbikv_pagecopy.so: argument validation, per-device context, pool handles, the layered
+// gather/scatter entry points, the run copy and the device->pinned-host staging pipeline.
+// Declarations and the reference call sites each entry point replaces: include/bikv_pagecopy.h.
+#include "../../include/bikv_pagecopy.h"
+#include "pagecopy_internal.h"
+#include "pagecopy_kernels.h"
+
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+namespace bikv {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int fail_hip(hipError_t e, const char* what) {
+  return fail(BIKV_EHIP, "%s failed: %s", what, hipGetErrorString(e));
+}
+
+// ---- per-device context: the host-mapped status block -------------------------------------
+struct DevCtx {
+  uint32_t* status_host = nullptr;  // pinned, mapped
+  uint32_t* status_dev = nullptr;   // the same memory as the device sees it
+};
+static std::mutex g_ctx_mu;
+static DevCtx g_ctx[64];
+
+int device_status(int device, uint32_t** dev_ptr) {
+  if (device < 0 || device >= 64) return fail(BIKV_EINVAL, "device index %d out of range", device);
+  std::lock_guard<std::mutex> lk(g_ctx_mu);
+  DevCtx& c = g_ctx[device];
+  if (!c.status_host) {
+    BIKV_HIP(hipSetDevice(device));
+    void* h = nullptr;
+    BIKV_HIP(hipHostMalloc(&h, ST_SLOTS * sizeof(uint32_t) * 8, hipHostMallocMapped | hipHostMallocPortable));
+    memset(h, 0, ST_SLOTS * sizeof(uint32_t) * 8);
+    void* d = nullptr;
+    hipError_t e = hipHostGetDevicePointer(&d, h, 0);
+    if (e != hipSuccess) {
+      (void)hipHostFree(h);
+      return fail_hip(e, "hipHostGetDevicePointer");
+    }
+    c.status_host = static_cast<uint32_t*>(h);
+    c.status_dev = static_cast<uint32_t*>(d);
+  }
+  *dev_ptr = c.status_dev;
+  return BIKV_OK;
+}
+
+static uint32_t take_status(int device) {
+  std::lock_guard<std::mutex> lk(g_ctx_mu);
+  DevCtx& c = g_ctx[device];
+  if (!c.status_host) return 0;
+  volatile uint32_t* s = c.status_host;
+  uint32_t bits = 0;
+  if (s[ST_SLOT_SRC]) bits |= BIKV_ST_SRC_RANGE;
+  if (s[ST_SLOT_DST]) bits |= BIKV_ST_DST_RANGE;
+  if (s[ST_SLOT_PAGE]) bits |= BIKV_ST_PAGE_ID;
+  s[ST_SLOT_SRC] = 0;
+  s[ST_SLOT_DST] = 0;
+  s[ST_SLOT_PAGE] = 0;
+  return bits;
+}
+
+int sync_and_check(int device, hipStream_t stream) {
+  BIKV_HIP(hipStreamSynchronize(stream));
+  const uint32_t bits = take_status(device);
+  if (bits)
+    return fail(BIKV_EBOUNDS, "kernel skipped out-of-range work (status bits 0x%x:%s%s%s)", bits,
+                (bits & BIKV_ST_SRC_RANGE) ? " source-range" : "",
+                (bits & BIKV_ST_DST_RANGE) ? " destination-range" : "",
+                (bits & BIKV_ST_PAGE_ID) ? " page-id" : "");
+  return BIKV_OK;
+}
+
+static int current_device(int* dev) {
+  BIKV_HIP(hipGetDevice(dev));
+  return BIKV_OK;
+}
+
+static int lowbit_width(uint64_t x) {
+  int w = 16;
+  while (w > 1 && (x & (uint64_t)(w - 1))) w >>= 1;
+  return w;
+}
+
+}  // namespace bikv
+
+using namespace bikv;
+
+// ---- pool handle --------------------------------------------------------------------------
+struct bikv_pool {
+  int device;
+  int n_planes;
+  int64_t n_pages;
+  int64_t tile_bytes, page_stride;
+  int64_t scale_tile_bytes, scale_page_stride;
+  const char** d_plane_base;        // device table: payload planes, then scale planes
+  uint64_t align_bits;              // OR of every base, stride and tile size (payload)
+  uint64_t scale_align_bits;
+};
+
+extern "C" int bikv_abi_version(void) { return BIKV_ABI_VERSION; }
+extern "C" const char* bikv_last_error(void) { return g_err; }
+
+extern "C" int bikv_check_status(int device, void* stream, uint32_t* bits_out) {
+  if (device < 0 || device >= 64) return fail(BIKV_EINVAL, "device index %d out of range", device);
+  BIKV_HIP(hipSetDevice(device));
+  BIKV_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  const uint32_t bits = take_status(device);
+  if (bits_out) *bits_out = bits;
+  if (bits) return fail(BIKV_EBOUNDS, "kernel skipped out-of-range work (status bits 0x%x)", bits);
+  return BIKV_OK;
+}
+
+extern "C" int bikv_set_tuning(const char* key, int64_t value) {
+  if (!key) return fail(BIKV_EINVAL, "null tuning key");
+  Tuning& t = tuning();
+  if (!strcmp(key, "seg")) {
+    if (value < 0 || value > kMaxSeg) return fail(BIKV_EINVAL, "seg must be in [0, %d]", kMaxSeg);
+    t.seg = (int)value;
+  } else if (!strcmp(key, "unroll")) {
+    if (value != 1 && value != 2 && value != 4 && value != 8)
+      return fail(BIKV_EINVAL, "unroll must be 1, 2, 4 or 8");
+    t.unroll = (int)value;
+  } else if (!strcmp(key, "nontemporal")) {
+    t.nontemporal = value ? 1 : 0;
+  } else if (!strcmp(key, "run_chunk_kib")) {
+    if (value < 0 || value > 1 << 20) return fail(BIKV_EINVAL, "run_chunk_kib out of range");
+    t.run_chunk_kib = (int)value;
+  } else {
+    return fail(BIKV_EINVAL, "unknown tuning key '%s'", key);
+  }
+  return BIKV_OK;
+}
+
+extern "C" int bikv_pool_create(const bikv_pool_desc* d, bikv_pool** out) {
+  if (!d || !out) return fail(BIKV_EINVAL, "null argument");
+  *out = nullptr;
+  if (d->n_planes <= 0 || d->n_planes > 65536) return fail(BIKV_EINVAL, "n_planes %d out of range", d->n_planes);
+  if (d->n_pages <= 0) return fail(BIKV_EINVAL, "n_pages must be positive");
+  if (d->tile_bytes <= 0 || d->page_stride_bytes < d->tile_bytes)
+    return fail(BIKV_EINVAL, "need 0 < tile_bytes <= page_stride_bytes (got %lld, %lld)",
+                (long long)d->tile_bytes, (long long)d->page_stride_bytes);
+  if (!d->plane_base) return fail(BIKV_EINVAL, "plane_base is null");
+  const bool has_scale = d->scale_tile_bytes > 0;
+  if (has_scale && (!d->scale_plane_base || d->scale_page_stride_bytes < d->scale_tile_bytes))
+    return fail(BIKV_EINVAL, "scale class needs scale_plane_base and scale_page_stride_bytes >= scale_tile_bytes");
+  if (d->scale_tile_bytes < 0) return fail(BIKV_EINVAL, "negative scale_tile_bytes");
+
+  std::vector<const char*> table((size_t)d->n_planes * 2, nullptr);
+  uint64_t ab = (uint64_t)d->tile_bytes | (uint64_t)d->page_stride_bytes, sab = 0;
+  for (int q = 0; q < d->n_planes; ++q) {
+    if (!d->plane_base[q]) return fail(BIKV_EINVAL, "plane_base[%d] is null", q);
+    table[q] = static_cast<const char*>(d->plane_base[q]);
+    ab |= (uint64_t)d->plane_base[q];
+  }
+  if (has_scale) {
+    sab = (uint64_t)d->scale_tile_bytes | (uint64_t)d->scale_page_stride_bytes;
+    for (int q = 0; q < d->n_planes; ++q) {
+      if (!d->scale_plane_base[q]) return fail(BIKV_EINVAL, "scale_plane_base[%d] is null", q);
+      table[d->n_planes + q] = static_cast<const char*>(d->scale_plane_base[q]);
+      sab |= (uint64_t)d->scale_plane_base[q];
+    }
+  }
+  uint32_t* st = nullptr;
+  int rc = device_status(d->device, &st);
+  if (rc) return rc;
+  BIKV_HIP(hipSetDevice(d->device));
+  void* dtab = nullptr;
+  BIKV_HIP(hipMalloc(&dtab, table.size() * sizeof(char*)));
+  hipError_t e = hipMemcpy(dtab, table.data(), table.size() * sizeof(char*), hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    (void)hipFree(dtab);
+    return fail_hip(e, "hipMemcpy(plane table)");
+  }
+  bikv_pool* p = new bikv_pool();
+  p->device = d->device;
+  p->n_planes = d->n_planes;
+  p->n_pages = d->n_pages;
+  p->tile_bytes = d->tile_bytes;
+  p->page_stride = d->page_stride_bytes;
+  p->scale_tile_bytes = has_scale ? d->scale_tile_bytes : 0;
+  p->scale_page_stride = has_scale ? d->scale_page_stride_bytes : 0;
+  p->d_plane_base = static_cast<const char**>(dtab);
+  p->align_bits = ab;
+  p->scale_align_bits = sab;
+  *out = p;
+  return BIKV_OK;
+}
+
+extern "C" int bikv_pool_destroy(bikv_pool* p) {
+  if (!p) return BIKV_OK;
+  (void)hipSetDevice(p->device);
+  hipError_t e = hipFree((void*)p->d_plane_base);
+  delete p;
+  if (e != hipSuccess) return fail_hip(e, "hipFree(plane table)");
+  return BIKV_OK;
+}
+
+namespace bikv {
+
+// Fills MoveArgs for one launch; `staging`/`scale_staging` are slot 0 of the (possibly windowed)
+// staging image after slot_bias has been applied.
+static int build_move(const bikv_pool* pool, const bikv_page_batch* b, const void* staging,
+                      int64_t staging_bytes, const void* scale_staging, int64_t scale_bytes,
+                      MoveArgs* m) {
+  if (!pool || !b) return fail(BIKV_EINVAL, "null pool or batch");
+  if (b->n_pages < 0) return fail(BIKV_EINVAL, "negative n_pages");
+  int pb = b->plane_begin, pc = b->plane_count;
+  if (pc <= 0) { pb = 0; pc = pool->n_planes; }
+  if (pb < 0 || pb + pc > pool->n_planes)
+    return fail(BIKV_EINVAL, "planes [%d, %d) outside [0, %d)", pb, pb + pc, pool->n_planes);
+  memset(m, 0, sizeof(*m));
+  m->n_batch = b->n_pages;
+  m->plane_begin = pb;
+  m->plane_count = pc;
+  if (b->n_pages == 0) return BIKV_OK;
+  if (!b->page_ids || !b->slots || !b->slot_strides)
+    return fail(BIKV_EINVAL, "page_ids, slots and slot_strides must be non-null");
+  if (!staging || staging_bytes < 0) return fail(BIKV_EINVAL, "staging buffer is null or negative-sized");
+  const bool has_scale = pool->scale_tile_bytes > 0;
+  if (has_scale && (!scale_staging || scale_bytes < 0))
+    return fail(BIKV_EINVAL, "pool has a scale class: scale_staging must be given");
+  uint32_t* st = nullptr;
+  int rc = device_status(pool->device, &st);
+  if (rc) return rc;
+  m->page_ids = b->page_ids;
+  m->slots = b->slots;
+  m->slot_strides = b->slot_strides;
+  m->n_pool_pages = pool->n_pages;
+  m->slot_bias = b->slot_bias;
+  m->status = st;
+  m->payload.plane_base = pool->d_plane_base;
+  m->payload.staging = static_cast<char*>(const_cast<void*>(staging));
+  m->payload.n_slots = staging_bytes / pool->tile_bytes;
+  m->payload.tile_bytes = pool->tile_bytes;
+  m->payload.page_stride = pool->page_stride;
+  m->payload.vec_width = lowbit_width(pool->align_bits | (uint64_t)staging);
+  if (has_scale) {
+    m->scale.plane_base = pool->d_plane_base + pool->n_planes;
+    m->scale.staging = static_cast<char*>(const_cast<void*>(scale_staging));
+    m->scale.n_slots = scale_bytes / pool->scale_tile_bytes;
+    m->scale.tile_bytes = pool->scale_tile_bytes;
+    m->scale.page_stride = pool->scale_page_stride;
+    m->scale.vec_width = lowbit_width(pool->scale_align_bits | (uint64_t)scale_staging);
+  }
+  return BIKV_OK;
+}
+
+static int move_pages(int dir, const bikv_pool* pool, const bikv_page_batch* b, const void* staging,
+                      int64_t staging_bytes, const void* scale_staging, int64_t scale_bytes,
+                      void* stream) {
+  MoveArgs m;
+  int rc = build_move(pool, b, staging, staging_bytes, scale_staging, scale_bytes, &m);
+  if (rc) return rc;
+  if (m.n_batch == 0) return BIKV_OK;
+  BIKV_HIP(hipSetDevice(pool->device));
+  hipError_t e = launch_tile_move(dir, m, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail_hip(e, dir == 0 ? "gather launch" : "scatter launch");
+  return BIKV_OK;
+}
+
+}  // namespace bikv
+
+extern "C" int bikv_gather_pages(const bikv_pool* pool, const bikv_page_batch* batch, void* staging,
+                                 int64_t staging_bytes, void* scale_staging,
+                                 int64_t scale_staging_bytes, void* stream) {
+  return move_pages(0, pool, batch, staging, staging_bytes, scale_staging, scale_staging_bytes, stream);
+}
+
+extern "C" int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* batch,
+                                  const void* staging, int64_t staging_bytes,
+                                  const void* scale_staging, int64_t scale_staging_bytes,
+                                  void* stream) {
+  return move_pages(1, pool, batch, staging, staging_bytes, scale_staging, scale_staging_bytes, stream);
+}
+
+extern "C" int bikv_copy_runs(const void* src, int64_t src_bytes, void* dst, int64_t dst_bytes,
+                              const int64_t* src_off, const int64_t* dst_off, int64_t n_runs,
+                              int64_t run_bytes, int64_t unit_bytes, void* stream) {
+  if (n_runs < 0 || run_bytes < 0) return fail(BIKV_EINVAL, "negative n_runs or run_bytes");
+  if (n_runs == 0 || run_bytes == 0) return BIKV_OK;
+  if (!src || !dst || !src_off || !dst_off) return fail(BIKV_EINVAL, "null pointer argument");
+  if (unit_bytes <= 0) return fail(BIKV_EINVAL, "unit_bytes must be positive");
+  if (n_runs >= (int64_t(1) << 31)) return fail(BIKV_EINVAL, "too many runs");
+  if (run_bytes > src_bytes || run_bytes > dst_bytes)
+    return fail(BIKV_EINVAL, "run_bytes %lld exceeds a buffer (src %lld, dst %lld bytes)",
+                (long long)run_bytes, (long long)src_bytes, (long long)dst_bytes);
+  int dev = 0;
+  int rc = current_device(&dev);
+  if (rc) return rc;
+  RunArgs a;
+  a.src = static_cast<const char*>(src);
+  a.dst = static_cast<char*>(dst);
+  a.src_bytes = src_bytes;
+  a.dst_bytes = dst_bytes;
+  a.src_off = src_off;
+  a.dst_off = dst_off;
+  a.n_runs = n_runs;
+  a.run_bytes = run_bytes;
+  a.unit_bytes = unit_bytes;
+  rc = device_status(dev, &a.status);
+  if (rc) return rc;
+  hipError_t e = launch_copy_runs(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail_hip(e, "copy_runs launch");
+  return BIKV_OK;
+}
+
+// ---- pinned host memory -------------------------------------------------------------------
+extern "C" int bikv_host_alloc(int64_t bytes, void** out) {
+  if (!out || bytes <= 0) return fail(BIKV_EINVAL, "bad host_alloc arguments");
+  BIKV_HIP(hipHostMalloc(out, (size_t)bytes, hipHostMallocMapped | hipHostMallocPortable));
+  return BIKV_OK;
+}
+
+extern "C" int bikv_host_free(void* p) {
+  if (!p) return BIKV_OK;
+  BIKV_HIP(hipHostFree(p));
+  return BIKV_OK;
+}
+
+extern "C" int bikv_d2h_copy(int device, void* host_dst, const void* dev_src, int64_t bytes,
+                             int64_t chunk_bytes, double* seconds_out) {
+  if (!host_dst || !dev_src || bytes <= 0) return fail(BIKV_EINVAL, "bad d2h_copy arguments");
+  BIKV_HIP(hipSetDevice(device));
+  hipStream_t s;
+  BIKV_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  if (chunk_bytes <= 0) chunk_bytes = bytes;
+  const auto t0 = std::chrono::steady_clock::now();
+  hipError_t e = hipSuccess;
+  for (int64_t off = 0; off < bytes && e == hipSuccess; off += chunk_bytes) {
+    const int64_t n = bytes - off < chunk_bytes ? bytes - off : chunk_bytes;
+    e = hipMemcpyAsync(static_cast<char*>(host_dst) + off, static_cast<const char*>(dev_src) + off,
+                       (size_t)n, hipMemcpyDeviceToHost, s);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  const auto t1 = std::chrono::steady_clock::now();
+  (void)hipStreamDestroy(s);
+  if (e != hipSuccess) return fail_hip(e, "hipMemcpyAsync(D2H)");
+  if (seconds_out) *seconds_out = std::chrono::duration<double>(t1 - t0).count();
+  return BIKV_OK;
+}
+
+// ---- device -> pinned-host staging pipeline -----------------------------------------------
+struct bikv_stager {
+  int device;
+  int64_t chunk_bytes;
+  int n_buf;
+  char* ring;
+  hipStream_t s_gather, s_copy;
+  std::vector<hipEvent_t> filled, drained;
+};
+
+extern "C" int bikv_stager_create(int device, int64_t chunk_bytes, int32_t n_buffers,
+                                  bikv_stager** out) {
+  if (!out) return fail(BIKV_EINVAL, "null out");
+  *out = nullptr;
+  if (chunk_bytes < 4096 || n_buffers < 1 || n_buffers > 64)
+    return fail(BIKV_EINVAL, "need chunk_bytes >= 4096 and 1 <= n_buffers <= 64");
+  uint32_t* st_ptr = nullptr;
+  int rc = device_status(device, &st_ptr);
+  if (rc) return rc;
+  BIKV_HIP(hipSetDevice(device));
+  bikv_stager* st = new bikv_stager();
+  st->device = device;
+  st->chunk_bytes = chunk_bytes;
+  st->n_buf = n_buffers;
+  st->ring = nullptr;
+  st->s_gather = nullptr;
+  st->s_copy = nullptr;
+  hipError_t e = hipMalloc((void**)&st->ring, (size_t)chunk_bytes * n_buffers);
+  if (e == hipSuccess) e = hipStreamCreateWithFlags(&st->s_gather, hipStreamNonBlocking);
+  if (e == hipSuccess) e = hipStreamCreateWithFlags(&st->s_copy, hipStreamNonBlocking);
+  for (int i = 0; i < n_buffers && e == hipSuccess; ++i) {
+    hipEvent_t a = nullptr, b = nullptr;
+    e = hipEventCreateWithFlags(&a, hipEventDisableTiming);
+    if (e == hipSuccess) st->filled.push_back(a);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&b, hipEventDisableTiming);
+    if (e == hipSuccess) st->drained.push_back(b);
+  }
+  if (e != hipSuccess) {
+    bikv_stager_destroy(st);
+    return fail_hip(e, "stager setup");
+  }
+  *out = st;
+  return BIKV_OK;
+}
+
+extern "C" int bikv_stager_destroy(bikv_stager* st) {
+  if (!st) return BIKV_OK;
+  (void)hipSetDevice(st->device);
+  for (hipEvent_t ev : st->filled) (void)hipEventDestroy(ev);
+  for (hipEvent_t ev : st->drained) (void)hipEventDestroy(ev);
+  if (st->s_gather) (void)hipStreamDestroy(st->s_gather);
+  if (st->s_copy) (void)hipStreamDestroy(st->s_copy);
+  if (st->ring) (void)hipFree(st->ring);
+  delete st;
+  return BIKV_OK;
+}
+
+namespace bikv {
+
+// One contiguous byte range of the staging image together with the rectangle of
+// (batch pages x planes) that fills it.
+struct Chunk {
+  int64_t first_page, n_pages;  // batch entries
+  int plane_begin, plane_count;
+  int64_t first_slot, n_slots;  // staging slots covered
+};
+
+// Cuts the staging image of a batch into chunks of at most `max_slots` slots. Requests are packed
+// back to back in batch order.
+static void plan_chunks(const int64_t* req_pages, int64_t n_req, int n_planes, int layout,
+                        int64_t max_slots, std::vector<Chunk>* out) {
+  int64_t first_page = 0, base_slot = 0;
+  if (layout == BIKV_LAYOUT_PAGE_MAJOR) {
+    // slot = global_page * n_planes + plane: any run of whole pages is contiguous, across requests
+    int64_t total = 0;
+    for (int64_t r = 0; r < n_req; ++r) total += req_pages[r];
+    int64_t per = max_slots / n_planes;
+    if (per < 1) per = 1;
+    for (int64_t p = 0; p < total; p += per) {
+      const int64_t n = total - p < per ? total - p : per;
+      out->push_back(Chunk{p, n, 0, n_planes, p * n_planes, n * n_planes});
+    }
+    return;
+  }
+  for (int64_t r = 0; r < n_req; ++r) {
+    const int64_t m = req_pages[r];
+    if (m > 0) {
+      if (m <= max_slots) {
+        int k = (int)(max_slots / m);  // whole plane rows per chunk
+        if (k > n_planes) k = n_planes;
+        for (int q = 0; q < n_planes; q += k) {
+          const int c = n_planes - q < k ? n_planes - q : k;
+          out->push_back(Chunk{first_page, m, q, c, base_slot + (int64_t)q * m, (int64_t)c * m});
+        }
+      } else {
+        for (int q = 0; q < n_planes; ++q)
+          for (int64_t j = 0; j < m; j += max_slots) {
+            const int64_t n = m - j < max_slots ? m - j : max_slots;
+            out->push_back(Chunk{first_page + j, n, q, 1, base_slot + (int64_t)q * m + j, n});
+          }
+      }
+    }
+    first_page += m;
+    base_slot += m * n_planes;
+  }
+}
+
+}  // namespace bikv
+
+extern "C" int64_t bikv_plan_chunks(const int64_t* req_pages, int64_t n_requests, int32_t n_planes,
+                                    int32_t layout, int64_t max_slots, int64_t* out, int64_t cap) {
+  if (!req_pages || n_requests < 0 || n_planes <= 0 || max_slots < 1 || (cap > 0 && !out))
+    return fail(BIKV_EINVAL, "bad plan_chunks arguments");
+  if (layout != BIKV_LAYOUT_LAYER_MAJOR && layout != BIKV_LAYOUT_PAGE_MAJOR)
+    return fail(BIKV_EINVAL, "unknown layout %d", layout);
+  for (int64_t r = 0; r < n_requests; ++r)
+    if (req_pages[r] < 0) return fail(BIKV_EINVAL, "negative req_pages[%lld]", (long long)r);
+  std::vector<Chunk> chunks;
+  plan_chunks(req_pages, n_requests, n_planes, layout, max_slots, &chunks);
+  for (size_t c = 0; c < chunks.size() && (int64_t)c < cap; ++c) {
+    int64_t* o = out + 6 * c;
+    o[0] = chunks[c].first_page; o[1] = chunks[c].n_pages;
+    o[2] = chunks[c].plane_begin; o[3] = chunks[c].plane_count;
+    o[4] = chunks[c].first_slot; o[5] = chunks[c].n_slots;
+  }
+  return (int64_t)chunks.size();
+}
+
+extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
+                                   const bikv_page_batch* batch, const int64_t* req_pages,
+                                   int64_t n_requests, int32_t layout, void* host_dst,
+                                   int64_t host_bytes, int32_t mode, bikv_stage_stats* stats) {
+  if (!st || !pool || !batch || !req_pages || !host_dst)
+    return fail(BIKV_EINVAL, "null argument");
+  if (pool->scale_tile_bytes > 0)
+    return fail(BIKV_EINVAL, "the host staging pipeline moves payload-only pools");
+  if (pool->device != st->device) return fail(BIKV_EINVAL, "pool and stager are on different devices");
+  if (layout != BIKV_LAYOUT_LAYER_MAJOR && layout != BIKV_LAYOUT_PAGE_MAJOR)
+    return fail(BIKV_EINVAL, "unknown layout %d", layout);
+  if (batch->plane_count > 0 && (batch->plane_begin != 0 || batch->plane_count != pool->n_planes))
+    return fail(BIKV_EINVAL, "the host staging pipeline moves all planes");
+  if (batch->slot_bias != 0) return fail(BIKV_EINVAL, "slot_bias must be 0");
+  int64_t total_pages = 0;
+  for (int64_t r = 0; r < n_requests; ++r) {
+    if (req_pages[r] < 0) return fail(BIKV_EINVAL, "negative req_pages[%lld]", (long long)r);
+    total_pages += req_pages[r];
+  }
+  if (total_pages != batch->n_pages)
+    return fail(BIKV_EINVAL, "req_pages sums to %lld but the batch has %lld pages",
+                (long long)total_pages, (long long)batch->n_pages);
+  const int64_t T = pool->tile_bytes;
+  const int64_t image_bytes = total_pages * pool->n_planes * T;
+  if (host_bytes < image_bytes)
+    return fail(BIKV_ERANGE, "host buffer holds %lld bytes, staging image needs %lld",
+                (long long)host_bytes, (long long)image_bytes);
+  if (stats) { stats->bytes = 0; stats->n_chunks = 0; stats->wall_seconds = 0.0; }
+  if (total_pages == 0) return BIKV_OK;
+  BIKV_HIP(hipSetDevice(st->device));
+  const auto t0 = std::chrono::steady_clock::now();
+
+  if (mode == BIKV_STAGE_DIRECT) {
+    void* dptr = nullptr;
+    BIKV_HIP(hipHostGetDevicePointer(&dptr, host_dst, 0));
+    int rc = bikv_gather_pages(pool, batch, dptr, image_bytes, nullptr, 0, st->s_gather);
+    if (rc) return rc;
+    rc = sync_and_check(st->device, st->s_gather);
+    if (rc) return rc;
+    if (stats) stats->n_chunks = 1;
+  } else if (mode == BIKV_STAGE_PIPELINED) {
+    const int64_t max_slots = st->chunk_bytes / T;
+    if (max_slots < 1)
+      return fail(BIKV_ERANGE, "chunk_bytes %lld is smaller than one tile (%lld bytes)",
+                  (long long)st->chunk_bytes, (long long)T);
+    std::vector<Chunk> chunks;
+    plan_chunks(req_pages, n_requests, pool->n_planes, layout, max_slots, &chunks);
+    hipError_t e = hipSuccess;
+    int rc = BIKV_OK;
+    for (size_t c = 0; c < chunks.size(); ++c) {
+      const Chunk& ch = chunks[c];
+      const int buf = (int)(c % (size_t)st->n_buf);
+      char* dev_chunk = st->ring + (int64_t)buf * st->chunk_bytes;
+      if (c >= (size_t)st->n_buf) {
+        e = hipStreamWaitEvent(st->s_gather, st->drained[buf], 0);
+        if (e != hipSuccess) break;
+      }
+      bikv_page_batch sub = *batch;
+      sub.page_ids = batch->page_ids + ch.first_page;
+      sub.slots = batch->slots + ch.first_page;
+      sub.slot_strides = batch->slot_strides + ch.first_page;
+      sub.n_pages = ch.n_pages;
+      sub.plane_begin = ch.plane_begin;
+      sub.plane_count = ch.plane_count;
+      sub.slot_bias = ch.first_slot;
+      rc = bikv_gather_pages(pool, &sub, dev_chunk, ch.n_slots * T, nullptr, 0, st->s_gather);
+      if (rc) break;
+      e = hipEventRecord(st->filled[buf], st->s_gather);
+      if (e != hipSuccess) break;
+      e = hipStreamWaitEvent(st->s_copy, st->filled[buf], 0);
+      if (e != hipSuccess) break;
+      e = hipMemcpyAsync(static_cast<char*>(host_dst) + ch.first_slot * T, dev_chunk,
+                         (size_t)(ch.n_slots * T), hipMemcpyDeviceToHost, st->s_copy);
+      if (e != hipSuccess) break;
+      e = hipEventRecord(st->drained[buf], st->s_copy);
+      if (e != hipSuccess) break;
+    }
+    // Drain both streams whatever happened, so that no work is left in flight on an error path.
+    const hipError_t e1 = hipStreamSynchronize(st->s_gather);
+    const hipError_t e2 = hipStreamSynchronize(st->s_copy);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail_hip(e, "staging pipeline");
+    if (e1 != hipSuccess) return fail_hip(e1, "hipStreamSynchronize(gather)");
+    if (e2 != hipSuccess) return fail_hip(e2, "hipStreamSynchronize(copy)");
+    rc = sync_and_check(st->device, st->s_gather);
+    if (rc) return rc;
+    if (stats) stats->n_chunks = (int64_t)chunks.size();
+  } else {
+    return fail(BIKV_EINVAL, "unknown staging mode %d", mode);
+  }
+  const auto t1 = std::chrono::steady_clock::now();
+  if (stats) {
+    stats->bytes = image_bytes;
+    stats->wall_seconds = std::chrono::duration<double>(t1 - t0).count();
+  }
+  return BIKV_OK;
+}

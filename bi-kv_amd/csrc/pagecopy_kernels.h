@@ -1,0 +1,70 @@
+// Internal launch interface between the C ABI (pagecopy_abi.hip, ipc_ring.hip) and the gfx950
+// kernels (pagecopy_kernels.hip). Not installed; the public surface is include/bikv_pagecopy.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bikv {
+
+// Status slots written by kernels (one 32-bit word per condition, plain stores of 1, so no
+// atomics are needed on the host-mapped status block).
+enum : int { ST_SLOT_SRC = 0, ST_SLOT_DST = 1, ST_SLOT_PAGE = 2, ST_SLOTS = 8 };
+
+// One tile class of a layered pool as the kernels see it.
+struct TileClass {
+  const char* const* plane_base;  // device-resident table, n_planes entries
+  char* staging;                  // slot 0 of the staging window
+  int64_t n_slots;                // slots available in the staging window
+  int64_t tile_bytes;
+  int64_t page_stride;
+  int32_t vec_width;              // widest power of two (<=16) dividing every address and size
+  int32_t log2_rows;              // fast mover only: tile_bytes == 4096 << log2_rows
+  int32_t seg;                    // batch pages per workgroup
+  uint32_t segs_per_plane;        // ceil(n_batch / seg)
+  uint32_t n_blocks;              // plane_count * segs_per_plane
+};
+
+struct MoveArgs {
+  TileClass payload;
+  TileClass scale;                // n_blocks == 0 when the pool has no scale class
+  const int64_t* page_ids;
+  const int64_t* slots;
+  const int64_t* slot_strides;
+  int64_t n_batch;
+  int64_t n_pool_pages;
+  int64_t slot_bias;
+  int32_t plane_begin;
+  int32_t plane_count;
+  uint32_t* status;
+};
+
+struct Tuning {
+  int seg = 0;          // 0 = choose from the batch shape
+  int unroll = 4;       // 16-byte vectors in flight per lane (1, 2, 4 or 8)
+  int nontemporal = 1;  // 1 = nt hint on the streaming loads and stores
+  int run_chunk_kib = 0;  // bytes of a run handled by one workgroup, KiB; 0 = choose
+};
+Tuning& tuning();
+
+constexpr int kBlock = 256;      // 4 wavefronts
+constexpr int kMaxSeg = 256;     // LDS descriptor slots per workgroup
+constexpr int kRowBytes = kBlock * 16;  // one 16-byte vector per lane
+
+// dir: 0 = gather (pool -> staging), 1 = scatter (staging -> pool).
+hipError_t launch_tile_move(int dir, MoveArgs& a, hipStream_t stream);
+
+struct RunArgs {
+  const char* src;
+  char* dst;
+  int64_t src_bytes;
+  int64_t dst_bytes;
+  const int64_t* src_off;
+  const int64_t* dst_off;
+  int64_t n_runs;
+  int64_t run_bytes;
+  int64_t unit_bytes;
+  uint32_t* status;
+};
+hipError_t launch_copy_runs(const RunArgs& a, hipStream_t stream);
+
+}  // namespace bikv

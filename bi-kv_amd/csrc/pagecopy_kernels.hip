@@ -1,0 +1,418 @@
+// gfx950 kernels of the KV page-copy path. Pure data movement: every lane moves 16-byte vectors
+// (global_load_dwordx4 / global_store_dwordx4), a wavefront moves 1 KiB per instruction, and a
+// 256-lane workgroup moves one 4 KiB "row" per vector slot. No arithmetic on the payload, so the
+// kernels are dtype-agnostic and bit-exact by construction (NaN payloads and fp8 bit patterns are
+// never routed through a floating-point type).
+//
+// Semantics follow the reference's two kernels, block_per_page_copy_kernel and
+// zero_copy_page_kernel (Bi-KV/SharedMemory/CUDA_Shared/copy_kernel.cu:9-36, 39-66):
+//   dst[dst_off[i] + e] = src[src_off[i] + e]   for every run i and every byte e of the run.
+// The reference moves one 2-byte scalar per thread per iteration with one 1024-thread block per
+// page; here the unit of scheduling is a 16 KiB..256 KiB span so that a batch of a few hundred
+// large pages still fills 256 CUs, and page descriptors are resolved once per workgroup into LDS
+// and broadcast from there.
+#include "pagecopy_kernels.h"
+
+namespace bikv {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <int VW> struct VecOf;
+template <> struct VecOf<16> { using T = u32x4; };
+template <> struct VecOf<8> { using T = u32x2; };
+template <> struct VecOf<4> { using T = uint32_t; };
+template <> struct VecOf<2> { using T = uint16_t; };
+template <> struct VecOf<1> { using T = uint8_t; };
+
+// Every payload access goes through an explicit global-address-space pointer: addresses here are
+// assembled from integers, and without the address space the compiler would have to emit flat_*
+// instructions (which also probe the LDS and scratch apertures) instead of global_*.
+#define BIKV_GLOBAL __attribute__((address_space(1)))
+
+template <bool NT, class T>
+__device__ __forceinline__ T ld(uint64_t addr) {
+  const BIKV_GLOBAL T* p = (const BIKV_GLOBAL T*)addr;
+  if constexpr (NT) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+template <bool NT, class T>
+__device__ __forceinline__ void st(uint64_t addr, T v) {
+  BIKV_GLOBAL T* p = (BIKV_GLOBAL T*)addr;
+  if constexpr (NT) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
+
+// A value that is the same in every lane, moved to scalar registers so that the address of a
+// vector access becomes (scalar base + per-lane offset).
+__device__ __forceinline__ uint64_t uniform64(uint64_t x) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
+__device__ __forceinline__ void raise(uint32_t* status, int slot) {
+  *reinterpret_cast<volatile uint32_t*>(status + slot) = 1u;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Layered tile move
+// ---------------------------------------------------------------------------------------------
+
+// Resolves the (pool address, staging address) pair of every page of this workgroup's segment
+// into LDS. A tile that fails a bounds check gets a null pair and is skipped by the movers.
+template <int DIR>
+__device__ __forceinline__ int stage_descriptors(const TileClass& c, const MoveArgs& a,
+                                                 uint32_t blk, uint64_t* s_pool,
+                                                 uint64_t* s_stage, bool* any_bad) {
+  const uint32_t q_rel = blk / c.segs_per_plane;
+  const uint32_t sidx = blk - q_rel * c.segs_per_plane;
+  const int64_t q = a.plane_begin + (int64_t)q_rel;
+  const int64_t i0 = (int64_t)sidx * c.seg;
+  const int64_t rem = a.n_batch - i0;
+  const int nseg = rem < (int64_t)c.seg ? (int)rem : c.seg;
+  const int tid = threadIdx.x;
+  bool bad = false;
+  if (tid < nseg) {
+    const int64_t pid = a.page_ids[i0 + tid];
+    const int64_t slot = a.slots[i0 + tid] + q * a.slot_strides[i0 + tid] - a.slot_bias;
+    const bool bad_page = (uint64_t)pid >= (uint64_t)a.n_pool_pages;
+    const bool bad_slot = (uint64_t)slot >= (uint64_t)c.n_slots;
+    uint64_t pp = 0, sp = 0;
+    if (bad_page) raise(a.status, ST_SLOT_PAGE);
+    if (bad_slot) raise(a.status, DIR == 0 ? ST_SLOT_DST : ST_SLOT_SRC);
+    if (!bad_page && !bad_slot) {
+      pp = (uint64_t)(c.plane_base[q] + pid * c.page_stride);
+      sp = (uint64_t)(c.staging + slot * c.tile_bytes);
+    }
+    s_pool[tid] = pp;
+    s_stage[tid] = sp;
+    bad = bad_page || bad_slot;
+  }
+  // also the barrier that publishes the descriptors
+  *any_bad = __syncthreads_or(bad ? 1 : 0) != 0;
+  return nseg;
+}
+
+// Fast mover: tiles are a power-of-two number of 4 KiB rows, everything is 16-byte aligned and
+// every tile of the segment passed its bounds checks. The segment's tiles are walked as one flat
+// sequence of rows, UNROLL rows at a time: UNROLL independent 16-byte loads per lane are issued
+// back to back, then the UNROLL stores. An 8 KiB tile with UNROLL 4 therefore keeps two tiles in
+// flight and a 64 KiB tile takes four passes. The loop body is branch-free so that the loads of one
+// pass are never serialised behind each other.
+template <int DIR, int UNROLL, bool NT>
+__device__ __forceinline__ void move_rows(const TileClass& c, int nseg, const uint64_t* s_pool,
+                                          const uint64_t* s_stage) {
+  const int lr = c.log2_rows;
+  const int mask = (1 << lr) - 1;
+  const int total = nseg << lr;
+  const int full = total & ~(UNROLL - 1);
+  const uint32_t lane_off = threadIdx.x * 16u;
+  for (int base = 0; base < full; base += UNROLL) {
+    u32x4 v[UNROLL];
+    uint64_t d[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int r = base + u;
+      const int tt = r >> lr;
+      const uint64_t row_off = (uint64_t)(r & mask) << 12;
+      const uint64_t pool = uniform64(s_pool[tt]) + row_off;
+      const uint64_t stg = uniform64(s_stage[tt]) + row_off;
+      d[u] = DIR == 0 ? stg : pool;
+      v[u] = ld<NT, u32x4>((DIR == 0 ? pool : stg) + lane_off);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) st<NT, u32x4>(d[u] + lane_off, v[u]);
+  }
+  for (int r = full; r < total; ++r) {
+    const int tt = r >> lr;
+    const uint64_t row_off = (uint64_t)(r & mask) << 12;
+    const uint64_t pool = uniform64(s_pool[tt]) + row_off;
+    const uint64_t stg = uniform64(s_stage[tt]) + row_off;
+    st<NT, u32x4>((DIR == 0 ? stg : pool) + lane_off,
+                  ld<NT, u32x4>((DIR == 0 ? pool : stg) + lane_off));
+  }
+}
+
+// General mover: any tile size and alignment, VW-byte accesses (VW = the widest power of two that
+// divides every base address, stride and the tile size). Used for the 32-byte scale tiles, for
+// tiles that are not a whole number of 4 KiB rows, and for misaligned pools.
+template <int DIR, int VW>
+__device__ __forceinline__ void move_generic_vw(const TileClass& c, int nseg,
+                                                const uint64_t* s_pool, const uint64_t* s_stage) {
+  using T = typename VecOf<VW>::T;
+  const uint32_t vpt = (uint32_t)(c.tile_bytes / VW);
+  const uint32_t total = (uint32_t)nseg * vpt;  // the launcher keeps seg*vpt below 2^31
+  for (uint32_t v = threadIdx.x; v < total; v += kBlock) {
+    const uint32_t tt = v / vpt;
+    const uint32_t ww = v - tt * vpt;
+    const uint64_t pool = s_pool[tt];
+    if (pool == 0) continue;
+    const uint64_t stg = s_stage[tt];
+    const uint64_t off = (uint64_t)ww * VW;
+    st<false, T>((DIR == 0 ? stg : pool) + off, ld<false, T>((DIR == 0 ? pool : stg) + off));
+  }
+}
+
+template <int DIR>
+__device__ __forceinline__ void move_generic(const TileClass& c, int nseg, const uint64_t* s_pool,
+                                             const uint64_t* s_stage) {
+  switch (c.vec_width) {
+    case 16: move_generic_vw<DIR, 16>(c, nseg, s_pool, s_stage); break;
+    case 8: move_generic_vw<DIR, 8>(c, nseg, s_pool, s_stage); break;
+    case 4: move_generic_vw<DIR, 4>(c, nseg, s_pool, s_stage); break;
+    case 2: move_generic_vw<DIR, 2>(c, nseg, s_pool, s_stage); break;
+    default: move_generic_vw<DIR, 1>(c, nseg, s_pool, s_stage); break;
+  }
+}
+
+// One launch moves both tile classes: workgroups [0, payload.n_blocks) take the payload,
+// the rest take the scale tiles, so payload and scales of a page always travel together.
+// Workgroup b of a class handles plane b / segs_per_plane and batch pages
+// [(b % segs_per_plane)*seg, +seg): consecutive workgroups write consecutive staging ranges of one
+// plane and read one plane's region of the pool.
+template <int DIR, int UNROLL, bool NT, bool ROWS>
+__global__ __launch_bounds__(kBlock) void tile_move_kernel(const MoveArgs a) {
+  __shared__ uint64_t s_pool[kMaxSeg];
+  __shared__ uint64_t s_stage[kMaxSeg];
+  uint32_t blk = blockIdx.x;
+  bool any_bad;
+  if (blk < a.payload.n_blocks) {
+    const int nseg = stage_descriptors<DIR>(a.payload, a, blk, s_pool, s_stage, &any_bad);
+    if constexpr (ROWS) {
+      // a segment holding a rejected tile takes the general mover, which skips null descriptors
+      if (!any_bad) move_rows<DIR, UNROLL, NT>(a.payload, nseg, s_pool, s_stage);
+      else move_generic<DIR>(a.payload, nseg, s_pool, s_stage);
+    } else {
+      move_generic<DIR>(a.payload, nseg, s_pool, s_stage);
+    }
+  } else {
+    blk -= a.payload.n_blocks;
+    const int nseg = stage_descriptors<DIR>(a.scale, a, blk, s_pool, s_stage, &any_bad);
+    move_generic<DIR>(a.scale, nseg, s_pool, s_stage);
+  }
+}
+
+template <int DIR, int UNROLL, bool NT>
+static hipError_t launch_rows(const MoveArgs& a, uint32_t grid, hipStream_t s) {
+  hipLaunchKernelGGL((tile_move_kernel<DIR, UNROLL, NT, true>), dim3(grid), dim3(kBlock), 0, s, a);
+  return hipGetLastError();
+}
+
+template <int DIR>
+static hipError_t launch_dir(const MoveArgs& a, bool rows, uint32_t grid, hipStream_t s) {
+  if (!rows) {
+    hipLaunchKernelGGL((tile_move_kernel<DIR, 1, false, false>), dim3(grid), dim3(kBlock), 0, s, a);
+    return hipGetLastError();
+  }
+  const bool nt = tuning().nontemporal != 0;
+  switch (tuning().unroll) {
+    case 1: return nt ? launch_rows<DIR, 1, true>(a, grid, s) : launch_rows<DIR, 1, false>(a, grid, s);
+    case 2: return nt ? launch_rows<DIR, 2, true>(a, grid, s) : launch_rows<DIR, 2, false>(a, grid, s);
+    case 8: return nt ? launch_rows<DIR, 8, true>(a, grid, s) : launch_rows<DIR, 8, false>(a, grid, s);
+    default: return nt ? launch_rows<DIR, 4, true>(a, grid, s) : launch_rows<DIR, 4, false>(a, grid, s);
+  }
+}
+
+// Picks the number of batch pages per workgroup: enough bytes per workgroup to amortise the
+// descriptor staging, but never so few workgroups that 256 CUs are left idle.
+static int choose_seg(int forced, int64_t n_batch, int plane_count, int64_t tile_bytes,
+                      int64_t units_per_tile) {
+  int seg;
+  if (forced > 0) {
+    seg = forced;
+  } else {
+    // aim at ~256 KiB per workgroup
+    int64_t want = (256 * 1024) / (tile_bytes > 0 ? tile_bytes : 1);
+    if (want < 1) want = 1;
+    seg = 1;
+    while (seg * 2 <= want && seg * 2 <= kMaxSeg) seg *= 2;
+    // keep at least ~8 workgroups per CU in the grid when the batch allows it
+    const int64_t min_blocks = 8 * 256;
+    while (seg > 1 && ((n_batch + seg - 1) / seg) * plane_count < min_blocks) seg /= 2;
+  }
+  if (seg > kMaxSeg) seg = kMaxSeg;
+  if (seg < 1) seg = 1;
+  while (seg > 1 && (int64_t)seg * units_per_tile >= (int64_t(1) << 31)) seg /= 2;
+  return seg;
+}
+
+static bool finish_class(TileClass& c, int forced_seg, int64_t n_batch, int plane_count) {
+  if (c.tile_bytes <= 0) { c.n_blocks = 0; c.seg = 1; c.segs_per_plane = 0; return true; }
+  const int64_t units = c.tile_bytes / c.vec_width;
+  if (units >= (int64_t(1) << 31)) return false;
+  c.seg = choose_seg(forced_seg, n_batch, plane_count, c.tile_bytes, units);
+  const int64_t spp = (n_batch + c.seg - 1) / c.seg;
+  const int64_t nb = spp * plane_count;
+  if (nb >= (int64_t(1) << 31)) return false;
+  c.segs_per_plane = (uint32_t)spp;
+  c.n_blocks = (uint32_t)nb;
+  return true;
+}
+
+hipError_t launch_tile_move(int dir, MoveArgs& a, hipStream_t stream) {
+  if (a.n_batch <= 0 || a.plane_count <= 0) return hipSuccess;
+  if (!finish_class(a.payload, tuning().seg, a.n_batch, a.plane_count)) return hipErrorInvalidValue;
+  // scale tiles are tiny: pack as many pages per workgroup as LDS descriptors allow
+  if (a.scale.tile_bytes > 0) {
+    if (!finish_class(a.scale, kMaxSeg, a.n_batch, a.plane_count)) return hipErrorInvalidValue;
+  } else {
+    a.scale.n_blocks = 0;
+  }
+  const uint64_t grid = (uint64_t)a.payload.n_blocks + a.scale.n_blocks;
+  if (grid == 0) return hipSuccess;
+  if (grid >= (uint64_t(1) << 31) / kBlock * 2) return hipErrorInvalidValue;  // grid*block < 2^32
+  // fast mover: 16-byte aligned tiles of 2^k rows of 4 KiB
+  const int64_t nrows = a.payload.tile_bytes / kRowBytes;
+  const bool rows = a.payload.vec_width == 16 && (a.payload.tile_bytes % kRowBytes) == 0 &&
+                    (nrows & (nrows - 1)) == 0;
+  a.payload.log2_rows = 0;
+  if (rows)
+    while ((int64_t(1) << a.payload.log2_rows) < nrows) ++a.payload.log2_rows;
+  return dir == 0 ? launch_dir<0>(a, rows, (uint32_t)grid, stream)
+                  : launch_dir<1>(a, rows, (uint32_t)grid, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Run copy (reference API)
+// ---------------------------------------------------------------------------------------------
+
+template <int VW>
+__device__ __forceinline__ void copy_span_vw(uint64_t s, uint64_t d, int64_t bytes) {
+  using T = typename VecOf<VW>::T;
+  const int64_t n = bytes / VW;
+  for (int64_t i = threadIdx.x; i < n; i += kBlock)
+    st<false, T>(d + (uint64_t)i * VW, ld<false, T>(s + (uint64_t)i * VW));
+  const int64_t done = n * VW;
+  for (int64_t i = done + threadIdx.x; i < bytes; i += kBlock)
+    st<false, uint8_t>(d + (uint64_t)i, ld<false, uint8_t>(s + (uint64_t)i));
+}
+
+// Large runs: workgroup b handles chunk (b % chunks_per_run) of run (b / chunks_per_run). The
+// run's two offsets are fetched once by lane 0, parked in LDS and broadcast.
+template <int UNROLL, bool NT>
+__global__ __launch_bounds__(kBlock) void copy_runs_kernel(const RunArgs a, int64_t chunk_bytes,
+                                                           uint32_t chunks_per_run) {
+  __shared__ int64_t s_off[2];
+  const uint32_t run = blockIdx.x / chunks_per_run;
+  const uint32_t ch = blockIdx.x - run * chunks_per_run;
+  if (threadIdx.x == 0) {
+    s_off[0] = a.src_off[run];
+    s_off[1] = a.dst_off[run];
+  }
+  __syncthreads();
+  const int64_t so_u = (int64_t)uniform64((uint64_t)s_off[0]);
+  const int64_t do_u = (int64_t)uniform64((uint64_t)s_off[1]);
+  const int64_t so = so_u * a.unit_bytes;
+  const int64_t dof = do_u * a.unit_bytes;
+  const bool bad_src = so_u < 0 || so < 0 || so > a.src_bytes - a.run_bytes;
+  const bool bad_dst = do_u < 0 || dof < 0 || dof > a.dst_bytes - a.run_bytes;
+  if (bad_src || bad_dst) {
+    if (threadIdx.x == 0) {
+      if (bad_src) raise(a.status, ST_SLOT_SRC);
+      if (bad_dst) raise(a.status, ST_SLOT_DST);
+    }
+    return;
+  }
+  const int64_t lo = (int64_t)ch * chunk_bytes;
+  const int64_t hi = lo + chunk_bytes < a.run_bytes ? lo + chunk_bytes : a.run_bytes;
+  const uint64_t s = (uint64_t)(a.src + so + lo);
+  const uint64_t d = (uint64_t)(a.dst + dof + lo);
+  const int64_t bytes = hi - lo;
+  const uint64_t al = s | d;
+  if ((al & 15) == 0) {
+    const int64_t nvec = bytes >> 4;
+    for (int64_t base = 0; base < nvec; base += (int64_t)kBlock * UNROLL) {
+      u32x4 v[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int64_t i = base + u * kBlock + threadIdx.x;
+        if (i < nvec) v[u] = ld<NT, u32x4>(s + ((uint64_t)i << 4));
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int64_t i = base + u * kBlock + threadIdx.x;
+        if (i < nvec) st<NT, u32x4>(d + ((uint64_t)i << 4), v[u]);
+      }
+    }
+    const int64_t done = nvec << 4;
+    for (int64_t i = done + threadIdx.x; i < bytes; i += kBlock)
+      st<false, uint8_t>(d + (uint64_t)i, ld<false, uint8_t>(s + (uint64_t)i));
+  } else if ((al & 7) == 0) {
+    copy_span_vw<8>(s, d, bytes);
+  } else if ((al & 3) == 0) {
+    copy_span_vw<4>(s, d, bytes);
+  } else if ((al & 1) == 0) {
+    copy_span_vw<2>(s, d, bytes);
+  } else {
+    copy_span_vw<1>(s, d, bytes);
+  }
+}
+
+// Small runs (<= 2 KiB): one lane per 16-byte piece, many runs per workgroup.
+__global__ __launch_bounds__(kBlock) void copy_small_runs_kernel(const RunArgs a,
+                                                                 uint32_t pieces_per_run,
+                                                                 int64_t total_pieces) {
+  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (p >= total_pieces) return;
+  const int64_t run = p / pieces_per_run;
+  const int64_t piece = p - run * pieces_per_run;
+  const int64_t so_u = a.src_off[run];
+  const int64_t do_u = a.dst_off[run];
+  const int64_t so = so_u * a.unit_bytes;
+  const int64_t dof = do_u * a.unit_bytes;
+  const bool bad_src = so_u < 0 || so < 0 || so > a.src_bytes - a.run_bytes;
+  const bool bad_dst = do_u < 0 || dof < 0 || dof > a.dst_bytes - a.run_bytes;
+  if (bad_src) raise(a.status, ST_SLOT_SRC);
+  if (bad_dst) raise(a.status, ST_SLOT_DST);
+  if (bad_src || bad_dst) return;
+  const int64_t lo = piece << 4;
+  const int64_t n = a.run_bytes - lo < 16 ? a.run_bytes - lo : 16;
+  const uint64_t s = (uint64_t)(a.src + so + lo);
+  const uint64_t d = (uint64_t)(a.dst + dof + lo);
+  if (n == 16 && (((s | d) & 15) == 0)) {
+    st<false, u32x4>(d, ld<false, u32x4>(s));
+  } else {
+    for (int64_t i = 0; i < n; ++i)
+      st<false, uint8_t>(d + (uint64_t)i, ld<false, uint8_t>(s + (uint64_t)i));
+  }
+}
+
+hipError_t launch_copy_runs(const RunArgs& a, hipStream_t stream) {
+  if (a.n_runs <= 0 || a.run_bytes <= 0) return hipSuccess;
+  if (a.run_bytes <= 2048) {
+    const int64_t ppr = (a.run_bytes + 15) >> 4;
+    const int64_t total = ppr * a.n_runs;
+    const int64_t grid = (total + kBlock - 1) / kBlock;
+    if (grid >= (int64_t(1) << 24)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(copy_small_runs_kernel, dim3((uint32_t)grid), dim3(kBlock), 0, stream, a,
+                       (uint32_t)ppr, total);
+    return hipGetLastError();
+  }
+  int64_t chunk = (int64_t)tuning().run_chunk_kib * 1024;
+  if (chunk <= 0) {
+    // ~4096 workgroups when the batch is big enough, 16 KiB..256 KiB each
+    const int64_t total = a.run_bytes * a.n_runs;
+    chunk = 16 * 1024;
+    while (chunk < 256 * 1024 && total / (chunk * 2) >= 4096) chunk *= 2;
+  }
+  chunk = (chunk + 4095) & ~int64_t(4095);
+  const int64_t cpr = (a.run_bytes + chunk - 1) / chunk;
+  const int64_t grid = cpr * a.n_runs;
+  if (cpr >= (int64_t(1) << 31) || grid >= (int64_t(1) << 24)) return hipErrorInvalidValue;
+  const bool nt = tuning().nontemporal != 0;
+  if (nt)
+    hipLaunchKernelGGL((copy_runs_kernel<4, true>), dim3((uint32_t)grid), dim3(kBlock), 0, stream,
+                       a, chunk, (uint32_t)cpr);
+  else
+    hipLaunchKernelGGL((copy_runs_kernel<4, false>), dim3((uint32_t)grid), dim3(kBlock), 0, stream,
+                       a, chunk, (uint32_t)cpr);
+  return hipGetLastError();
+}
+
+Tuning& tuning() {
+  static Tuning t;
+  return t;
+}
+
+}  // namespace bikv

@@ -1,0 +1,289 @@
+/*
+ * bikv_pagecopy.h — C ABI of libbikv_pagecopy.so, the MI355X (gfx950) KV page-copy library.
+ *
+ * The library replaces the device side of Bi-KV's `ipc_service` extension
+ * (Bi-KV/SharedMemory/CUDA_Shared/{copy_kernel.cu, ipc_service.cpp, ipc_wrapper.h}) and adds the
+ * layered (per layer, per K/V plane) page gather/scatter and the device->pinned-host staging pipeline.
+ * Everything here is plain C: raw pointers, sizes, and two small PODs. No torch types cross the
+ * boundary; a `void* stream` is a hipStream_t (NULL = the legacy default stream).
+ *
+ * Conventions
+ *   - Every function returning int returns BIKV_OK (0) or a negative BIKV_E* code; the text of the
+ *     last failure on the calling thread is available from bikv_last_error().
+ *   - "device array" = memory the GPU can dereference (HBM, or pinned host memory mapped into the
+ *     device address space). The library never reads device arrays on the host.
+ *   - All offsets and sizes are 64-bit. (The reference computes sizes in `int`,
+ *     copy_kernel.cu:81-84, and overflows at 2 GiB.)
+ *   - Kernels bounds-check every run/tile against the extents passed here. A violating run/tile is
+ *     skipped (nothing is read or written for it) and a bit is raised in a per-device status word;
+ *     the synchronous entry points and bikv_check_status() turn that into BIKV_EBOUNDS.
+ */
+#ifndef BIKV_PAGECOPY_H
+#define BIKV_PAGECOPY_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BIKV_ABI_VERSION 1
+
+enum {
+  BIKV_OK = 0,
+  BIKV_EINVAL = -1,   /* bad argument (null pointer, negative size, misuse) */
+  BIKV_EHIP = -2,     /* a HIP runtime call failed; message carries hipGetErrorString */
+  BIKV_ESYS = -3,     /* shm_open/mmap/ftruncate/... failed; message carries strerror */
+  BIKV_ESTATE = -4,   /* role not initialised / already initialised */
+  BIKV_EBOUNDS = -5,  /* a kernel skipped at least one run/tile that fell outside its buffers */
+  BIKV_ERANGE = -6    /* request larger than a fixed capacity (ring buffer, chunk) */
+};
+
+/* Bits of the per-device status word raised by kernels. */
+enum {
+  BIKV_ST_SRC_RANGE = 1u,   /* a source run/tile was outside the source extent */
+  BIKV_ST_DST_RANGE = 2u,   /* a destination run/tile was outside the destination extent */
+  BIKV_ST_PAGE_ID = 4u      /* a page id was outside [0, n_pages) */
+};
+
+int bikv_abi_version(void);
+const char* bikv_last_error(void);
+
+/* Reads and clears the status word of `device` after synchronising `stream`.
+ * Returns BIKV_OK, or BIKV_EBOUNDS with *bits_out (nullable) holding the BIKV_ST_* bits. */
+int bikv_check_status(int device, void* stream, uint32_t* bits_out);
+
+/* Kernel launch knobs, for measurement. Keys: "seg" (batch pages per workgroup, 0 = automatic),
+ * "unroll" (16-byte vectors in flight per lane: 1, 2, 4, 8), "nontemporal" (0/1),
+ * "run_chunk_kib" (bytes of a run per workgroup, KiB; 0 = automatic). Process-wide. */
+int bikv_set_tuning(const char* key, int64_t value);
+
+/* --------------------------------------------------------------------------------------------
+ * 1. Run copy — the reference's generic offset->offset page copy.
+ *
+ * Replaces block_per_page_copy_kernel (copy_kernel.cu:9-36) and zero_copy_page_kernel
+ * (copy_kernel.cu:39-66): for every run i < n_runs
+ *     dst[dst_off[i]*unit .. +run_bytes) = src[src_off[i]*unit .. +run_bytes)
+ * Gather = scattered src_off, dense dst_off; scatter = the same call with the roles swapped.
+ * `src`/`dst` may be HBM or device-mapped pinned host memory (the zero-copy variant reads the
+ * pinned host pool directly, copy_kernel.cu:142). `src_off`/`dst_off` are int64 device arrays in
+ * units of `unit_bytes` (the reference passes element offsets; pass unit_bytes = element size, or
+ * 1 for byte offsets). Source runs may overlap or repeat; destination runs must be disjoint.
+ * Asynchronous on `stream`.
+ * ------------------------------------------------------------------------------------------ */
+int bikv_copy_runs(const void* src, int64_t src_bytes,
+                   void* dst, int64_t dst_bytes,
+                   const int64_t* src_off, const int64_t* dst_off,
+                   int64_t n_runs, int64_t run_bytes, int64_t unit_bytes,
+                   void* stream);
+
+/* --------------------------------------------------------------------------------------------
+ * 2. Layered paged pool — gather/scatter of (page, layer, K/V) tiles.
+ *
+ * The pool is the Worker-side paged KV cache (Worker.py:74-78, Model/qwen2.py:532-536): one plane
+ * per (layer, K/V) — plane index q = layer*kv_planes + kv — each holding n_pages tiles of
+ * tile_bytes contiguous bytes, consecutive pages page_stride_bytes apart. A second, optional tile
+ * class ("scale") describes per-page side data that must travel with the payload (fp32 scales of an
+ * fp8 pool): same planes and page ids, its own base pointers, tile size and stride.
+ *
+ * The staging side is an array of tile-sized slots. Page i of a call lands, for plane q, in slot
+ *     slot[i] + q * slot_stride[i]
+ * i.e. byte offset slot*tile_bytes of `staging` (and slot*scale_tile_bytes of `scale_staging`).
+ *   layer-major request buffer [L][2][m][tile]: slot = base_r + j,           slot_stride = m
+ *   page-major  request buffer [m][L][2][tile]: slot = base_r + j*n_planes,  slot_stride = 1
+ * (page-major at page granularity is the reference's token-major transfer layout, qwen2.py:519-522).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct bikv_pool bikv_pool; /* opaque; owns a small device-resident plane table */
+
+typedef struct bikv_pool_desc {
+  int32_t device;
+  int32_t n_planes;                /* layers * kv_planes */
+  int64_t n_pages;                 /* pages per plane; page ids are checked against it */
+  int64_t tile_bytes;              /* contiguous bytes of one (page, plane) tile */
+  int64_t page_stride_bytes;       /* >= tile_bytes */
+  const void* const* plane_base;   /* HOST array of n_planes device pointers */
+  int64_t scale_tile_bytes;        /* 0 = no scale class */
+  int64_t scale_page_stride_bytes;
+  const void* const* scale_plane_base; /* HOST array of n_planes device pointers, or NULL */
+} bikv_pool_desc;
+
+int bikv_pool_create(const bikv_pool_desc* desc, bikv_pool** out);
+int bikv_pool_destroy(bikv_pool* pool);
+
+/* One batch of page moves. All three index arrays are int64 device arrays of n_pages entries.
+ * Only planes [plane_begin, plane_begin+plane_count) are moved (plane_count <= 0 = all planes).
+ * `slot_bias` is subtracted from every slot before it is scaled, so a window of a larger logical
+ * staging buffer can be targeted (used by the chunked host pipeline). */
+typedef struct bikv_page_batch {
+  const int64_t* page_ids;
+  const int64_t* slots;
+  const int64_t* slot_strides;
+  int64_t n_pages;
+  int32_t plane_begin;
+  int32_t plane_count;
+  int64_t slot_bias;
+} bikv_page_batch;
+
+/* gather: pool -> staging. Duplicate and out-of-order page ids are legal. Asynchronous on stream.
+ * Replaces the per-layer form of the reference's gather (kvcache.py:132-239 driving
+ * copy_kernel.cu:9-36) for the paged compute layout. scale_staging may be NULL iff the pool has no
+ * scale class. */
+int bikv_gather_pages(const bikv_pool* pool, const bikv_page_batch* batch,
+                      void* staging, int64_t staging_bytes,
+                      void* scale_staging, int64_t scale_staging_bytes,
+                      void* stream);
+
+/* scatter: staging -> pool; the exact inverse. Page ids must be unique within the call.
+ * Replaces the Worker's disabled host scatter `send_tensor[send_indices] = compute_buffer[...]`
+ * (Worker.py:207) and the swapped-offset use of copy_kernel.cu:9-36. */
+int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* batch,
+                       const void* staging, int64_t staging_bytes,
+                       const void* scale_staging, int64_t scale_staging_bytes,
+                       void* stream);
+
+/* --------------------------------------------------------------------------------------------
+ * 3. Device -> pinned-host staging pipeline.
+ *
+ * The reference stages KV for the transport in host tensors (kvcache.py:105-108, Worker.py:203-206)
+ * that the RDMA endpoint sends from a pinned host region (onesided_rdma.h:301-337). This pipeline
+ * fills such a region: the gather runs chunk by chunk into a small ring of device buffers on a
+ * compute stream while hipMemcpyAsync drains finished chunks to `host_dst` on a copy stream.
+ *
+ * `req_pages` (HOST array, n_requests entries) gives the number of pages of each request; pages of
+ * request r occupy batch entries [sum(req_pages[:r]), +req_pages[r]) and, in staging, a contiguous
+ * block of req_pages[r]*n_planes slots whose layout is `layout`. Chunks are cut on request, plane
+ * and page boundaries so that each chunk is one contiguous byte range of the staging image.
+ * `host_dst` must be pinned (hipHostMalloc / torch pin_memory) and hold the whole staging image.
+ * Synchronous: returns when all bytes are in host memory.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct bikv_stager bikv_stager; /* opaque; owns the device chunk ring, 2 streams, events */
+
+enum { BIKV_LAYOUT_LAYER_MAJOR = 0, BIKV_LAYOUT_PAGE_MAJOR = 1 };
+enum { BIKV_STAGE_PIPELINED = 0, /* gather to HBM chunk, then hipMemcpyAsync D2H */
+       BIKV_STAGE_DIRECT = 1 };  /* kernel stores straight into the mapped pinned buffer */
+
+int bikv_stager_create(int device, int64_t chunk_bytes, int32_t n_buffers, bikv_stager** out);
+int bikv_stager_destroy(bikv_stager* st);
+
+typedef struct bikv_stage_stats {
+  int64_t bytes;        /* payload bytes delivered to host memory */
+  int64_t n_chunks;
+  double wall_seconds;  /* host wall time of the call */
+} bikv_stage_stats;
+
+int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
+                        const int64_t* req_pages, int64_t n_requests, int32_t layout,
+                        void* host_dst, int64_t host_bytes, int32_t mode,
+                        bikv_stage_stats* stats /* nullable */);
+
+/* The chunk plan bikv_gather_to_host would use, without touching a GPU: writes up to `cap` chunks
+ * as 6 int64 each (first_page, n_pages, plane_begin, plane_count, first_slot, n_slots) into `out`
+ * and returns the total number of chunks (which may exceed cap), or a negative code. */
+int64_t bikv_plan_chunks(const int64_t* req_pages, int64_t n_requests, int32_t n_planes,
+                         int32_t layout, int64_t max_slots_per_chunk, int64_t* out, int64_t cap);
+
+/* Plain pinned-buffer copy, for measuring the host link on the same box. Synchronous. */
+int bikv_d2h_copy(int device, void* host_dst, const void* dev_src, int64_t bytes,
+                  int64_t chunk_bytes /* 0 = one copy */, double* seconds_out);
+
+/* Pinned host memory (hipHostMalloc, mapped + portable). */
+int bikv_host_alloc(int64_t bytes, void** out);
+int bikv_host_free(void* p);
+
+/* --------------------------------------------------------------------------------------------
+ * 4. Producer/consumer ring — the `ipc_service` roles.
+ *
+ * The control block lives in POSIX shared memory and is byte-compatible with the reference's
+ * SharedControl (ipc_wrapper.h:14-28): sizeof 480, field offsets asserted below. The consumer
+ * creates the shm object and the device ring buffer and stores a 64-byte hipIpcMemHandle_t in
+ * `ipc_handle`; a producer in another process maps it, a producer in the SAME process uses the
+ * consumer's pointer directly. One producer role and one consumer role per process, as in the
+ * reference (ipc_service.cpp:9-17); not thread-safe.
+ * ------------------------------------------------------------------------------------------ */
+#define BIKV_IPC_HANDLE_SIZE 64
+#define BIKV_MAX_DIM 5
+
+typedef struct bikv_shared_control {
+  unsigned char sem_start[32];    /* sem_t */
+  unsigned char sem_complete[32]; /* sem_t; initialised, never waited on (as in the reference) */
+  int32_t dtype_code;             /* reference: `data_ready`, never written. 0 = float16 */
+  int32_t error_code;             /* unused, as in the reference */
+  int32_t device_id;
+  char hostname[256];
+  size_t data_size;
+  size_t tensor_dim;
+  size_t current_offset;
+  size_t last_valid_offset;
+  size_t buffer_size;
+  unsigned char ipc_handle[BIKV_IPC_HANDLE_SIZE];
+  int64_t tensor_shape[BIKV_MAX_DIM];
+} bikv_shared_control;
+
+#if defined(__cplusplus)
+static_assert(sizeof(bikv_shared_control) == 480, "SharedControl ABI");
+static_assert(offsetof(bikv_shared_control, dtype_code) == 64, "SharedControl ABI");
+static_assert(offsetof(bikv_shared_control, device_id) == 72, "SharedControl ABI");
+static_assert(offsetof(bikv_shared_control, hostname) == 76, "SharedControl ABI");
+static_assert(offsetof(bikv_shared_control, data_size) == 336, "SharedControl ABI");
+static_assert(offsetof(bikv_shared_control, tensor_dim) == 344, "SharedControl ABI");
+static_assert(offsetof(bikv_shared_control, current_offset) == 352, "SharedControl ABI");
+static_assert(offsetof(bikv_shared_control, last_valid_offset) == 360, "SharedControl ABI");
+static_assert(offsetof(bikv_shared_control, buffer_size) == 368, "SharedControl ABI");
+static_assert(offsetof(bikv_shared_control, ipc_handle) == 376, "SharedControl ABI");
+static_assert(offsetof(bikv_shared_control, tensor_shape) == 440, "SharedControl ABI");
+#endif
+
+/* TensorDims (ipc_wrapper.h:41-47). total_tokens is carried but ignored, as in the reference. */
+typedef struct bikv_tensor_dims {
+  int64_t total_tokens;
+  int64_t head_size;
+  int64_t num_kv_heads;
+  int64_t num_layers;
+  int64_t kv_pair;
+} bikv_tensor_dims;
+
+/* consumer_init (ipc_service.cpp:20-74): unlink+create shm, init semaphores, record hostname and
+ * device, allocate the device ring, publish its IPC handle. */
+int bikv_consumer_init(int device, const char* shm_name, size_t buffer_bytes);
+/* producer_init (ipc_service.cpp:77-110): open shm, same-host check, map the ring. */
+int bikv_producer_init(int device, const char* shm_name);
+/* producer_cleanup / consumer_cleanup (ipc_service.cpp:171-202). Idempotent. */
+void bikv_producer_cleanup(void);
+void bikv_consumer_cleanup(void);
+
+/* producer_copy_pages / producer_zero_copy_pages (ipc_service.cpp:205-239 ->
+ * copy_kernel.cu:68-129,133-196): run copy from `src` into the ring at the current write offset,
+ * then the reference's bookkeeping — wrap to 0 if the batch does not fit behind current_offset,
+ * last_valid_offset = current_offset, current_offset += data_size, tensor_dim = 5,
+ * tensor_shape = [n_runs*page_size, head, kv_heads, layers, kv_pair], sem_post(sem_start).
+ * data_size = n_runs*page_size*head*kv_heads*layers*kv_pair*elem_bytes (the reference hard-codes
+ * sizeof(half), copy_kernel.cu:84). Offsets are int64 device arrays in ELEMENTS. `src` may be HBM
+ * or mapped pinned host memory. Blocks until the copy has finished (stream sync, where the
+ * reference uses cudaDeviceSynchronize). dtype_code is published for the consumer. */
+int bikv_producer_copy_pages(const void* src, int64_t src_bytes,
+                             const int64_t* src_off, const int64_t* dst_off, int64_t n_runs,
+                             int64_t page_size, const bikv_tensor_dims* dims,
+                             int64_t elem_bytes, int32_t dtype_code, void* stream);
+
+/* producer_send (ipc_service.cpp:113-143): contiguous device tensor -> ring, publishes the real
+ * shape (ndim <= 5). */
+int bikv_producer_send(const void* dev_src, size_t bytes, const int64_t* shape, size_t ndim,
+                       int32_t dtype_code, void* stream);
+
+/* consumer_receive (ipc_service.cpp:146-168): sem_wait(sem_start) (timeout_ms < 0 = wait forever,
+ * as the reference does; on timeout returns BIKV_ESTATE), then hands out a NON-OWNING pointer into
+ * the ring, valid until the producer wraps over it. */
+int bikv_consumer_receive(int64_t timeout_ms, void** ptr, int64_t shape[BIKV_MAX_DIM],
+                          size_t* ndim, size_t* data_bytes, int32_t* device_id,
+                          int32_t* dtype_code);
+
+/* Read-only views for tests and diagnostics (NULL when the role is not initialised). */
+const bikv_shared_control* bikv_producer_control(void);
+const bikv_shared_control* bikv_consumer_control(void);
+void* bikv_consumer_buffer(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BIKV_PAGECOPY_H */

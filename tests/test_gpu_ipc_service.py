@@ -1,0 +1,187 @@
+"""The `ipc_service` drop-in on a real GPU: the reference's two scripted scenarios
+(Bi-KV/SharedMemory/CUDA_Shared/test_page_ipc.py, test_zero_copy.py) with producer and consumer in
+one process, seeded-data variants of them (the constant-7 data of the originals cannot detect a
+wrong offset), producer_send / consumer_receive, ring wrap-around and the error paths."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture()
+def ipc(lib, cuda):
+    import ipc_service
+    ipc_service.producer_cleanup()
+    ipc_service.consumer_cleanup()
+    yield ipc_service
+    ipc_service.producer_cleanup()
+    ipc_service.consumer_cleanup()
+
+
+def _dims(ipc, s, total_tokens):
+    d = ipc.TensorDims()
+    d.total_tokens = total_tokens
+    d.head_size, d.num_kv_heads, d.num_layers, d.kv_pair = s["head_size"], s["num_kv_heads"], s["num_layers"], s["kv_pair"]
+    return d
+
+
+def _scenario(name):
+    with open(os.path.join(GOLDEN, "reference_scenarios.json")) as f:
+        return json.load(f)[name]
+
+
+def test_reference_page_ipc_scenario(ipc, cuda):
+    """200 pages x 50 tokens of 7s, identity offsets, 2 GiB ring, 10 transfers: dim 5, shape
+    (10000,128,2,28,2), all 7 (test_page_ipc.py:127-150); and the ring advances by 273.4 MiB per
+    transfer and restarts at 0 when the next batch would not fit."""
+    s = _scenario("test_page_ipc")
+    print("[case] reference test_page_ipc scenario", flush=True)
+    name = f"/bikv_test_page_ipc_{os.getpid()}"
+    ipc.consumer_init(0, name, s["buffer_size"])
+    ipc.producer_init(0, name.encode())       # callers pass bytes (kvcache.py:72) or str (the scripts)
+    ept = s["head_size"] * s["num_kv_heads"] * s["num_layers"] * s["kv_pair"]
+    page_elements = s["page_size"] * ept
+    n = s["num_pages"]
+    cache = torch.full((n, s["page_size"], s["head_size"], s["num_kv_heads"], s["num_layers"], s["kv_pair"]),
+                       s["fill_value"], dtype=torch.float16, device=cuda)
+    offs = torch.tensor([i * page_elements for i in range(n)], dtype=torch.int64, device=cuda)
+    dims = _dims(ipc, s, n * s["page_size"])
+    per = n * page_elements * 2
+    ptrs = []
+    for k in range(s["num_transfers"] - 1):
+        ipc.producer_copy_pages(cache, offs, offs, s["page_size"], dims)
+        result = ipc.consumer_receive()
+        assert result.dim() == s["expected_dim"]
+        assert tuple(result.shape) == tuple(s["expected_shape"])
+        assert result.dtype == torch.float16 and result.device == cuda
+        assert torch.allclose(result, torch.full_like(result, s["expected_value"]))
+        ptrs.append(result.data_ptr())
+    fit = s["buffer_size"] // per            # 7 transfers fit a 2 GiB ring
+    base = ptrs[0]
+    assert [p - base for p in ptrs] == [(k % fit) * per for k in range(len(ptrs))]
+
+
+def test_reference_zero_copy_scenario(ipc, cuda):
+    s = _scenario("test_zero_copy")
+    print("[case] reference test_zero_copy scenario", flush=True)
+    name = f"/bikv_test_zero_copy_{os.getpid()}"
+    ipc.consumer_init(0, name, s["buffer_size"])
+    ipc.producer_init(0, name)
+    ept = s["head_size"] * s["num_kv_heads"] * s["num_layers"] * s["kv_pair"]
+    page_elements = s["page_size"] * ept
+    n = s["num_pages"]
+    cpu_data = torch.full((n * page_elements,), s["fill_value"], dtype=torch.float16).pin_memory()
+    page_indices = torch.arange(n, dtype=torch.int64, device=cuda)
+    dest = torch.arange(0, n * page_elements, page_elements, dtype=torch.int64, device=cuda)
+    dims = _dims(ipc, s, n * s["page_size"])
+    for _ in range(3):
+        ipc.producer_zero_copy_pages(cpu_data, page_indices, dest, s["page_size"], dims)
+        t = ipc.consumer_receive()
+        assert tuple(t.shape) == tuple(s["expected_shape"])
+        assert torch.all(t == s["expected_value"])
+        assert t.is_cuda
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.uint8])
+def test_copy_pages_seeded_data_against_oracle(ipc, oracle, cuda, dtype):
+    """Random data, shuffled page order, duplicate source pages: what constant data cannot check."""
+    print(f"[case] producer_copy_pages seeded {dtype}", flush=True)
+    name = f"/bikv_test_seeded_{os.getpid()}"
+    d = ipc.TensorDims()
+    d.head_size, d.num_kv_heads, d.num_layers, d.kv_pair = 64, 2, 3, 2
+    page_size, pool_pages, n = 16, 40, 23
+    page_elements = page_size * 64 * 2 * 3 * 2
+    es = torch.empty((), dtype=dtype).element_size()
+    ipc.consumer_init(0, name, 3 * n * page_elements * es + 1000)
+    ipc.producer_init(0, name)
+    rng = np.random.default_rng(17)
+    np_dt = {1: np.uint8, 2: np.uint16}[es]
+    pool_h = rng.integers(0, 256, size=pool_pages * page_elements * es, dtype=np.uint8).view(np_dt)
+    pool_d = torch.from_numpy(pool_h.view(np.uint8)).to(cuda).view(dtype)
+    for step in range(4):                                   # the 4th transfer wraps
+        ids = rng.integers(0, pool_pages, size=n)
+        so = ids * page_elements
+        do = rng.permutation(n).astype(np.int64) * page_elements
+        ipc.producer_copy_pages(pool_d, torch.from_numpy(so).to(cuda), torch.from_numpy(do).to(cuda), page_size, d)
+        got = ipc.consumer_receive(timeout_ms=5000)
+        assert got.dtype == dtype and tuple(got.shape) == (n * page_size, 64, 2, 3, 2)
+        want = np.zeros(n * page_elements, dtype=np_dt)
+        oracle.copy_runs_c(pool_h, want, so, do, page_elements)
+        assert got.cpu().contiguous().view(torch.uint8).numpy().tobytes() == want.tobytes()
+    from bikv_pagecopy import _lib
+    ctrl = _lib.load().bikv_consumer_control().contents
+    ring = oracle.Ring(buffer_size=ctrl.buffer_size)
+    for step in range(4):
+        oracle.ring_step_c(ring, n, page_size, (64, 2, 3, 2), es)
+    assert (ctrl.current_offset, ctrl.last_valid_offset, ctrl.data_size, ctrl.tensor_dim) == \
+        (ring.current_offset, ring.last_valid_offset, ring.data_size, ring.tensor_dim)
+    assert list(ctrl.tensor_shape) == list(ring.tensor_shape)
+
+
+def test_producer_send_round_trip(ipc, oracle, cuda):
+    print("[case] producer_send / consumer_receive", flush=True)
+    name = f"/bikv_test_send_{os.getpid()}"
+    ipc.consumer_init(0, name, 1 << 20)
+    ipc.producer_init(0, name)
+    ring = oracle.Ring(buffer_size=1 << 20)
+    base = None
+    for shape in [(1000, 128), (7, 5, 3, 2, 4), (300000,), (300000,), (2, 3)]:
+        t = torch.randn(shape, device=cuda).to(torch.float16)
+        ipc.producer_send(t)
+        r = ipc.consumer_receive(timeout_ms=5000)
+        assert r.shape == t.shape and r.dtype == torch.float16 and torch.equal(r, t)
+        at = oracle.ring_send_c(ring, t.numel() * 2, list(shape))
+        base = base if base is not None else r.data_ptr() - at
+        assert r.data_ptr() - base == at            # same wrap rule as the reference
+    with pytest.raises(RuntimeError, match="float16"):
+        ipc.producer_send(torch.zeros(4, device=cuda))
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ipc.producer_send(torch.zeros(4, 4, dtype=torch.float16, device=cuda).t())
+    with pytest.raises(RuntimeError, match="CUDA"):
+        ipc.producer_send(torch.zeros(4, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="does not fit"):
+        ipc.producer_send(torch.zeros(1 << 20, dtype=torch.float16, device=cuda))
+
+
+def test_error_paths(ipc, cuda):
+    print("[case] ipc_service error paths", flush=True)
+    name = f"/bikv_test_err_{os.getpid()}"
+    d = ipc.TensorDims()
+    d.head_size, d.num_kv_heads, d.num_layers, d.kv_pair = 8, 1, 1, 2
+    off = torch.zeros(2, dtype=torch.int64, device=cuda)
+    data = torch.zeros(1024, dtype=torch.float16, device=cuda)
+    with pytest.raises(RuntimeError, match="not initialised"):
+        ipc.producer_copy_pages(data, off, off, 4, d)
+    with pytest.raises(RuntimeError, match="not initialised"):
+        ipc.consumer_receive(timeout_ms=10)
+    ipc.consumer_init(0, name, 4096)
+    with pytest.raises(RuntimeError, match="already initialised"):
+        ipc.consumer_init(0, name, 4096)
+    ipc.producer_init(0, name)
+    with pytest.raises(RuntimeError, match="timed out"):
+        ipc.consumer_receive(timeout_ms=50)             # nothing was produced
+    with pytest.raises(RuntimeError, match="Cache data must be on CUDA"):
+        ipc.producer_copy_pages(data.cpu(), off, off, 4, d)
+    with pytest.raises(RuntimeError, match="Cache data must be contiguous"):
+        ipc.producer_copy_pages(data[::2], off, off, 4, d)
+    with pytest.raises(RuntimeError, match="CPU data must be pinned memory"):
+        ipc.producer_zero_copy_pages(data.cpu(), off, off, 4, d)
+    with pytest.raises(RuntimeError, match="Page indices must be on CUDA"):
+        ipc.producer_zero_copy_pages(data.cpu().pin_memory(), off.cpu(), off, 4, d)
+    with pytest.raises(RuntimeError, match="does not fit"):
+        ipc.producer_copy_pages(data, torch.zeros(64, dtype=torch.int64, device=cuda),
+                                torch.zeros(64, dtype=torch.int64, device=cuda), 4, d)
+    bad = torch.tensor([0, 100000], dtype=torch.int64, device=cuda)
+    with pytest.raises(RuntimeError, match="source-range"):
+        ipc.producer_copy_pages(data, bad, torch.tensor([0, 64], dtype=torch.int64, device=cuda), 4, d)
+    # nothing was published by the failed calls
+    with pytest.raises(RuntimeError, match="timed out"):
+        ipc.consumer_receive(timeout_ms=50)
+    ipc.consumer_cleanup()
+    assert not os.path.exists("/dev/shm" + name)        # the consumer unlinks its object

@@ -1,0 +1,395 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI, on a real GPU.
+
+Bit-exact is the bar everywhere: this path moves bytes. Every comparison is on raw bytes, so NaN
+payloads and fp8 bit patterns count.
+"""
+import hashlib
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _announce(msg):
+    print(f"[case] {msg}", flush=True)
+
+
+def _rand_pool(rng, n_planes, n_pages, tile_bytes):
+    return rng.integers(0, 256, size=(n_planes, n_pages, tile_bytes), dtype=np.uint8)
+
+
+def _to_np(t):
+    return t.detach().cpu().contiguous().view(torch.uint8).numpy()
+
+
+@pytest.fixture(scope="module")
+def bk(lib):
+    import bikv_pagecopy
+    return bikv_pagecopy
+
+
+# ---- configuration 1, against the committed digests and the oracle ------------------------------
+@pytest.mark.parametrize("layout", ["layer_major", "page_major"])
+def test_config1_gather_scatter_bit_exact(bk, oracle, cuda, layout):
+    from bikv_pagecopy import workloads
+    _announce(f"config1 {layout}")
+    with open(os.path.join(GOLDEN, "config1.json")) as f:
+        g = json.load(f)
+    shape = workloads.SHAPES["tiny"]
+    wl = workloads.named("tiny")
+    pool_h = np.random.default_rng(0).standard_normal(
+        (shape.n_planes, shape.n_pages, shape.tile_bytes // 2)).astype(np.float16)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    batch = pool.make_batch(wl["gather"], layout)
+    staging, _ = pool.gather(batch)
+    pool.check()
+    got = _to_np(staging)
+    want = oracle.gather_layered_c(pool_h, wl["gather"], layout)
+    assert got.tobytes() == want.tobytes()
+    assert hashlib.sha256(got.tobytes()).hexdigest() == g[layout]["staging_sha256"]
+    # the per-request view is the contiguous [64, 16, 2, 64] buffer per plane the config asks for
+    v = batch.request_view(staging.view(torch.float16), 0)
+    if layout == "layer_major":
+        assert v.shape == (2, 64, 16 * 2 * 64)
+        assert torch.equal(v[1].cpu(), torch.from_numpy(pool_h[1, wl["gather"][0]]))
+    sbatch = pool.make_batch(wl["scatter"], layout)
+    pool.scatter(sbatch, staging)
+    pool.check()
+    oracle.scatter_layered_c(pool_h, wl["scatter"], want, layout)
+    after = _to_np(pool_d)
+    assert after.tobytes() == pool_h.tobytes()
+    assert hashlib.sha256(after.tobytes()).hexdigest() == g[layout]["pool_after_scatter_sha256"]
+
+
+# ---- the other four shapes with scaled-down pools -----------------------------------------------
+def _run_shape(bk, oracle, cuda, shape, wl, layout, seed):
+    rng = np.random.default_rng(seed)
+    pool_h = _rand_pool(rng, shape.n_planes, shape.n_pages, shape.tile_bytes)
+    scale_h = _rand_pool(rng, shape.n_planes, shape.n_pages, shape.scale_tile_bytes) if shape.scales else None
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    scale_d = torch.from_numpy(scale_h).to(cuda) if shape.scales else None
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1, scale=scale_d)
+    batch = pool.make_batch(wl["gather"], layout)
+    staging, sstaging = pool.gather(batch)
+    pool.check()
+    want = oracle.gather_layered_c(pool_h, wl["gather"], layout)
+    assert _to_np(staging).tobytes() == want.tobytes()
+    if shape.scales:
+        swant = oracle.gather_layered_c(scale_h, wl["gather"], layout)
+        assert _to_np(sstaging).tobytes() == swant.tobytes()
+    if wl.get("scatter"):
+        # scatter the first len(scatter) requests' worth of staged data into fresh pages
+        sreq = wl["scatter"]
+        src_reqs = [rng.permutation(shape.n_pages)[: len(r)] for r in sreq]
+        sb_src = pool.make_batch(src_reqs, layout)
+        st2, sst2 = pool.gather(sb_src)
+        pool.check()
+        w2 = oracle.gather_layered_c(pool_h, src_reqs, layout)
+        sb = pool.make_batch(sreq, layout)
+        pool.scatter(sb, st2, sst2)
+        pool.check()
+        oracle.scatter_layered_c(pool_h, sreq, w2, layout)
+        assert _to_np(pool_d).tobytes() == pool_h.tobytes()
+        if shape.scales:
+            sw2 = oracle.gather_layered_c(scale_h, src_reqs, layout)
+            oracle.scatter_layered_c(scale_h, sreq, sw2, layout)
+            assert _to_np(scale_d).tobytes() == scale_h.tobytes()
+
+
+@pytest.mark.parametrize("layout", ["layer_major", "page_major"])
+def test_qwen2_1p5b_shape_scaled_pool(bk, oracle, cuda, layout):
+    from bikv_pagecopy import workloads as w
+    shape = w.SHAPES["qwen2_1p5b"].scaled(384)   # 8 KiB tiles, 56 planes: 2 tiles per unrolled pass
+    wl = w.uniform_requests(shape, 6, 512, 1024, seed=2)
+    _announce(f"qwen2_1p5b scaled {layout}: {sum(map(len, wl['gather']))} pages")
+    _run_shape(bk, oracle, cuda, shape, wl, layout, 102)
+
+
+def test_qwen2_7b_shape_scaled_pool_with_duplicates(bk, oracle, cuda):
+    from bikv_pagecopy import workloads as w
+    shape = w.SHAPES["qwen2_7b"].scaled(256)     # 16 KiB tiles
+    wl = w.mixed_gather_scatter(shape, 6, 256, 1024, seed=3, dup_fraction=0.10)
+    g = np.concatenate(wl["gather"])
+    assert len(set(g.tolist())) < len(g), "workload must contain duplicate gather ids"
+    _announce(f"qwen2_7b scaled: {len(g)} gather pages, dup present")
+    _run_shape(bk, oracle, cuda, shape, wl, "layer_major", 103)
+
+
+def test_llama3_8b_shape_scaled_pool(bk, oracle, cuda):
+    from bikv_pagecopy import workloads as w
+    shape = w.SHAPES["llama3_8b"].scaled(48)      # 64 KiB tiles: four unrolled passes per tile
+    wl = w.lognormal_requests(shape, 5, 256, 1024, seed=4)
+    _announce(f"llama3_8b scaled: {sum(map(len, wl['gather']))} pages")
+    _run_shape(bk, oracle, cuda, shape, wl, "layer_major", 104)
+
+
+@pytest.mark.parametrize("layout", ["layer_major", "page_major"])
+def test_llama3_70b_fp8_payload_and_scales_move_together(bk, oracle, cuda, layout):
+    from bikv_pagecopy import workloads as w
+    shape = w.SHAPES["llama3_70b_fp8"].scaled(96)  # 16 KiB payload + 32 B scales, 160 planes
+    wl = w.zipf_requests(shape, 12, 16, 512, seed=5)
+    assert wl["scatter"], "need a scatter leg"
+    _announce(f"llama3_70b_fp8 scaled {layout}: {sum(map(len, wl['gather']))} pages")
+    _run_shape(bk, oracle, cuda, shape, wl, layout, 105)
+
+
+# ---- shapes the fast mover does not take ----------------------------------------------------------
+@pytest.mark.parametrize("tile_bytes", [16, 48, 100, 1000, 4096 * 3, 4096 + 16, 2, 7])
+def test_odd_tile_sizes(bk, oracle, cuda, tile_bytes):
+    _announce(f"odd tile {tile_bytes}")
+    rng = np.random.default_rng(tile_bytes)
+    pool_h = _rand_pool(rng, 3, 70, tile_bytes)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    reqs = [rng.permutation(70)[:33], np.array([4, 4, 4]), rng.permutation(70)[:1]]
+    batch = pool.make_batch(reqs)
+    staging, _ = pool.gather(batch)
+    pool.check()
+    assert _to_np(staging).tobytes() == oracle.gather_layered_c(pool_h, reqs).tobytes()
+
+
+def test_misaligned_pool_and_staging(bk, oracle, cuda):
+    """Pool planes and staging that start 2 bytes off a 16-byte boundary take the narrow mover."""
+    _announce("misaligned")
+    rng = np.random.default_rng(77)
+    n_planes, n_pages, tile = 2, 40, 8192
+    backing = torch.zeros(n_planes * n_pages * tile + 64, dtype=torch.uint8, device=cuda)
+    pool_h = _rand_pool(rng, n_planes, n_pages, tile)
+    view = backing[2: 2 + pool_h.size].view(n_planes, n_pages, tile)
+    view.copy_(torch.from_numpy(pool_h))
+    assert view.data_ptr() % 16 == 2
+    pool = bk.PagedKVPool([view[q].data_ptr() for q in range(n_planes)], n_pages, tile, tile, cuda)
+    reqs = [rng.permutation(n_pages)[:17]]
+    batch = pool.make_batch(reqs)
+    st_back = torch.zeros(batch.n_slots * tile + 64, dtype=torch.uint8, device=cuda)
+    staging = st_back[6: 6 + batch.n_slots * tile]
+    pool.gather(batch, staging)
+    pool.check()
+    assert _to_np(staging).tobytes() == oracle.gather_layered_c(pool_h, reqs).tobytes()
+    assert not st_back[:6].any() and not st_back[6 + batch.n_slots * tile:].any()
+
+
+def test_kv_adjacent_layer_layout(bk, oracle, cuda):
+    """Per-layer [pages, 2, block, heads, dim] tensors as in Model/qwen2.py:532-536."""
+    _announce("kv-adjacent layers")
+    rng = np.random.default_rng(31)
+    L, N, P, H, D = 3, 24, 16, 2, 128
+    layers_h = [rng.standard_normal((N, 2, P, H, D)).astype(np.float16) for _ in range(L)]
+    layers_d = [torch.from_numpy(a).to(cuda) for a in layers_h]
+    pool = bk.PagedKVPool.from_layers_kv_adjacent(layers_d)
+    assert pool.n_planes == 2 * L and pool.page_stride_bytes == 2 * pool.tile_bytes
+    # the oracle's plane-major view of the same data
+    planes_h = np.stack([layers_h[l][:, k].reshape(N, -1) for l in range(L) for k in range(2)])
+    reqs = [rng.permutation(N)[:9], rng.permutation(N)[:4]]
+    batch = pool.make_batch(reqs)
+    staging, _ = pool.gather(batch)
+    pool.check()
+    want = oracle.gather_layered_c(np.ascontiguousarray(planes_h), reqs)
+    assert _to_np(staging).tobytes() == want.view(np.uint8).tobytes()
+    # scatter back into other pages and compare each layer tensor
+    perm = rng.permutation(N)
+    sreqs = [perm[:9], perm[9:13]]
+    pool.scatter(pool.make_batch(sreqs), staging)
+    pool.check()
+    planes_c = np.ascontiguousarray(planes_h)
+    oracle.scatter_layered_c(planes_c, sreqs, want)
+    for l in range(L):
+        got = layers_d[l].cpu().numpy()
+        for k in range(2):
+            assert got[:, k].reshape(N, -1).tobytes() == planes_c[2 * l + k].tobytes()
+
+
+# ---- edge cases ----------------------------------------------------------------------------------
+def test_empty_batch_and_empty_requests(bk, oracle, cuda):
+    _announce("empty")
+    pool_d = torch.zeros((2, 8, 4096), dtype=torch.uint8, device=cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    b = pool.make_batch([])
+    st, _ = pool.gather(b)
+    pool.check()
+    assert st.numel() == 0
+    b = pool.make_batch([[], [], []])
+    st, _ = pool.gather(b)
+    pool.check()
+    assert st.numel() == 0
+
+
+def test_nan_payloads_and_all_bit_patterns_survive(bk, cuda):
+    _announce("bit patterns")
+    allbits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(torch.float16)  # every fp16 pattern
+    pool_d = allbits.repeat(2 * 16).view(2, 16, 65536).contiguous().to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    b = pool.make_batch([[15, 0, 15]])
+    st, _ = pool.gather(b)
+    pool.check()
+    got = st.view(torch.int16).view(2, 3, 65536).cpu()
+    assert torch.equal(got[0, 0], allbits.view(torch.int16)) and torch.equal(got[1, 2], allbits.view(torch.int16))
+
+
+def test_plane_subrange_and_slot_bias(bk, oracle, cuda, lib):
+    """The windowed form the host pipeline uses: planes [q0, q0+k) into a window of the image."""
+    import ctypes as C
+    from bikv_pagecopy import _lib
+    _announce("plane window")
+    rng = np.random.default_rng(55)
+    pool_h = _rand_pool(rng, 8, 30, 4096)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    reqs = [rng.permutation(30)[:11]]
+    batch = pool.make_batch(reqs)
+    want = oracle.gather_layered_c(pool_h, reqs).reshape(8, 11, 4096)
+    window = torch.full((3 * 11 * 4096,), 0xA5, dtype=torch.uint8, device=cuda)
+    d = batch.desc(plane_begin=2, plane_count=3, slot_bias=2 * 11)
+    _lib.check(lib.bikv_gather_pages(pool._h, C.byref(d), window.data_ptr(), window.numel(), None, 0,
+                                     C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    pool.check()
+    assert _to_np(window).tobytes() == want[2:5].tobytes()
+
+
+def test_out_of_range_ids_and_slots_are_skipped_and_reported(bk, oracle, cuda):
+    """A bad page id or a staging buffer that is too small must not touch memory outside the
+    buffers: the tile is skipped, the call reports it, every other tile is still moved."""
+    _announce("bounds rejection")
+    rng = np.random.default_rng(66)
+    pool_h = _rand_pool(rng, 2, 20, 4096)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    reqs = [np.array([3, 20, 5, -1, 7], dtype=np.int64)]
+    batch = pool.make_batch(reqs)
+    st = torch.full((batch.n_slots * 4096,), 0xA5, dtype=torch.uint8, device=cuda)
+    pool.gather(batch, st)
+    with pytest.raises(RuntimeError, match="page-id"):
+        pool.check()
+    got = _to_np(st).reshape(2, 5, 4096)
+    for j, pid in enumerate(reqs[0]):
+        if 0 <= pid < 20:
+            assert np.array_equal(got[:, j], pool_h[:, pid])
+        else:
+            assert np.all(got[:, j] == 0xA5)
+    pool.check()  # status was cleared by the failing check
+    good = pool.make_batch([np.array([1, 2, 3, 4])])
+    small = torch.full((2 * 4 * 4096 - 4096,), 0xA5, dtype=torch.uint8, device=cuda)  # one slot short
+    pool.gather(good, small)
+    with pytest.raises(RuntimeError, match="destination-range"):
+        pool.check()
+    # scatter with a bad id leaves the pool untouched for that id
+    before = _to_np(pool_d).copy()
+    bad = pool.make_batch([np.array([25])])
+    pool.scatter(bad, torch.zeros(2 * 4096, dtype=torch.uint8, device=cuda))
+    with pytest.raises(RuntimeError, match="page-id"):
+        pool.check()
+    assert _to_np(pool_d).tobytes() == before.tobytes()
+
+
+def test_tuning_knobs_do_not_change_results(bk, oracle, cuda):
+    _announce("launch geometry independence")
+    rng = np.random.default_rng(88)
+    pool_h = _rand_pool(rng, 4, 64, 16384)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    reqs = [rng.permutation(64)[:37], rng.permutation(64)[:5]]
+    want = oracle.gather_layered_c(pool_h, reqs).tobytes()
+    batch = pool.make_batch(reqs)
+    try:
+        for seg in (0, 1, 3, 16, 256):
+            for unroll in (1, 2, 4, 8):
+                for nt in (0, 1):
+                    bk.set_tuning(seg=seg, unroll=unroll, nontemporal=nt)
+                    st = torch.zeros(batch.n_slots * 16384, dtype=torch.uint8, device=cuda)
+                    pool.gather(batch, st)
+                    pool.check()
+                    assert _to_np(st).tobytes() == want, (seg, unroll, nt)
+    finally:
+        bk.set_tuning(seg=0, unroll=4, nontemporal=1)
+
+
+# ---- run copy (reference API) -------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,run_elems", [
+    (torch.float16, 14336 * 16), (torch.bfloat16, 4096), (torch.float32, 1000), (torch.float64, 33),
+    (torch.uint8, 5), (torch.uint8, 2049), (torch.float16, 8), (torch.float16, 1029)])
+def test_copy_runs_gather_and_scatter(bk, oracle, cuda, dtype, run_elems):
+    _announce(f"copy_runs {dtype} run_elems={run_elems}")
+    rng = np.random.default_rng(run_elems)
+    es = torch.empty((), dtype=dtype).element_size()
+    n_pages, n = 37, 19
+    src_h = rng.integers(0, 256, size=n_pages * run_elems * es, dtype=np.uint8)
+    src_d = torch.from_numpy(src_h).to(cuda).view(dtype)
+    ids = rng.integers(0, n_pages, size=n)                  # duplicates allowed on the source side
+    so = ids * run_elems
+    do = rng.permutation(n).astype(np.int64) * run_elems    # dense but out of order
+    dst_d = torch.full((n * run_elems * es,), 0xA5, dtype=torch.uint8, device=cuda).view(dtype)
+    bk.copy_runs(src_d, dst_d, torch.from_numpy(so).to(cuda), torch.from_numpy(do).to(cuda), run_elems)
+    from bikv_pagecopy import runs
+    runs.check(cuda)
+    dst_h = np.full(n * run_elems * es, 0xA5, dtype=np.uint8)
+    np_dt = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[es]
+    assert oracle.copy_runs_c(src_h.view(np_dt), dst_h.view(np_dt), so, do, run_elems) == 0
+    assert _to_np(dst_d).tobytes() == dst_h.tobytes()
+    # scatter back: dense source, scattered unique destinations
+    back_ids = rng.permutation(n_pages)[:n].astype(np.int64) * run_elems
+    pool2_d = torch.zeros_like(src_d)
+    bk.copy_runs(dst_d, pool2_d, torch.from_numpy(do).to(cuda), torch.from_numpy(back_ids).to(cuda), run_elems)
+    runs.check(cuda)
+    pool2_h = np.zeros_like(src_h)
+    oracle.copy_runs_c(dst_h.view(np_dt), pool2_h.view(np_dt), do, back_ids, run_elems)
+    assert _to_np(pool2_d).tobytes() == pool2_h.tobytes()
+
+
+def test_copy_runs_element_offsets_that_break_16_byte_alignment(bk, oracle, cuda):
+    """fp16 element offsets need only be 2-byte aligned: every run picks its own access width."""
+    _announce("copy_runs unaligned offsets")
+    rng = np.random.default_rng(12)
+    run = 3000
+    src_h = rng.integers(0, 65536, size=40000, dtype=np.uint16)
+    so = np.array([0, 1, 2, 3, 4, 8, 1001, 20000], dtype=np.int64)
+    do = np.array([0, 3001, 6003, 9008, 12012, 15015, 18023, 21024], dtype=np.int64)
+    dst_h = np.full(25000, 0xA5A5, dtype=np.uint16)
+    oracle.copy_runs_c(src_h, dst_h, so, do, run)
+    src_d = torch.from_numpy(src_h.view(np.int16)).to(cuda).view(torch.float16)
+    dst_d = torch.from_numpy(np.full(25000, 0xA5A5, dtype=np.uint16).view(np.int16)).to(cuda).view(torch.float16)
+    bk.copy_runs(src_d, dst_d, torch.from_numpy(so).to(cuda), torch.from_numpy(do).to(cuda), run)
+    from bikv_pagecopy import runs
+    runs.check(cuda)
+    assert _to_np(dst_d).tobytes() == dst_h.tobytes()
+
+
+def test_copy_runs_rejects_offsets_outside_the_buffers(bk, cuda):
+    _announce("copy_runs bounds")
+    from bikv_pagecopy import runs
+    src = torch.arange(0, 4096, dtype=torch.int16, device=cuda)
+    dst = torch.zeros(4096, dtype=torch.int16, device=cuda)
+    so = torch.tensor([0, 4000, -5, 1024], dtype=torch.int64, device=cuda)
+    do = torch.tensor([0, 1024, 2048, 3500], dtype=torch.int64, device=cuda)
+    bk.copy_runs(src, dst, so, do, 1024)
+    with pytest.raises(RuntimeError, match="source-range"):
+        runs.check(cuda)
+    assert torch.equal(dst[:1024], src[:1024]) and not dst[1024:].any()
+    with pytest.raises(RuntimeError, match="contiguous"):
+        bk.copy_runs(src[::2], dst, so, do, 4)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        bk.copy_runs(src, dst, so.cpu(), do, 4)
+
+
+def test_copy_runs_zero_copy_from_pinned_host(bk, oracle, cuda):
+    """The zero_copy_page_kernel form: the source is pinned host memory read by the GPU."""
+    _announce("copy_runs pinned source")
+    rng = np.random.default_rng(13)
+    run = 14336 * 4
+    src_h = rng.integers(0, 65536, size=12 * run, dtype=np.uint16)
+    pinned = torch.from_numpy(src_h.view(np.int16)).pin_memory().view(torch.float16)
+    ids = rng.permutation(12)[:7].astype(np.int64)
+    so, do = ids * run, np.arange(7, dtype=np.int64) * run
+    dst = torch.zeros(7 * run, dtype=torch.float16, device=cuda)
+    bk.copy_runs(pinned, dst, torch.from_numpy(so).to(cuda), torch.from_numpy(do).to(cuda), run, device=cuda)
+    from bikv_pagecopy import runs
+    runs.check(cuda)
+    want = np.zeros(7 * run, dtype=np.uint16)
+    oracle.copy_runs_c(src_h, want, so, do, run)
+    assert _to_np(dst).tobytes() == want.tobytes()

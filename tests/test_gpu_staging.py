@@ -1,0 +1,64 @@
+"""Device -> pinned-host staging on a real GPU: both modes against the oracle's staging image."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("layout", ["layer_major", "page_major"])
+@pytest.mark.parametrize("mode", ["pipelined", "direct"])
+def test_gather_to_host_matches_oracle(lib, oracle, cuda, layout, mode):
+    import bikv_pagecopy as bk
+    print(f"[case] gather_to_host {layout} {mode}", flush=True)
+    rng = np.random.default_rng(41)
+    n_planes, n_pages, tile = 6, 90, 16384
+    pool_h = rng.integers(0, 256, size=(n_planes, n_pages, tile), dtype=np.uint8)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    # request sizes around the chunk size: whole-plane-row chunks, split rows, a single page, empty
+    reqs = [rng.permutation(n_pages)[:m] for m in (3, 40, 1, 0, 17)]
+    batch = pool.make_batch(reqs, layout)
+    want = oracle.gather_layered_c(pool_h, reqs, layout).tobytes()
+    for chunk_tiles, n_buf in ((8, 2), (1, 3), (64, 1)):
+        stager = bk.HostStager(cuda, chunk_bytes=chunk_tiles * tile, n_buffers=n_buf)
+        host = bk.pinned_empty(batch.n_slots * tile)
+        host.fill_(0xA5)
+        nbytes, n_chunks, sec = stager.gather_to_host(pool, batch, host, mode)
+        assert nbytes == batch.n_slots * tile and sec > 0
+        assert host.numpy().tobytes() == want, (chunk_tiles, n_buf)
+        if mode == "pipelined":
+            plan = bk.plan_chunks(batch.req_pages, n_planes, layout, chunk_tiles)
+            assert n_chunks == len(plan)
+        stager.close()
+
+
+def test_gather_to_host_argument_checks(lib, cuda):
+    import bikv_pagecopy as bk
+    print("[case] gather_to_host checks", flush=True)
+    pool_d = torch.zeros((2, 8, 4096), dtype=torch.uint8, device=cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    batch = pool.make_batch([[1, 2, 3]])
+    stager = bk.HostStager(cuda, chunk_bytes=4096, n_buffers=2)
+    with pytest.raises(RuntimeError, match="pinned"):
+        stager.gather_to_host(pool, batch, torch.empty(batch.n_slots * 4096, dtype=torch.uint8))
+    with pytest.raises(RuntimeError, match="staging image needs"):
+        stager.gather_to_host(pool, batch, bk.pinned_empty(4096))
+    tiny = bk.HostStager(cuda, chunk_bytes=4096, n_buffers=1)
+    big_d = torch.zeros((1, 4, 8192), dtype=torch.uint8, device=cuda)
+    big = bk.PagedKVPool.from_stacked(big_d, plane_dims=1)
+    with pytest.raises(RuntimeError, match="smaller than one tile"):
+        tiny.gather_to_host(big, big.make_batch([[0]]), bk.pinned_empty(8192))
+    with pytest.raises(RuntimeError):
+        bk.HostStager(cuda, chunk_bytes=16, n_buffers=2)
+
+
+def test_measure_d2h_runs(lib, cuda):
+    import bikv_pagecopy as bk
+    print("[case] d2h yardstick", flush=True)
+    dev = torch.arange(0, 1 << 22, dtype=torch.int32, device=cuda).view(torch.uint8)
+    host = bk.pinned_empty(dev.numel())
+    for chunk in (0, 1 << 20):
+        host.zero_()
+        sec = bk.measure_d2h(cuda, host, dev, chunk)
+        assert sec > 0 and torch.equal(host, dev.cpu())
