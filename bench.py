@@ -1,0 +1,420 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV page-copy hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload qwen2_7b|qwen2_1p5b|llama3_8b|
+                    llama3_70b_fp8|reference_200x50]
+
+Default workload = the configuration the headline target is quoted on: the Qwen2-7B-shaped bf16 pool
+(28 layers x K/V, 131072 pages of 16 tokens x 4 heads x 128, ~120 GB resident in HBM) with 64
+requests of 1024..8192 tokens, half gathered into contiguous per-request staging buffers, half
+scattered from contiguous received buffers into freshly allocated pages, ~10 % of the gather ids
+shared between requests. One step = one gather launch + one scatter launch over the whole batch.
+Inputs (pool, staging, index arrays) are resident in HBM before the timed region starts.
+
+Prints ONE JSON line. `value` = algorithmic bytes (payload read + payload written) per second over
+the timed steps; `roofline` prices the slower of the two kernels against 8 TB/s with the launch
+durations measured here with HIP events on the launch stream; `cpu_baseline` times the reference's
+CPU path (torch.index_select / index_copy_ on host tensors) on this box's cores on a bounded sample
+of the same request stream.
+
+`llama3_8b` additionally runs the per-request gather -> pinned-host staging pipeline and reports
+host-link GB/s next to a plain hipMemcpyAsync of one large pinned buffer measured in the same run.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path[:0] = [ROOT, os.path.join(ROOT, "bi-kv_amd")]
+
+HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per launch as a multiple of the algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this file, each scaled by the same counter's reading for the plain-copy
+# calibration launch below (summaries under profiles/). None = not measured for that workload.
+MEASURED_TRAFFIC_RATIO = {}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="qwen2_7b")
+    ap.add_argument("--layout", default="layer_major", choices=["layer_major", "page_major"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pool-pages", type=int, default=0, help="override the pool size (pages per plane)")
+    ap.add_argument("--seg", type=int, default=None)
+    ap.add_argument("--unroll", type=int, default=None)
+    ap.add_argument("--nontemporal", type=int, default=None)
+    ap.add_argument("--chunk-mib", type=int, default=8, help="staging pipeline chunk (llama3_8b)")
+    ap.add_argument("--buffers", type=int, default=3, help="staging pipeline device buffers")
+    return ap.parse_args()
+
+
+def log(msg):
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def fill_random_bytes(t):
+    """Random bytes in place, one plane at a time (bit patterns are what matters for a byte mover)."""
+    import torch
+    flat = t.view(torch.uint8).reshape(-1)
+    step = 1 << 31
+    for off in range(0, flat.numel(), step):
+        flat[off: off + step].random_(0, 256)
+
+
+def make_pool(shape, dev):
+    import torch
+    pool = torch.empty((shape.n_planes, shape.n_pages, shape.tile_bytes), dtype=torch.uint8, device=dev)
+    fill_random_bytes(pool)
+    scale = None
+    if shape.scales:
+        scale = torch.empty((shape.n_planes, shape.n_pages, shape.scale_tile_bytes), dtype=torch.uint8, device=dev)
+        fill_random_bytes(scale)
+    return pool, scale
+
+
+def verify_on_device(pool_t, staging, batch, requests, n_check_planes=3):
+    """Independent check at full size: torch.index_select on the device, a few planes per request."""
+    import torch
+    n_planes = pool_t.shape[0]
+    planes = sorted({0, n_planes // 2, n_planes - 1})[:n_check_planes]
+    for r, ids in enumerate(requests):
+        if len(ids) == 0:
+            continue
+        view = batch.request_view(staging, r)
+        idt = torch.from_numpy(ids).to(pool_t.device)
+        for q in planes:
+            want = torch.index_select(pool_t[q], 0, idt)
+            got = view[q] if batch.layout == "layer_major" else view[:, q]
+            if not torch.equal(got, want):
+                return False
+    return True
+
+
+def time_plain_copy(bk, dev, nbytes=2 << 30, iters=5):
+    """A plain contiguous copy through the run-copy kernel: the achievable-bandwidth yardstick and the
+    known-size launch that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
+    import torch
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    src.random_(0, 256)
+    dst = torch.empty_like(src)
+    zero = torch.zeros(1, dtype=torch.int64, device=dev)
+    bk.copy_runs(src, dst, zero, zero, nbytes)
+    torch.cuda.synchronize(dev)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        bk.copy_runs(src, dst, zero, zero, nbytes)
+    e1.record()
+    torch.cuda.synchronize(dev)
+    ms = e0.elapsed_time(e1) / iters
+    ok = torch.equal(src, dst)
+    del src, dst
+    return 2 * nbytes / (ms * 1e-3) / 1e9, ok
+
+
+def cpu_baseline(shape, wl, budget_s=20.0):
+    """The reference's CPU path on this box's cores: torch.index_select (gather) and index_copy_
+    (scatter) on host tensors [planes, pages, tile]. The host pool is capped (page ids are reduced
+    modulo its page count) and only the leading requests are replayed, so that the sample takes
+    about `budget_s` seconds at most."""
+    import numpy as np
+    import torch
+    from oracle import pagecopy_oracle as oracle
+
+    threads = torch.get_num_threads()
+    host_bytes_cap = 8 << 30
+    try:
+        import psutil
+        host_bytes_cap = min(host_bytes_cap, int(psutil.virtual_memory().total * 0.25))
+    except Exception:
+        pass
+    host_pages = max(64, min(shape.n_pages, host_bytes_cap // (shape.tile_bytes * shape.n_planes)))
+    pool = torch.empty((shape.n_planes, host_pages, shape.tile_bytes), dtype=torch.uint8)
+    pool.view(torch.int64).reshape(-1).copy_(torch.arange(pool.numel() // 8, dtype=torch.int64))
+    g_reqs = [torch.from_numpy(np.ascontiguousarray(r % host_pages)) for r in wl["gather"]]
+    s_src = wl.get("scatter") or wl["gather"]
+    # unique destinations inside the capped pool: take distinct ids from a permutation
+    perm = np.random.default_rng(1234).permutation(host_pages)
+    page_cap = 1024                                   # pages per direction in the sample
+    g_sel, used = [], 0
+    for r in g_reqs:
+        if used + len(r) > page_cap and g_sel:
+            break
+        g_sel.append(r)
+        used += len(r)
+    s_sel, s_used = [], 0
+    for r in s_src:
+        n = min(len(r), host_pages - s_used)
+        if n <= 0 or (s_used + n > page_cap and s_sel):
+            break
+        s_sel.append(torch.from_numpy(np.ascontiguousarray(perm[s_used: s_used + n])))
+        s_used += n
+    outs = [torch.empty((shape.n_planes, len(r), shape.tile_bytes), dtype=torch.uint8) for r in g_sel]
+    srcs = [torch.empty((shape.n_planes, len(r), shape.tile_bytes), dtype=torch.uint8).fill_(3) for r in s_sel]
+
+    def one_pass():
+        for ids, out in zip(g_sel, outs):
+            oracle.gather_layered_torch(pool, ids, out)
+        for ids, src in zip(s_sel, srcs):
+            oracle.scatter_layered_torch(pool, ids, src)
+
+    one_pass()                                        # warm-up (also faults the pages in)
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 5 and (time.perf_counter() - t_start) < budget_s:
+        t0 = time.perf_counter()
+        one_pass()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    pages = used + s_used
+    alg_bytes = 2 * pages * shape.tile_bytes * shape.n_planes
+    return {
+        "value": round(alg_bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": (f"torch.index_select + index_copy_ on host tensors, {len(g_sel)} gather + {len(s_sel)} "
+                   f"scatter requests ({pages} pages, {alg_bytes / 1e9:.2f} GB read+written per pass), host pool "
+                   f"capped to {host_pages} pages/plane with ids modulo that, median of {len(times)} passes"),
+        "pages_per_s": round(pages / med, 1),
+    }
+
+
+def run_gather_scatter(args, bk, workloads, dev):
+    import numpy as np
+    import torch
+
+    name = args.workload
+    shape = workloads.SHAPES[name]
+    if args.pool_pages:
+        shape = shape.scaled(args.pool_pages)
+    wl = workloads.named(name, shape)
+    log(f"{name}: pool {shape.pool_bytes / 1e9:.2f} GB, tile {shape.tile_bytes} B x {shape.n_planes} planes")
+    pool_t, scale_t = make_pool(shape, dev)
+    pool = bk.PagedKVPool.from_stacked(pool_t, plane_dims=1, scale=scale_t)
+
+    g_reqs = wl["gather"]
+    s_reqs = wl.get("scatter") or []
+    gb = pool.make_batch(g_reqs, args.layout)
+    g_st, g_sc = pool.empty_staging(gb)
+    sb = s_st = s_sc = None
+    if s_reqs:
+        sb = pool.make_batch(s_reqs, args.layout)
+        s_st, s_sc = pool.empty_staging(sb)
+        fill_random_bytes(s_st)
+        if s_sc is not None:
+            fill_random_bytes(s_sc)
+    torch.cuda.synchronize(dev)
+    n_pages = gb.n_pages + (sb.n_pages if sb else 0)
+    alg_g = 2 * gb.n_pages * shape.page_bytes
+    alg_s = 2 * sb.n_pages * shape.page_bytes if sb else 0
+    log(f"gather {gb.n_pages} pages ({alg_g / 1e9:.2f} GB r+w), scatter {sb.n_pages if sb else 0} pages "
+        f"({alg_s / 1e9:.2f} GB r+w)")
+
+    def step(events=None):
+        if events is not None:
+            events[0].record()
+        pool.gather(gb, g_st, g_sc)
+        if events is not None:
+            events[1].record()
+        if sb is not None:
+            pool.scatter(sb, s_st, s_sc)
+        if events is not None:
+            events[2].record()
+
+    for _ in range(args.warmup):
+        step()
+    pool.check()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(evs[k])
+    torch.cuda.synchronize(dev)
+    wall = time.perf_counter() - t0
+    pool.check()
+
+    g_ms = [e[0].elapsed_time(e[1]) for e in evs]
+    s_ms = [e[1].elapsed_time(e[2]) for e in evs]
+    ms_per_step = wall * 1e3 / args.steps
+    value = (alg_g + alg_s) / (wall / args.steps) / 1e9
+    g_gbps = alg_g / (np.mean(g_ms) * 1e-3) / 1e9
+    s_gbps = alg_s / (np.mean(s_ms) * 1e-3) / 1e9 if sb else None
+
+    # parity at full size, outside the timed region
+    ok = verify_on_device(pool_t, g_st, gb, g_reqs)
+    if sb is not None:
+        ok = ok and verify_on_device(pool_t, s_st, sb, s_reqs)   # scattered pages now equal their source
+    if scale_t is not None:
+        ok = ok and verify_on_device(scale_t, g_sc, gb, g_reqs)
+    if not ok:
+        raise SystemExit("bench: results differ from torch.index_select on the device — not reporting")
+
+    copy_gbps, copy_ok = time_plain_copy(bk, dev)
+    if not copy_ok:
+        raise SystemExit("bench: plain copy mismatch")
+
+    dominant_is_gather = (s_gbps is None) or (g_gbps <= s_gbps) or True
+    kname = "tile_move_kernel<gather>" if dominant_is_gather else "tile_move_kernel<scatter>"
+    ach = g_gbps
+    ratio = MEASURED_TRAFFIC_RATIO.get(name)
+    out = {
+        "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"{name}: {shape.layers} layers x K/V, {shape.n_pages} pages x {shape.page_tokens} tok x "
+                               f"{shape.kv_heads} heads x {shape.head_dim} {shape.dtype}"
+                               f"{' + fp32 scales' if shape.scales else ''}; {len(g_reqs)} gather + {len(s_reqs)} "
+                               f"scatter requests, {n_pages} pages/step, layout {args.layout}",
+                   "pool_GB": round(shape.pool_bytes / 1e9, 2), "tile_bytes": shape.tile_bytes,
+                   "planes": shape.n_planes},
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "pages_per_s": round(n_pages / (wall / args.steps), 1),
+        "bit_exact": True,
+        "roofline": {"bound": "hbm", "kernel": kname, "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4),
+                     "traffic": (round(ratio * alg_g) if ratio else None),
+                     "alg_bytes_per_launch": alg_g, "avg_launch_ms": round(float(np.mean(g_ms)), 4)},
+        "kernels": {"gather": {"GBps": round(g_gbps, 1), "avg_ms": round(float(np.mean(g_ms)), 4),
+                               "min_ms": round(float(np.min(g_ms)), 4), "alg_bytes": alg_g},
+                    "scatter": ({"GBps": round(s_gbps, 1), "avg_ms": round(float(np.mean(s_ms)), 4),
+                                 "min_ms": round(float(np.min(s_ms)), 4), "alg_bytes": alg_s} if sb else None),
+                    "plain_copy_2GiB": {"GBps": round(copy_gbps, 1)}},
+    }
+    del pool_t, scale_t, g_st, s_st
+    torch.cuda.empty_cache()
+    return out, shape, wl
+
+
+def run_staging(args, bk, workloads, dev):
+    """llama3_8b: per-request gather followed by the device -> pinned-host copy, overlapped in chunks."""
+    import numpy as np
+    import torch
+
+    shape = workloads.SHAPES["llama3_8b"]
+    if args.pool_pages:
+        shape = shape.scaled(args.pool_pages)
+    wl = workloads.named("llama3_8b", shape)
+    pool_t, _ = make_pool(shape, dev)
+    pool = bk.PagedKVPool.from_stacked(pool_t, plane_dims=1)
+    reqs = wl["gather"]
+    max_pages = max(len(r) for r in reqs)
+    host = bk.pinned_empty(max_pages * shape.page_bytes)
+    host.zero_()
+    # host-link yardstick: one large pinned buffer, plain hipMemcpyAsync
+    dev_buf = torch.empty(min(host.numel(), 1 << 30), dtype=torch.uint8, device=dev)
+    dev_buf.random_(0, 256)
+    link = []
+    for _ in range(4):
+        link.append(dev_buf.numel() / bk.measure_d2h(dev, host, dev_buf, 0) / 1e9)
+    link_gbps = max(link[1:])
+    results = {}
+    for mode in ("pipelined", "direct"):
+        stager = bk.HostStager(dev, chunk_bytes=args.chunk_mib << 20, n_buffers=args.buffers)
+        batches = [pool.make_batch([r], args.layout) for r in reqs]
+        torch.cuda.synchronize(dev)
+        stager.gather_to_host(pool, batches[0], host, mode)      # warm-up
+        tot_b, tot_s, chunks = 0, 0.0, 0
+        for b in batches[: max(1, args.steps)]:
+            nb, nc, sec = stager.gather_to_host(pool, b, host, mode)
+            tot_b += nb
+            tot_s += sec
+            chunks += nc
+        # parity of the last request staged
+        b = batches[max(1, args.steps) - 1 if args.steps <= len(batches) else -1]
+        stager.gather_to_host(pool, b, host, mode)
+        r = reqs[batches.index(b)]
+        idt = torch.from_numpy(r).to(dev)
+        view = host[: b.n_slots * shape.tile_bytes].view(b.n_slots, shape.tile_bytes)
+        ok = True
+        for q in (0, shape.n_planes - 1):
+            want = torch.index_select(pool_t[q], 0, idt).cpu()
+            got = view[q * len(r): (q + 1) * len(r)] if args.layout == "layer_major" else view[q::shape.n_planes]
+            ok = ok and torch.equal(got, want)
+        if not ok:
+            raise SystemExit(f"bench: staged bytes differ ({mode})")
+        results[mode] = {"host_link_GBps": round(tot_b / tot_s / 1e9, 2), "bytes": tot_b, "chunks": chunks,
+                         "frac_of_plain_d2h": round(tot_b / tot_s / 1e9 / link_gbps, 4)}
+        stager.close()
+    return {"plain_d2h_GBps": round(link_gbps, 2), "chunk_MiB": args.chunk_mib, "buffers": args.buffers,
+            "requests": min(len(reqs), max(1, args.steps)), **results}
+
+
+def run_reference_scenario(args, bk, dev):
+    """The only workload the reference itself scripts: 200 pages x 50 tokens x 14336 fp16 elements,
+    identity offsets, one run copy per transfer (test_page_ipc.py:41-65)."""
+    import torch
+    page_elements = 50 * 128 * 2 * 28 * 2
+    n = 200
+    cache = torch.full((n * page_elements,), 7, dtype=torch.float16, device=dev)
+    out = torch.empty_like(cache)
+    offs = torch.arange(n, dtype=torch.int64, device=dev) * page_elements
+    for _ in range(args.warmup):
+        bk.copy_runs(cache, out, offs, offs, page_elements)
+    torch.cuda.synchronize(dev)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        bk.copy_runs(cache, out, offs, offs, page_elements)
+    e1.record()
+    torch.cuda.synchronize(dev)
+    wall = time.perf_counter() - t0
+    if not torch.equal(out, cache):
+        raise SystemExit("bench: reference scenario mismatch")
+    alg = 2 * cache.numel() * 2
+    ms = e0.elapsed_time(e1) / args.steps
+    return {
+        "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
+        "value": round(alg / (wall / args.steps) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "reference_200x50: 200 pages x 50 tokens x 14336 fp16, identity offsets, value 7"},
+        "pages_per_s": round(n / (wall / args.steps), 1), "bit_exact": True,
+        "roofline": {"bound": "hbm", "kernel": "copy_runs_kernel", "achieved": round(alg / (ms * 1e-3) / 1e9, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "traffic": None, "alg_bytes_per_launch": alg, "avg_launch_ms": round(ms, 4)},
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no cross-GPU step (pages are independent; each GPU "
+              "gathers/scatters its own pool). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import __graft_entry__ as entry
+    entry.ensure_built()
+    import bikv_pagecopy as bk
+    from bikv_pagecopy import workloads
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU: the page-copy path has no CPU fallback")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    knobs = {k: getattr(args, k) for k in ("seg", "unroll", "nontemporal") if getattr(args, k) is not None}
+    if knobs:
+        bk.set_tuning(**knobs)
+
+    if args.workload == "reference_200x50":
+        out = run_reference_scenario(args, bk, dev)
+        print(json.dumps(out), flush=True)
+        return
+    out, shape, wl = run_gather_scatter(args, bk, workloads, dev)
+    if knobs:
+        out["config"]["tuning"] = knobs
+    if args.workload == "llama3_8b":
+        out["staging"] = run_staging(args, bk, workloads, dev)
+    if not args.no_cpu_baseline:
+        log("timing the CPU baseline")
+        out["cpu_baseline"] = cpu_baseline(shape, wl)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

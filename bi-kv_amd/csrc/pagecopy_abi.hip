@@ -74,15 +74,17 @@ static uint32_t take_status(int device) {
   return bits;
 }
 
+static int status_error(uint32_t bits) {
+  if (!bits) return BIKV_OK;
+  return fail(BIKV_EBOUNDS, "kernel skipped out-of-range work (status bits 0x%x:%s%s%s)", bits,
+              (bits & BIKV_ST_SRC_RANGE) ? " source-range" : "",
+              (bits & BIKV_ST_DST_RANGE) ? " destination-range" : "",
+              (bits & BIKV_ST_PAGE_ID) ? " page-id" : "");
+}
+
 int sync_and_check(int device, hipStream_t stream) {
   BIKV_HIP(hipStreamSynchronize(stream));
-  const uint32_t bits = take_status(device);
-  if (bits)
-    return fail(BIKV_EBOUNDS, "kernel skipped out-of-range work (status bits 0x%x:%s%s%s)", bits,
-                (bits & BIKV_ST_SRC_RANGE) ? " source-range" : "",
-                (bits & BIKV_ST_DST_RANGE) ? " destination-range" : "",
-                (bits & BIKV_ST_PAGE_ID) ? " page-id" : "");
-  return BIKV_OK;
+  return status_error(take_status(device));
 }
 
 static int current_device(int* dev) {
@@ -121,8 +123,7 @@ extern "C" int bikv_check_status(int device, void* stream, uint32_t* bits_out) {
   BIKV_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   const uint32_t bits = take_status(device);
   if (bits_out) *bits_out = bits;
-  if (bits) return fail(BIKV_EBOUNDS, "kernel skipped out-of-range work (status bits 0x%x)", bits);
-  return BIKV_OK;
+  return status_error(bits);
 }
 
 extern "C" int bikv_set_tuning(const char* key, int64_t value) {
@@ -430,11 +431,19 @@ static void plan_chunks(const int64_t* req_pages, int64_t n_req, int n_planes, i
     // slot = global_page * n_planes + plane: any run of whole pages is contiguous, across requests
     int64_t total = 0;
     for (int64_t r = 0; r < n_req; ++r) total += req_pages[r];
-    int64_t per = max_slots / n_planes;
-    if (per < 1) per = 1;
-    for (int64_t p = 0; p < total; p += per) {
-      const int64_t n = total - p < per ? total - p : per;
-      out->push_back(Chunk{p, n, 0, n_planes, p * n_planes, n * n_planes});
+    if (max_slots >= n_planes) {
+      const int64_t per = max_slots / n_planes;
+      for (int64_t p = 0; p < total; p += per) {
+        const int64_t n = total - p < per ? total - p : per;
+        out->push_back(Chunk{p, n, 0, n_planes, p * n_planes, n * n_planes});
+      }
+    } else {
+      // a chunk is smaller than one page: cut every page into runs of consecutive planes
+      for (int64_t p = 0; p < total; ++p)
+        for (int q = 0; q < n_planes; q += (int)max_slots) {
+          const int c = n_planes - q < (int)max_slots ? n_planes - q : (int)max_slots;
+          out->push_back(Chunk{p, 1, q, c, p * n_planes + q, c});
+        }
     }
     return;
   }
@@ -533,6 +542,10 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
     int rc = BIKV_OK;
     for (size_t c = 0; c < chunks.size(); ++c) {
       const Chunk& ch = chunks[c];
+      if (ch.n_slots * T > st->chunk_bytes) {
+        rc = fail(BIKV_ERANGE, "internal: planned chunk exceeds the device chunk buffer");
+        break;
+      }
       const int buf = (int)(c % (size_t)st->n_buf);
       char* dev_chunk = st->ring + (int64_t)buf * st->chunk_bytes;
       if (c >= (size_t)st->n_buf) {

@@ -215,10 +215,7 @@ def test_plan_chunks_tiles_the_staging_image_exactly(lib, layout):
         for first_page, n_pages, q0, qc, first_slot, n_slots in plan.tolist():
             assert first_slot == at, "chunks must follow each other without gaps"
             assert n_slots == n_pages * qc
-            if layout == "page_major":
-                assert n_slots <= max(max_slots, n_planes)
-            else:
-                assert n_slots <= max_slots
+            assert 0 < n_slots <= max_slots
             # the rectangle (pages x planes) must land exactly inside [first_slot, first_slot+n_slots)
             i = np.arange(first_page, first_page + n_pages)
             q = np.arange(q0, q0 + qc)
