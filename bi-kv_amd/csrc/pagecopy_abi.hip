@@ -136,8 +136,12 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
     if (value != 1 && value != 2 && value != 4 && value != 8)
       return fail(BIKV_EINVAL, "unroll must be 1, 2, 4 or 8");
     t.unroll = (int)value;
+  } else if (!strcmp(key, "wave_block")) {
+    if (value != 64 && value != 128 && value != 256)
+      return fail(BIKV_EINVAL, "wave_block must be 64, 128 or 256");
+    t.wave_block = (int)value;
   } else if (!strcmp(key, "nontemporal")) {
-    t.nontemporal = value ? 1 : 0;
+    t.nontemporal = value < 0 ? -1 : (value ? 1 : 0);
   } else if (!strcmp(key, "run_chunk_kib")) {
     if (value < 0 || value > 1 << 20) return fail(BIKV_EINVAL, "run_chunk_kib out of range");
     t.run_chunk_kib = (int)value;

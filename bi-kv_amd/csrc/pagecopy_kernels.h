@@ -39,9 +39,11 @@ struct MoveArgs {
 };
 
 struct Tuning {
-  int seg = 0;          // 0 = choose from the batch shape
+  int seg = 0;          // 0 = wave mover when the shape qualifies, else segment movers with an
+                        // automatic segment; > 0 = segment movers with this many pages per workgroup
+  int wave_block = 64;  // lanes per workgroup of the wave mover (64, 128 or 256)
   int unroll = 4;       // 16-byte vectors in flight per lane (1, 2, 4 or 8)
-  int nontemporal = 1;  // 1 = nt hint on the streaming loads and stores
+  int nontemporal = -1; // nt hint on payload loads and stores: 1 on, 0 off, -1 gathers only
   int run_chunk_kib = 0;  // bytes of a run handled by one workgroup, KiB; 0 = choose
 };
 Tuning& tuning();

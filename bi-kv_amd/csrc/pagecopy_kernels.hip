@@ -205,13 +205,140 @@ static hipError_t launch_dir(const MoveArgs& a, bool rows, uint32_t grid, hipStr
     hipLaunchKernelGGL((tile_move_kernel<DIR, 1, false, false>), dim3(grid), dim3(kBlock), 0, s, a);
     return hipGetLastError();
   }
-  const bool nt = tuning().nontemporal != 0;
+  const bool nt = tuning().nontemporal > 0 || (tuning().nontemporal < 0 && DIR == 0);
   switch (tuning().unroll) {
     case 1: return nt ? launch_rows<DIR, 1, true>(a, grid, s) : launch_rows<DIR, 1, false>(a, grid, s);
     case 2: return nt ? launch_rows<DIR, 2, true>(a, grid, s) : launch_rows<DIR, 2, false>(a, grid, s);
     case 8: return nt ? launch_rows<DIR, 8, true>(a, grid, s) : launch_rows<DIR, 8, false>(a, grid, s);
     default: return nt ? launch_rows<DIR, 4, true>(a, grid, s) : launch_rows<DIR, 4, false>(a, grid, s);
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Wave mover: the layout that measures fastest on MI355X for a pure copy — one 16-byte load and one
+// 16-byte store per lane, one small workgroup (64 lanes = 1 KiB by default) per piece of a tile,
+// millions of independent workgroups. Nothing is unrolled: with a single vector per lane the store
+// of a wave follows its load immediately, reads and writes stay finely interleaved at the memory
+// controllers, and the occupancy of the many tiny waves hides the latency.
+//
+// Grid: x = (batch page, piece of the tile), y = plane. The descriptor of a workgroup (page id,
+// slot, slot stride, plane base) depends only on blockIdx, so it is fetched with scalar loads
+// through the constant address space: the scalar cache does the broadcast that the LDS does in the
+// segment movers above, without a barrier. Consecutive workgroups walk the pieces of one tile, then
+// the next page of the same plane, so each plane's staging range is written front to back.
+//
+// Workgroups with blockIdx.x >= payload.n_blocks move the scale class (tiny tiles): one lane per
+// vector, each lane fetching the descriptor of its own tile.
+// ---------------------------------------------------------------------------------------------
+#define BIKV_CONST __attribute__((address_space(4)))
+
+template <class T>
+__device__ __forceinline__ T cload(const T* p) {
+  return *(const BIKV_CONST T*)(uint64_t)p;
+}
+
+template <int DIR, int VW>
+__device__ __forceinline__ void move_one(uint64_t pool, uint64_t stg) {
+  using T = typename VecOf<VW>::T;
+  st<false, T>(DIR == 0 ? stg : pool, ld<false, T>(DIR == 0 ? pool : stg));
+}
+
+template <int DIR, bool NT, int B>
+__global__ __launch_bounds__(B) void tile_move_wave_kernel(const MoveArgs a) {
+  const uint32_t bx = blockIdx.x;
+  const int64_t q = a.plane_begin + (int64_t)blockIdx.y;
+  if (bx < a.payload.n_blocks) {
+    const uint32_t lp = (uint32_t)a.payload.log2_rows;
+    const uint32_t i = bx >> lp;
+    const uint32_t part = bx & ((1u << lp) - 1u);
+    const int64_t pid = cload(a.page_ids + i);
+    const int64_t slot = cload(a.slots + i) + q * cload(a.slot_strides + i) - a.slot_bias;
+    const uint64_t plane = (uint64_t)cload(a.payload.plane_base + q);  // issued with the others
+    const bool bad_page = (uint64_t)pid >= (uint64_t)a.n_pool_pages;
+    const bool bad_slot = (uint64_t)slot >= (uint64_t)a.payload.n_slots;
+    if (bad_page || bad_slot) {
+      if (threadIdx.x == 0 && part == 0) {
+        if (bad_page) raise(a.status, ST_SLOT_PAGE);
+        if (bad_slot) raise(a.status, DIR == 0 ? ST_SLOT_DST : ST_SLOT_SRC);
+      }
+      return;
+    }
+    const uint64_t pool = plane + (uint64_t)(pid * a.payload.page_stride);
+    const uint64_t stg = (uint64_t)a.payload.staging + (uint64_t)(slot * a.payload.tile_bytes);
+    const uint64_t off = (uint64_t)part * (B * 16u) + threadIdx.x * 16u;
+    st<NT, u32x4>((DIR == 0 ? stg : pool) + off, ld<NT, u32x4>((DIR == 0 ? pool : stg) + off));
+  } else {
+    const uint32_t vpt = a.scale.segs_per_plane;  // vectors per scale tile (wave mover's meaning)
+    // the launcher keeps (scale workgroups * B) below 2^32, so 32-bit arithmetic is exact here
+    const uint32_t v = (bx - a.payload.n_blocks) * (uint32_t)B + threadIdx.x;
+    if ((uint64_t)v >= (uint64_t)a.n_batch * vpt) return;
+    const uint32_t i = v / vpt;
+    const uint32_t w = v - i * vpt;
+    const int64_t pid = a.page_ids[i];
+    const int64_t slot = a.slots[i] + q * a.slot_strides[i] - a.slot_bias;
+    const bool bad_page = (uint64_t)pid >= (uint64_t)a.n_pool_pages;
+    const bool bad_slot = (uint64_t)slot >= (uint64_t)a.scale.n_slots;
+    if (bad_page) raise(a.status, ST_SLOT_PAGE);
+    if (bad_slot) raise(a.status, DIR == 0 ? ST_SLOT_DST : ST_SLOT_SRC);
+    if (bad_page || bad_slot) return;
+    const uint64_t off = (uint64_t)w * (uint64_t)a.scale.vec_width;
+    const uint64_t pool = (uint64_t)a.scale.plane_base[q] + (uint64_t)(pid * a.scale.page_stride) + off;
+    const uint64_t stg = (uint64_t)a.scale.staging + (uint64_t)(slot * a.scale.tile_bytes) + off;
+    switch (a.scale.vec_width) {
+      case 16: move_one<DIR, 16>(pool, stg); break;
+      case 8: move_one<DIR, 8>(pool, stg); break;
+      case 4: move_one<DIR, 4>(pool, stg); break;
+      case 2: move_one<DIR, 2>(pool, stg); break;
+      default: move_one<DIR, 1>(pool, stg); break;
+    }
+  }
+}
+
+template <int DIR, int B>
+static hipError_t launch_wave_b(const MoveArgs& a, dim3 grid, hipStream_t s) {
+  // measured on MI355X: the nt hint lifts a gather (random reads, dense writes) by ~15 % and costs a
+  // scatter (dense reads, random writes) ~3 %, so "auto" (-1) turns it on for gathers only
+  const int nt = tuning().nontemporal;
+  if (nt > 0 || (nt < 0 && DIR == 0))
+    hipLaunchKernelGGL((tile_move_wave_kernel<DIR, true, B>), grid, dim3(B), 0, s, a);
+  else
+    hipLaunchKernelGGL((tile_move_wave_kernel<DIR, false, B>), grid, dim3(B), 0, s, a);
+  return hipGetLastError();
+}
+
+template <int DIR>
+static hipError_t launch_wave(const MoveArgs& a, int block, dim3 grid, hipStream_t s) {
+  switch (block) {
+    case 128: return launch_wave_b<DIR, 128>(a, grid, s);
+    case 256: return launch_wave_b<DIR, 256>(a, grid, s);
+    default: return launch_wave_b<DIR, 64>(a, grid, s);
+  }
+}
+
+// The wave mover takes a payload whose tiles are 2^k pieces of block*16 bytes, all 16-byte aligned.
+// Returns false when the shape does not qualify (the segment movers take it then).
+static bool plan_wave(MoveArgs& a, int block, dim3* grid) {
+  const int64_t piece = (int64_t)block * 16;
+  TileClass& p = a.payload;
+  if (p.vec_width != 16 || p.tile_bytes % piece != 0) return false;
+  const int64_t parts = p.tile_bytes / piece;
+  if ((parts & (parts - 1)) != 0) return false;
+  int lp = 0;
+  while ((int64_t(1) << lp) < parts) ++lp;
+  const int64_t px = a.n_batch << lp;
+  int64_t sx = 0;
+  if (a.scale.tile_bytes > 0) {
+    const int64_t vpt = a.scale.tile_bytes / a.scale.vec_width;
+    if (vpt >= (int64_t(1) << 31)) return false;
+    a.scale.segs_per_plane = (uint32_t)vpt;
+    sx = (a.n_batch * vpt + block - 1) / block;
+  }
+  if (px + sx >= (int64_t(1) << 31) / block * 2 || a.plane_count > 65535) return false;
+  p.log2_rows = lp;
+  p.n_blocks = (uint32_t)px;
+  a.scale.n_blocks = (uint32_t)sx;
+  *grid = dim3((uint32_t)(px + sx), (uint32_t)a.plane_count, 1);
+  return true;
 }
 
 // Picks the number of batch pages per workgroup: enough bytes per workgroup to amortise the
@@ -252,6 +379,13 @@ static bool finish_class(TileClass& c, int forced_seg, int64_t n_batch, int plan
 
 hipError_t launch_tile_move(int dir, MoveArgs& a, hipStream_t stream) {
   if (a.n_batch <= 0 || a.plane_count <= 0) return hipSuccess;
+  if (tuning().seg == 0) {
+    // default: the wave mover, whenever the payload shape qualifies
+    dim3 grid;
+    if (plan_wave(a, tuning().wave_block, &grid))
+      return dir == 0 ? launch_wave<0>(a, tuning().wave_block, grid, stream)
+                      : launch_wave<1>(a, tuning().wave_block, grid, stream);
+  }
   if (!finish_class(a.payload, tuning().seg, a.n_batch, a.plane_count)) return hipErrorInvalidValue;
   // scale tiles are tiny: pack as many pages per workgroup as LDS descriptors allow
   if (a.scale.tile_bytes > 0) {
@@ -378,8 +512,78 @@ __global__ __launch_bounds__(kBlock) void copy_small_runs_kernel(const RunArgs a
   }
 }
 
+// Moves up to 16 bytes between two addresses of any alignment with the widest accesses both allow.
+__device__ __forceinline__ void move_upto16(uint64_t s, uint64_t d, int n) {
+  const uint64_t al = s | d;
+  int done = 0;
+  if ((al & 7) == 0) {
+    for (; done + 8 <= n; done += 8) st<false, u32x2>(d + done, ld<false, u32x2>(s + done));
+  } else if ((al & 3) == 0) {
+    for (; done + 4 <= n; done += 4) st<false, uint32_t>(d + done, ld<false, uint32_t>(s + done));
+  } else if ((al & 1) == 0) {
+    for (; done + 2 <= n; done += 2) st<false, uint16_t>(d + done, ld<false, uint16_t>(s + done));
+  }
+  for (; done < n; ++done) st<false, uint8_t>(d + done, ld<false, uint8_t>(s + done));
+}
+
+// Large runs, wave style (same shape as the wave mover above): grid x = 1 KiB piece of the run,
+// (y, z) = run; one 16-byte vector per lane; the run's two offsets come in through scalar loads.
+// A run whose addresses are not 16-byte aligned, and the ragged end of a run, fall back to narrower
+// accesses lane by lane.
+template <bool NT, int B>
+__global__ __launch_bounds__(B) void copy_runs_wave_kernel(const RunArgs a) {
+  const uint64_t run = (uint64_t)blockIdx.y + (uint64_t)blockIdx.z * gridDim.y;
+  if (run >= (uint64_t)a.n_runs) return;
+  const int64_t so_u = cload(a.src_off + run);
+  const int64_t do_u = cload(a.dst_off + run);
+  const int64_t so = so_u * a.unit_bytes;
+  const int64_t dof = do_u * a.unit_bytes;
+  const bool bad_src = so_u < 0 || so < 0 || so > a.src_bytes - a.run_bytes;
+  const bool bad_dst = do_u < 0 || dof < 0 || dof > a.dst_bytes - a.run_bytes;
+  if (bad_src || bad_dst) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+      if (bad_src) raise(a.status, ST_SLOT_SRC);
+      if (bad_dst) raise(a.status, ST_SLOT_DST);
+    }
+    return;
+  }
+  const int64_t lo = (int64_t)blockIdx.x * (B * 16) + threadIdx.x * 16;
+  if (lo >= a.run_bytes) return;
+  const uint64_t s = (uint64_t)(a.src + so + lo);
+  const uint64_t d = (uint64_t)(a.dst + dof + lo);
+  const int64_t left = a.run_bytes - lo;
+  if (left >= 16 && ((s | d) & 15) == 0) {
+    st<NT, u32x4>(d, ld<NT, u32x4>(s));
+  } else {
+    move_upto16(s, d, left < 16 ? (int)left : 16);
+  }
+}
+
+template <int B>
+static hipError_t launch_runs_wave(const RunArgs& a, hipStream_t stream) {
+  const int64_t piece = (int64_t)B * 16;
+  const int64_t gx = (a.run_bytes + piece - 1) / piece;
+  if (gx >= (int64_t(1) << 32) / B) return hipErrorInvalidValue;
+  const int64_t gy = a.n_runs < 32768 ? a.n_runs : 32768;
+  const int64_t gz = (a.n_runs + gy - 1) / gy;
+  if (gz > 65535) return hipErrorInvalidValue;
+  const dim3 grid((uint32_t)gx, (uint32_t)gy, (uint32_t)gz);
+  if (tuning().nontemporal != 0)
+    hipLaunchKernelGGL((copy_runs_wave_kernel<true, B>), grid, dim3(B), 0, stream, a);
+  else
+    hipLaunchKernelGGL((copy_runs_wave_kernel<false, B>), grid, dim3(B), 0, stream, a);
+  return hipGetLastError();
+}
+
 hipError_t launch_copy_runs(const RunArgs& a, hipStream_t stream) {
   if (a.n_runs <= 0 || a.run_bytes <= 0) return hipSuccess;
+  if (a.run_bytes > 2048 && tuning().run_chunk_kib == 0) {
+    switch (tuning().wave_block) {
+      case 128: return launch_runs_wave<128>(a, stream);
+      case 256: return launch_runs_wave<256>(a, stream);
+      default: return launch_runs_wave<64>(a, stream);
+    }
+  }
   if (a.run_bytes <= 2048) {
     const int64_t ppr = (a.run_bytes + 15) >> 4;
     const int64_t total = ppr * a.n_runs;

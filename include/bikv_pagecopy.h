@@ -54,8 +54,11 @@ const char* bikv_last_error(void);
  * Returns BIKV_OK, or BIKV_EBOUNDS with *bits_out (nullable) holding the BIKV_ST_* bits. */
 int bikv_check_status(int device, void* stream, uint32_t* bits_out);
 
-/* Kernel launch knobs, for measurement. Keys: "seg" (batch pages per workgroup, 0 = automatic),
- * "unroll" (16-byte vectors in flight per lane: 1, 2, 4, 8), "nontemporal" (0/1),
+/* Kernel launch knobs, for measurement. Keys: "seg" (0 = default: the wave mover, one 16-byte
+ * vector per lane, whenever the tile shape qualifies; n > 0 = the LDS-staged segment mover with n
+ * batch pages per workgroup), "wave_block" (lanes per workgroup of the wave mover: 64, 128, 256),
+ * "unroll" (segment mover: 16-byte vectors in flight per lane: 1, 2, 4, 8), "nontemporal" (nt hint on
+ * payload accesses: 1 on, 0 off, -1 = default: gathers and run copies only),
  * "run_chunk_kib" (bytes of a run per workgroup, KiB; 0 = automatic). Process-wide. */
 int bikv_set_tuning(const char* key, int64_t value);
 

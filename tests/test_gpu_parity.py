@@ -297,17 +297,29 @@ def test_tuning_knobs_do_not_change_results(bk, oracle, cuda):
     reqs = [rng.permutation(64)[:37], rng.permutation(64)[:5]]
     want = oracle.gather_layered_c(pool_h, reqs).tobytes()
     batch = pool.make_batch(reqs)
+    sreqs = [rng.permutation(64)[:42]]
+    sbatch = pool.make_batch(sreqs)
+    src = torch.from_numpy(rng.integers(0, 256, size=sbatch.n_slots * 16384, dtype=np.uint8)).to(cuda)
+    want_pool = pool_h.copy()
+    oracle.scatter_layered_c(want_pool, sreqs, src.cpu().numpy())
     try:
-        for seg in (0, 1, 3, 16, 256):
-            for unroll in (1, 2, 4, 8):
-                for nt in (0, 1):
-                    bk.set_tuning(seg=seg, unroll=unroll, nontemporal=nt)
-                    st = torch.zeros(batch.n_slots * 16384, dtype=torch.uint8, device=cuda)
-                    pool.gather(batch, st)
-                    pool.check()
-                    assert _to_np(st).tobytes() == want, (seg, unroll, nt)
+        # seg 0 = wave mover (wave_block lanes per workgroup); seg > 0 = LDS-staged segment mover
+        cases = [dict(seg=0, wave_block=wb, nontemporal=nt) for wb in (64, 128, 256) for nt in (-1, 0, 1)]
+        cases += [dict(seg=seg, unroll=u, nontemporal=nt) for seg in (1, 3, 16, 256) for u in (1, 2, 4, 8)
+                  for nt in (0, 1)]
+        for kw in cases:
+            bk.set_tuning(**kw)
+            st = torch.zeros(batch.n_slots * 16384, dtype=torch.uint8, device=cuda)
+            pool.gather(batch, st)
+            pool.check()
+            assert _to_np(st).tobytes() == want, kw
+            pool_d.copy_(torch.from_numpy(pool_h))
+            pool.scatter(sbatch, src)
+            pool.check()
+            assert _to_np(pool_d).tobytes() == want_pool.tobytes(), kw
+            pool_d.copy_(torch.from_numpy(pool_h))
     finally:
-        bk.set_tuning(seg=0, unroll=4, nontemporal=1)
+        bk.set_tuning(seg=0, wave_block=64, unroll=4, nontemporal=-1)
 
 
 # ---- run copy (reference API) -------------------------------------------------------------------
