@@ -34,7 +34,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch as a multiple of the algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this file, each scaled by the same counter's reading for the plain-copy
 # calibration launch below (summaries under profiles/). None = not measured for that workload.
-MEASURED_TRAFFIC_RATIO = {}
+MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9954, "scatter": 1.0117}}
 
 
 def parse_args():
@@ -50,8 +50,10 @@ def parse_args():
     ap.add_argument("--unroll", type=int, default=None)
     ap.add_argument("--nontemporal", type=int, default=None)
     ap.add_argument("--wave-block", dest="wave_block", type=int, default=None)
+    ap.add_argument("--staging-cap-gb", dest="staging_cap_gb", type=float, default=32.0,
+                    help="largest staging buffer of one launch; bigger batches take several launches")
     ap.add_argument("--chunk-mib", type=int, default=8, help="staging pipeline chunk (llama3_8b)")
-    ap.add_argument("--buffers", type=int, default=3, help="staging pipeline device buffers")
+    ap.add_argument("--buffers", type=int, default=2, help="staging pipeline lanes (stream + HBM chunk each)")
     return ap.parse_args()
 
 
@@ -199,30 +201,56 @@ def run_gather_scatter(args, bk, workloads, dev):
 
     g_reqs = wl["gather"]
     s_reqs = wl.get("scatter") or []
-    gb = pool.make_batch(g_reqs, args.layout)
-    g_st, g_sc = pool.empty_staging(gb)
-    sb = s_st = s_sc = None
-    if s_reqs:
-        sb = pool.make_batch(s_reqs, args.layout)
-        s_st, s_sc = pool.empty_staging(sb)
+
+    # A launch covers as many whole requests as fit a staging buffer of --staging-cap-gb; the
+    # Qwen2-7B-shaped batch fits in one launch per direction, the 70B-shaped one needs a few.
+    def groups_of(reqs):
+        cap_pages = max(1, int(args.staging_cap_gb * 1e9) // shape.page_bytes)
+        out, cur, used = [], [], 0
+        for r in reqs:
+            if cur and used + len(r) > cap_pages:
+                out.append(cur)
+                cur, used = [], 0
+            cur.append(r)
+            used += len(r)
+        if cur:
+            out.append(cur)
+        return [(pool.make_batch(g, args.layout), g) for g in out]
+
+    g_groups, s_groups = groups_of(g_reqs), groups_of(s_reqs)
+    max_slots = max(b.n_slots for b, _ in g_groups + s_groups)
+    g_st = torch.empty(max_slots * shape.tile_bytes, dtype=torch.uint8, device=dev)
+    g_sc = torch.empty(max_slots * shape.scale_tile_bytes, dtype=torch.uint8, device=dev) if shape.scales else None
+    s_st = s_sc = None
+    if s_groups:
+        s_st = torch.empty_like(g_st)
         fill_random_bytes(s_st)
-        if s_sc is not None:
+        if shape.scales:
+            s_sc = torch.empty_like(g_sc)
             fill_random_bytes(s_sc)
+
+    def views(batch, st, sc):
+        return (st[: batch.n_slots * shape.tile_bytes],
+                sc[: batch.n_slots * shape.scale_tile_bytes] if sc is not None else None)
+
     torch.cuda.synchronize(dev)
-    n_pages = gb.n_pages + (sb.n_pages if sb else 0)
-    alg_g = 2 * gb.n_pages * shape.page_bytes
-    alg_s = 2 * sb.n_pages * shape.page_bytes if sb else 0
-    log(f"gather {gb.n_pages} pages ({alg_g / 1e9:.2f} GB r+w), scatter {sb.n_pages if sb else 0} pages "
-        f"({alg_s / 1e9:.2f} GB r+w)")
+    g_pages = sum(b.n_pages for b, _ in g_groups)
+    s_pages = sum(b.n_pages for b, _ in s_groups)
+    n_pages = g_pages + s_pages
+    alg_g = 2 * g_pages * shape.page_bytes
+    alg_s = 2 * s_pages * shape.page_bytes
+    log(f"gather {g_pages} pages in {len(g_groups)} launch(es) ({alg_g / 1e9:.2f} GB r+w), scatter {s_pages} pages in "
+        f"{len(s_groups)} launch(es) ({alg_s / 1e9:.2f} GB r+w)")
 
     def step(events=None):
         if events is not None:
             events[0].record()
-        pool.gather(gb, g_st, g_sc)
+        for b, _ in g_groups:
+            pool.gather(b, *views(b, g_st, g_sc))
         if events is not None:
             events[1].record()
-        if sb is not None:
-            pool.scatter(sb, s_st, s_sc)
+        for b, _ in s_groups:
+            pool.scatter(b, *views(b, s_st, s_sc))
         if events is not None:
             events[2].record()
 
@@ -238,21 +266,35 @@ def run_gather_scatter(args, bk, workloads, dev):
     wall = time.perf_counter() - t0
     pool.check()
 
-    g_ms = [e[0].elapsed_time(e[1]) for e in evs]
-    s_ms = [e[1].elapsed_time(e[2]) for e in evs]
+    # per-launch averages (a direction's launches are back to back between two events)
+    g_ms = [e[0].elapsed_time(e[1]) / len(g_groups) for e in evs]
+    s_ms = [e[1].elapsed_time(e[2]) / max(1, len(s_groups)) for e in evs]
     ms_per_step = wall * 1e3 / args.steps
     value = (alg_g + alg_s) / (wall / args.steps) / 1e9
-    g_gbps = alg_g / (np.mean(g_ms) * 1e-3) / 1e9
-    s_gbps = alg_s / (np.mean(s_ms) * 1e-3) / 1e9 if sb else None
+    g_gbps = alg_g / len(g_groups) / (np.mean(g_ms) * 1e-3) / 1e9
+    s_gbps = alg_s / len(s_groups) / (np.mean(s_ms) * 1e-3) / 1e9 if s_groups else None
+    sb = s_groups or None
 
-    # parity at full size, outside the timed region
-    ok = verify_on_device(pool_t, g_st, gb, g_reqs)
-    if sb is not None:
-        ok = ok and verify_on_device(pool_t, s_st, sb, s_reqs)   # scattered pages now equal their source
-    if scale_t is not None:
-        ok = ok and verify_on_device(scale_t, g_sc, gb, g_reqs)
+    # parity at full size, outside the timed region: scattered pages must equal their source, and
+    # each gather launch is repeated and checked against torch.index_select on the device
+    ok = True
+    for b, reqs in s_groups:
+        st, sc = views(b, s_st, s_sc)
+        ok = ok and verify_on_device(pool_t, st, b, reqs)
+        if scale_t is not None:
+            ok = ok and verify_on_device(scale_t, sc, b, reqs)
+    for b, reqs in g_groups:
+        st, sc = views(b, g_st, g_sc)
+        st.zero_()
+        pool.gather(b, st, sc)
+        pool.check()
+        ok = ok and verify_on_device(pool_t, st, b, reqs)
+        if scale_t is not None:
+            ok = ok and verify_on_device(scale_t, sc, b, reqs)
     if not ok:
         raise SystemExit("bench: results differ from torch.index_select on the device — not reporting")
+    alg_g //= len(g_groups)          # per launch, for the roofline entries below
+    alg_s //= max(1, len(s_groups))
 
     copy_gbps, copy_ok = time_plain_copy(bk, dev)
     if not copy_ok:
@@ -264,7 +306,9 @@ def run_gather_scatter(args, bk, workloads, dev):
     ach = g_gbps if dominant_is_gather else s_gbps
     alg_dom = alg_g if dominant_is_gather else alg_s
     ms_dom = float(np.mean(g_ms if dominant_is_gather else s_ms))
-    ratio = MEASURED_TRAFFIC_RATIO.get(name)
+    ratio = MEASURED_TRAFFIC_RATIO.get(name, {}).get("gather" if dominant_is_gather else "scatter")
+    if args.pool_pages or args.layout != "layer_major":
+        ratio = None                                   # measured on the full-size default workload only
     out = {
         "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -273,7 +317,8 @@ def run_gather_scatter(args, bk, workloads, dev):
         "config": {"workload": f"{name}: {shape.layers} layers x K/V, {shape.n_pages} pages x {shape.page_tokens} tok x "
                                f"{shape.kv_heads} heads x {shape.head_dim} {shape.dtype}"
                                f"{' + fp32 scales' if shape.scales else ''}; {len(g_reqs)} gather + {len(s_reqs)} "
-                               f"scatter requests, {n_pages} pages/step, layout {args.layout}",
+                               f"scatter requests, {n_pages} pages/step in {len(g_groups)}+{len(s_groups)} launches, "
+                               f"layout {args.layout}",
                    "pool_GB": round(shape.pool_bytes / 1e9, 2), "tile_bytes": shape.tile_bytes,
                    "planes": shape.n_planes},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),

@@ -3,9 +3,9 @@
 The reference stages outgoing KV in host tensors allocated per call (Bi-KV/DistributedStorage/
 kvcache.py:105-108, Bi-KV/Worker/Worker.py:203-206) which the RDMA endpoint then sends from a
 pinned region (Bi-KV/NetworkTransport/onesided_rdma.h:301-337). HostStager fills such a pinned
-region straight from the paged pool: chunked gather on one HIP stream overlapped with
-hipMemcpyAsync on another (mode "pipelined"), or kernel stores directly into the mapped pinned
-buffer (mode "direct").
+region straight from the paged pool: chunks are gathered into per-stream HBM buffers and copied out
+with hipMemcpyAsync, several streams in flight (mode "pipelined"), or the gather kernel stores
+directly into the mapped pinned buffer (mode "direct").
 """
 import ctypes as C
 
@@ -24,7 +24,7 @@ def pinned_empty(nbytes: int) -> torch.Tensor:
 
 
 class HostStager:
-    def __init__(self, device, chunk_bytes: int = 8 << 20, n_buffers: int = 3):
+    def __init__(self, device, chunk_bytes: int = 8 << 20, n_buffers: int = 2):
         self.device = torch.device(device)
         self.chunk_bytes = int(chunk_bytes)
         self.n_buffers = int(n_buffers)

@@ -150,8 +150,9 @@ int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* batch,
  *
  * The reference stages KV for the transport in host tensors (kvcache.py:105-108, Worker.py:203-206)
  * that the RDMA endpoint sends from a pinned host region (onesided_rdma.h:301-337). This pipeline
- * fills such a region: the gather runs chunk by chunk into a small ring of device buffers on a
- * compute stream while hipMemcpyAsync drains finished chunks to `host_dst` on a copy stream.
+ * fills such a region chunk by chunk: chunk c is gathered into the HBM buffer of stream c % n_buffers
+ * and copied from there to `host_dst` with hipMemcpyAsync on the same stream, so that the copy of one
+ * chunk overlaps the gather (and queued copy) of the next ones.
  *
  * `req_pages` (HOST array, n_requests entries) gives the number of pages of each request; pages of
  * request r occupy batch entries [sum(req_pages[:r]), +req_pages[r]) and, in staging, a contiguous
@@ -160,7 +161,7 @@ int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* batch,
  * `host_dst` must be pinned (hipHostMalloc / torch pin_memory) and hold the whole staging image.
  * Synchronous: returns when all bytes are in host memory.
  * ------------------------------------------------------------------------------------------ */
-typedef struct bikv_stager bikv_stager; /* opaque; owns the device chunk ring, 2 streams, events */
+typedef struct bikv_stager bikv_stager; /* opaque; owns n_buffers HIP streams, each with a chunk buffer */
 
 enum { BIKV_LAYOUT_LAYER_MAJOR = 0, BIKV_LAYOUT_PAGE_MAJOR = 1 };
 enum { BIKV_STAGE_PIPELINED = 0, /* gather to HBM chunk, then hipMemcpyAsync D2H */
