@@ -9,9 +9,9 @@ Three independent statements of the same semantics, so that they can be checked 
                 reduces to);
   * `*_loops` — pure-Python per-byte / per-page loops that follow the reference line by line, for
                 tiny inputs only.
-plus `*_torch`, the reference's CPU path as BASELINE describes it (torch.index_select /
-index_copy_ on host tensors; the vectorised form of Bi-KV/Worker/Worker.py:207), which the
-benchmark times as the CPU baseline.
+plus `*_torch`, the reference's CPU path as a library routine (torch.index_select / index_copy_ on
+host tensors; the vectorised form of the disabled host gather Bi-KV/Worker/Worker.py:207), which
+the benchmark times as the CPU baseline.
 
 Reference lines restated: Bi-KV/SharedMemory/CUDA_Shared/copy_kernel.cu:9-66 (the two kernels),
 :81-89,116-127 (ring step), ipc_service.cpp:118-138 (producer_send bookkeeping),
