@@ -45,11 +45,15 @@ def parse_args():
     ap.add_argument("--workload", default="qwen2_7b")
     ap.add_argument("--layout", default="layer_major", choices=["layer_major", "page_major"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-layout", dest="no_other_layout", action="store_true",
+                    help="skip the second measurement with the other staging layout")
     ap.add_argument("--pool-pages", type=int, default=0, help="override the pool size (pages per plane)")
     ap.add_argument("--seg", type=int, default=None)
     ap.add_argument("--unroll", type=int, default=None)
     ap.add_argument("--nontemporal", type=int, default=None)
     ap.add_argument("--wave-block", dest="wave_block", type=int, default=None)
+    ap.add_argument("--order", type=int, default=None)
+    ap.add_argument("--log2-chunk", dest="log2_chunk", type=int, default=None)
     ap.add_argument("--staging-cap-gb", dest="staging_cap_gb", type=float, default=32.0,
                     help="largest staging buffer of one launch; bigger batches take several launches")
     ap.add_argument("--chunk-mib", type=int, default=8, help="staging pipeline chunk (llama3_8b)")
@@ -186,7 +190,7 @@ def cpu_baseline(shape, wl, budget_s=20.0):
     }
 
 
-def run_gather_scatter(args, bk, workloads, dev):
+def run_gather_scatter(args, bk, workloads, dev, with_copy=True):
     import numpy as np
     import torch
 
@@ -296,7 +300,7 @@ def run_gather_scatter(args, bk, workloads, dev):
     alg_g //= len(g_groups)          # per launch, for the roofline entries below
     alg_s //= max(1, len(s_groups))
 
-    copy_gbps, copy_ok = time_plain_copy(bk, dev)
+    copy_gbps, copy_ok = time_plain_copy(bk, dev) if with_copy else (0.0, True)
     if not copy_ok:
         raise SystemExit("bench: plain copy mismatch")
 
@@ -332,7 +336,7 @@ def run_gather_scatter(args, bk, workloads, dev):
                                "min_ms": round(float(np.min(g_ms)), 4), "alg_bytes": alg_g},
                     "scatter": ({"GBps": round(s_gbps, 1), "avg_ms": round(float(np.mean(s_ms)), 4),
                                  "min_ms": round(float(np.min(s_ms)), 4), "alg_bytes": alg_s} if sb else None),
-                    "plain_copy_2GiB": {"GBps": round(copy_gbps, 1)}},
+                    "plain_copy_2GiB": ({"GBps": round(copy_gbps, 1)} if with_copy else None)},
     }
     del pool_t, scale_t, g_st, s_st
     torch.cuda.empty_cache()
@@ -450,7 +454,7 @@ def main():
         raise SystemExit("bench.py needs a GPU: the page-copy path has no CPU fallback")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    knobs = {k: getattr(args, k) for k in ("seg", "unroll", "nontemporal", "wave_block") if getattr(args, k) is not None}
+    knobs = {k: getattr(args, k) for k in ("seg", "unroll", "nontemporal", "wave_block", "order", "log2_chunk") if getattr(args, k) is not None}
     if knobs:
         bk.set_tuning(**knobs)
 
@@ -461,6 +465,16 @@ def main():
     out, shape, wl = run_gather_scatter(args, bk, workloads, dev)
     if knobs:
         out["config"]["tuning"] = knobs
+    if not args.no_other_layout:
+        # the same request stream with the other staging image (reported next to the headline number)
+        import copy
+        alt = copy.copy(args)
+        alt.layout = "page_major" if args.layout == "layer_major" else "layer_major"
+        alt.steps, alt.warmup = max(3, args.steps // 2), 2
+        log(f"same workload, staging layout {alt.layout}")
+        o2, _, _ = run_gather_scatter(alt, bk, workloads, dev, with_copy=False)
+        out["other_layout"] = {"layout": alt.layout, "value": o2["value"], "pct_of_hbm_peak": o2["pct_of_hbm_peak"],
+                               "steps": alt.steps, "kernels": {k: v for k, v in o2["kernels"].items() if v}}
     if args.workload == "llama3_8b":
         out["staging"] = run_staging(args, bk, workloads, dev)
     if not args.no_cpu_baseline:

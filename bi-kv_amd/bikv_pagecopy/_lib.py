@@ -18,6 +18,7 @@ ABI_VERSION = 1
 OK, EINVAL, EHIP, ESYS, ESTATE, EBOUNDS, ERANGE = 0, -1, -2, -3, -4, -5, -6
 ST_SRC_RANGE, ST_DST_RANGE, ST_PAGE_ID = 1, 2, 4
 LAYOUT_LAYER_MAJOR, LAYOUT_PAGE_MAJOR = 0, 1
+HINT_NONE, HINT_LAYER_MAJOR, HINT_PAGE_MAJOR = 0, 1, 2
 STAGE_PIPELINED, STAGE_DIRECT = 0, 1
 
 
@@ -44,6 +45,8 @@ class PageBatchDesc(C.Structure):
         ("plane_begin", C.c_int32),
         ("plane_count", C.c_int32),
         ("slot_bias", C.c_int64),
+        ("layout_hint", C.c_int32),
+        ("reserved", C.c_int32),
     ]
 
 

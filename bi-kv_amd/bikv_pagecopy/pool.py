@@ -58,6 +58,7 @@ class PageBatch:
         d.plane_begin = plane_begin
         d.plane_count = plane_count
         d.slot_bias = slot_bias
+        d.layout_hint = _lib.HINT_LAYER_MAJOR if self.layout == LAYER_MAJOR else _lib.HINT_PAGE_MAJOR
         return d
 
     def request_view(self, staging: torch.Tensor, r: int) -> torch.Tensor:

@@ -140,6 +140,12 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
     if (value != 64 && value != 128 && value != 256)
       return fail(BIKV_EINVAL, "wave_block must be 64, 128 or 256");
     t.wave_block = (int)value;
+  } else if (!strcmp(key, "order")) {
+    if (value < -1 || value > 1) return fail(BIKV_EINVAL, "order must be -1, 0 or 1");
+    t.order = (int)value;
+  } else if (!strcmp(key, "log2_chunk")) {
+    if (value < -1 || value > 16) return fail(BIKV_EINVAL, "log2_chunk must be in [-1, 16]");
+    t.log2_chunk = (int)value;
   } else if (!strcmp(key, "nontemporal")) {
     t.nontemporal = value < 0 ? -1 : (value ? 1 : 0);
   } else if (!strcmp(key, "run_chunk_kib")) {
@@ -232,6 +238,7 @@ static int build_move(const bikv_pool* pool, const bikv_page_batch* b, const voi
   m->n_batch = b->n_pages;
   m->plane_begin = pb;
   m->plane_count = pc;
+  m->layout_hint = b->layout_hint;
   if (b->n_pages == 0) return BIKV_OK;
   if (!b->page_ids || !b->slots || !b->slot_strides)
     return fail(BIKV_EINVAL, "page_ids, slots and slot_strides must be non-null");

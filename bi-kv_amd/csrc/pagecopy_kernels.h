@@ -35,6 +35,9 @@ struct MoveArgs {
   int64_t slot_bias;
   int32_t plane_begin;
   int32_t plane_count;
+  int32_t order;                  // wave mover: 0 = plane by plane, 1 = page chunk by page chunk
+  int32_t log2_chunk;             // order 1: pages per chunk = 2^log2_chunk
+  int32_t layout_hint;            // host side only: 0 none, 1 layer-major, 2 page-major staging
   uint32_t* status;
 };
 
@@ -42,8 +45,11 @@ struct Tuning {
   int seg = 0;          // 0 = wave mover when the shape qualifies, else segment movers with an
                         // automatic segment; > 0 = segment movers with this many pages per workgroup
   int wave_block = 64;  // lanes per workgroup of the wave mover (64, 128 or 256)
+  int order = -1;       // wave mover walk: 0 = plane by plane, 1 = chunk of pages by chunk of pages,
+                        // -1 = chosen from the batch's layout hint
+  int log2_chunk = -1;  // order 1: 2^log2_chunk pages per chunk; -1 = chosen
   int unroll = 4;       // 16-byte vectors in flight per lane (1, 2, 4 or 8)
-  int nontemporal = -1; // nt hint on payload loads and stores: 1 on, 0 off, -1 gathers only
+  int nontemporal = -1; // nt hint on payload loads and stores: 1 on, 0 off, -1 = chosen
   int run_chunk_kib = 0;  // bytes of a run handled by one workgroup, KiB; 0 = choose
 };
 Tuning& tuning();

@@ -57,8 +57,11 @@ int bikv_check_status(int device, void* stream, uint32_t* bits_out);
 /* Kernel launch knobs, for measurement. Keys: "seg" (0 = default: the wave mover, one 16-byte
  * vector per lane, whenever the tile shape qualifies; n > 0 = the LDS-staged segment mover with n
  * batch pages per workgroup), "wave_block" (lanes per workgroup of the wave mover: 64, 128, 256),
+ * "order" (wave mover walk: 0 = plane by plane, 1 = chunks of pages with their planes together,
+ * -1 = default: chosen from the batch's layout hint), "log2_chunk" (order 1: pages per chunk,
+ * -1 = chosen),
  * "unroll" (segment mover: 16-byte vectors in flight per lane: 1, 2, 4, 8), "nontemporal" (nt hint on
- * payload accesses: 1 on, 0 off, -1 = default: gathers and run copies only),
+ * payload accesses: 1 on, 0 off, -1 = default: chosen per direction and layout),
  * "run_chunk_kib" (bytes of a run per workgroup, KiB; 0 = automatic). Process-wide. */
 int bikv_set_tuning(const char* key, int64_t value);
 
@@ -126,7 +129,11 @@ typedef struct bikv_page_batch {
   int32_t plane_begin;
   int32_t plane_count;
   int64_t slot_bias;
+  int32_t layout_hint;  /* BIKV_HINT_*: how slots were laid out; affects speed only, never results */
+  int32_t reserved;
 } bikv_page_batch;
+
+enum { BIKV_HINT_NONE = 0, BIKV_HINT_LAYER_MAJOR = 1, BIKV_HINT_PAGE_MAJOR = 2 };
 
 /* gather: pool -> staging. Duplicate and out-of-order page ids are legal. Asynchronous on stream.
  * Replaces the per-layer form of the reference's gather (kvcache.py:132-239 driving

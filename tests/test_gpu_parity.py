@@ -305,6 +305,8 @@ def test_tuning_knobs_do_not_change_results(bk, oracle, cuda):
     try:
         # seg 0 = wave mover (wave_block lanes per workgroup); seg > 0 = LDS-staged segment mover
         cases = [dict(seg=0, wave_block=wb, nontemporal=nt) for wb in (64, 128, 256) for nt in (-1, 0, 1)]
+        # wave mover walks: plane by plane, or chunks of 2^k pages with their planes together
+        cases += [dict(seg=0, wave_block=64, order=o, log2_chunk=lc) for o in (0, 1) for lc in (-1, 0, 1, 3, 6, 10)]
         cases += [dict(seg=seg, unroll=u, nontemporal=nt) for seg in (1, 3, 16, 256) for u in (1, 2, 4, 8)
                   for nt in (0, 1)]
         for kw in cases:
@@ -319,7 +321,7 @@ def test_tuning_knobs_do_not_change_results(bk, oracle, cuda):
             assert _to_np(pool_d).tobytes() == want_pool.tobytes(), kw
             pool_d.copy_(torch.from_numpy(pool_h))
     finally:
-        bk.set_tuning(seg=0, wave_block=64, unroll=4, nontemporal=-1)
+        bk.set_tuning(seg=0, wave_block=64, unroll=4, nontemporal=-1, order=-1, log2_chunk=-1)
 
 
 # ---- run copy (reference API) -------------------------------------------------------------------
