@@ -102,7 +102,7 @@ _SIGNATURES = {
     "bikv_stager_destroy": (C.c_int, [C.c_void_p]),
     "bikv_gather_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PageBatchDesc),
                                       C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_void_p,
-                                      C.c_int64, C.c_int32, C.POINTER(StageStats)]),
+                                      C.c_int64, C.c_void_p, C.c_int64, C.c_int32, C.POINTER(StageStats)]),
     "bikv_plan_chunks": (C.c_int64, [C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_int32, C.c_int64,
                                      C.POINTER(C.c_int64), C.c_int64]),
     "bikv_d2h_copy": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,

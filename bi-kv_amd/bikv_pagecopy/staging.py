@@ -34,14 +34,21 @@ class HostStager:
         _lib.check(_lib.load().bikv_stager_create(idx, self.chunk_bytes, self.n_buffers, C.byref(h)))
         self._h = h
 
-    def gather_to_host(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "pipelined"):
-        """Fills `host` (pinned) with the staging image of `batch`; returns (bytes, chunks, seconds)."""
+    def gather_to_host(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "pipelined",
+                       host_scale: torch.Tensor = None):
+        """Fills `host` (pinned) with the staging image of `batch` (and `host_scale` with the scale
+        image of an fp8 pool); returns (bytes, chunks, seconds)."""
         if mode not in _MODES:
             raise ValueError(f"unknown mode {mode!r}")
-        if host.is_cuda or not host.is_pinned():
-            raise RuntimeError("CPU data must be pinned memory")  # message of copy_kernel.cu:142
-        if not host.is_contiguous():
-            raise RuntimeError("host staging buffer must be contiguous")
+        for t in (host, host_scale):
+            if t is None:
+                continue
+            if t.is_cuda or not t.is_pinned():
+                raise RuntimeError("CPU data must be pinned memory")  # message of copy_kernel.cu:142
+            if not t.is_contiguous():
+                raise RuntimeError("host staging buffer must be contiguous")
+        if pool.scale_tile_bytes and host_scale is None:
+            raise RuntimeError("pool has scales: a pinned host_scale buffer is required")
         # work queued on the caller's stream (e.g. the upload of the index arrays) must be visible
         torch.cuda.current_stream(self.device).synchronize()
         d = batch.desc()
@@ -49,7 +56,10 @@ class HostStager:
         rp = batch.req_pages.ctypes.data_as(C.POINTER(C.c_int64))
         _lib.check(_lib.load().bikv_gather_to_host(
             self._h, pool._h, C.byref(d), rp, len(batch.req_pages), _LAYOUT_CODE[batch.layout],
-            host.data_ptr(), host.numel() * host.element_size(), _MODES[mode], C.byref(stats)))
+            host.data_ptr(), host.numel() * host.element_size(),
+            host_scale.data_ptr() if host_scale is not None else None,
+            host_scale.numel() * host_scale.element_size() if host_scale is not None else 0,
+            _MODES[mode], C.byref(stats)))
         return stats.bytes, stats.n_chunks, stats.wall_seconds
 
     def close(self):

@@ -378,6 +378,8 @@ struct bikv_stager {
   int64_t chunk_bytes;
   int n_buf;
   char* ring;
+  char* scale_ring;          // grown on demand: n_buf chunks of scale tiles
+  int64_t scale_ring_bytes;
   std::vector<hipStream_t> lanes;
 };
 
@@ -396,6 +398,8 @@ extern "C" int bikv_stager_create(int device, int64_t chunk_bytes, int32_t n_buf
   st->chunk_bytes = chunk_bytes;
   st->n_buf = n_buffers;
   st->ring = nullptr;
+  st->scale_ring = nullptr;
+  st->scale_ring_bytes = 0;
   hipError_t e = hipMalloc((void**)&st->ring, (size_t)chunk_bytes * n_buffers);
   for (int i = 0; i < n_buffers && e == hipSuccess; ++i) {
     hipStream_t s = nullptr;
@@ -418,6 +422,7 @@ extern "C" int bikv_stager_destroy(bikv_stager* st) {
     (void)hipStreamDestroy(s);
   }
   if (st->ring) (void)hipFree(st->ring);
+  if (st->scale_ring) (void)hipFree(st->scale_ring);
   delete st;
   return BIKV_OK;
 }
@@ -504,11 +509,14 @@ extern "C" int64_t bikv_plan_chunks(const int64_t* req_pages, int64_t n_requests
 extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
                                    const bikv_page_batch* batch, const int64_t* req_pages,
                                    int64_t n_requests, int32_t layout, void* host_dst,
-                                   int64_t host_bytes, int32_t mode, bikv_stage_stats* stats) {
+                                   int64_t host_bytes, void* host_scale_dst,
+                                   int64_t host_scale_bytes, int32_t mode,
+                                   bikv_stage_stats* stats) {
   if (!st || !pool || !batch || !req_pages || !host_dst)
     return fail(BIKV_EINVAL, "null argument");
-  if (pool->scale_tile_bytes > 0)
-    return fail(BIKV_EINVAL, "the host staging pipeline moves payload-only pools");
+  const bool has_scale = pool->scale_tile_bytes > 0;
+  if (has_scale && !host_scale_dst)
+    return fail(BIKV_EINVAL, "pool has a scale class: host_scale_dst must be given");
   if (pool->device != st->device) return fail(BIKV_EINVAL, "pool and stager are on different devices");
   if (layout != BIKV_LAYOUT_LAYER_MAJOR && layout != BIKV_LAYOUT_PAGE_MAJOR)
     return fail(BIKV_EINVAL, "unknown layout %d", layout);
@@ -524,10 +532,15 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
     return fail(BIKV_EINVAL, "req_pages sums to %lld but the batch has %lld pages",
                 (long long)total_pages, (long long)batch->n_pages);
   const int64_t T = pool->tile_bytes;
+  const int64_t S = pool->scale_tile_bytes;
   const int64_t image_bytes = total_pages * pool->n_planes * T;
+  const int64_t scale_image_bytes = total_pages * pool->n_planes * S;
   if (host_bytes < image_bytes)
     return fail(BIKV_ERANGE, "host buffer holds %lld bytes, staging image needs %lld",
                 (long long)host_bytes, (long long)image_bytes);
+  if (has_scale && host_scale_bytes < scale_image_bytes)
+    return fail(BIKV_ERANGE, "host scale buffer holds %lld bytes, scale image needs %lld",
+                (long long)host_scale_bytes, (long long)scale_image_bytes);
   if (stats) { stats->bytes = 0; stats->n_chunks = 0; stats->wall_seconds = 0.0; }
   if (total_pages == 0) return BIKV_OK;
   BIKV_HIP(hipSetDevice(st->device));
@@ -535,8 +548,10 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
 
   if (mode == BIKV_STAGE_DIRECT) {
     void* dptr = nullptr;
+    void* sptr = nullptr;
     BIKV_HIP(hipHostGetDevicePointer(&dptr, host_dst, 0));
-    int rc = bikv_gather_pages(pool, batch, dptr, image_bytes, nullptr, 0, st->lanes[0]);
+    if (has_scale) BIKV_HIP(hipHostGetDevicePointer(&sptr, host_scale_dst, 0));
+    int rc = bikv_gather_pages(pool, batch, dptr, image_bytes, sptr, scale_image_bytes, st->lanes[0]);
     if (rc) return rc;
     rc = sync_and_check(st->device, st->lanes[0]);
     if (rc) return rc;
@@ -546,6 +561,16 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
     if (max_slots < 1)
       return fail(BIKV_ERANGE, "chunk_bytes %lld is smaller than one tile (%lld bytes)",
                   (long long)st->chunk_bytes, (long long)T);
+    // the scale tiles of a chunk ride in a second, much smaller buffer per lane
+    const int64_t scale_chunk = has_scale ? ((max_slots * S + 255) & ~int64_t(255)) : 0;
+    if (scale_chunk * st->n_buf > st->scale_ring_bytes) {
+      for (hipStream_t s : st->lanes) BIKV_HIP(hipStreamSynchronize(s));
+      if (st->scale_ring) BIKV_HIP(hipFree(st->scale_ring));
+      st->scale_ring = nullptr;
+      st->scale_ring_bytes = 0;
+      BIKV_HIP(hipMalloc((void**)&st->scale_ring, (size_t)(scale_chunk * st->n_buf)));
+      st->scale_ring_bytes = scale_chunk * st->n_buf;
+    }
     std::vector<Chunk> chunks;
     plan_chunks(req_pages, n_requests, pool->n_planes, layout, max_slots, &chunks);
     hipError_t e = hipSuccess;
@@ -558,6 +583,7 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
       }
       const int lane = (int)(c % (size_t)st->n_buf);
       char* dev_chunk = st->ring + (int64_t)lane * st->chunk_bytes;
+      char* dev_scale = has_scale ? st->scale_ring + (int64_t)lane * scale_chunk : nullptr;
       bikv_page_batch sub = *batch;
       sub.page_ids = batch->page_ids + ch.first_page;
       sub.slots = batch->slots + ch.first_page;
@@ -567,11 +593,17 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
       sub.plane_count = ch.plane_count;
       sub.slot_bias = ch.first_slot;
       // stream order on the lane keeps the buffer safe: this gather runs after the lane's previous copy
-      rc = bikv_gather_pages(pool, &sub, dev_chunk, ch.n_slots * T, nullptr, 0, st->lanes[lane]);
+      rc = bikv_gather_pages(pool, &sub, dev_chunk, ch.n_slots * T, dev_scale, ch.n_slots * S,
+                             st->lanes[lane]);
       if (rc) break;
       e = hipMemcpyAsync(static_cast<char*>(host_dst) + ch.first_slot * T, dev_chunk,
                          (size_t)(ch.n_slots * T), hipMemcpyDeviceToHost, st->lanes[lane]);
       if (e != hipSuccess) break;
+      if (has_scale) {
+        e = hipMemcpyAsync(static_cast<char*>(host_scale_dst) + ch.first_slot * S, dev_scale,
+                           (size_t)(ch.n_slots * S), hipMemcpyDeviceToHost, st->lanes[lane]);
+        if (e != hipSuccess) break;
+      }
     }
     // Drain every lane whatever happened, so that no work is left in flight on an error path.
     hipError_t es = hipSuccess;
@@ -590,7 +622,7 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
   }
   const auto t1 = std::chrono::steady_clock::now();
   if (stats) {
-    stats->bytes = image_bytes;
+    stats->bytes = image_bytes + scale_image_bytes;
     stats->wall_seconds = std::chrono::duration<double>(t1 - t0).count();
   }
   return BIKV_OK;

@@ -165,7 +165,8 @@ int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* batch,
  * request r occupy batch entries [sum(req_pages[:r]), +req_pages[r]) and, in staging, a contiguous
  * block of req_pages[r]*n_planes slots whose layout is `layout`. Chunks are cut on request, plane
  * and page boundaries so that each chunk is one contiguous byte range of the staging image.
- * `host_dst` must be pinned (hipHostMalloc / torch pin_memory) and hold the whole staging image.
+ * `host_dst` must be pinned (hipHostMalloc / torch pin_memory) and hold the whole staging image; the
+ * scale tiles of a pool with a scale class go, slot for slot, into a second pinned image.
  * Synchronous: returns when all bytes are in host memory.
  * ------------------------------------------------------------------------------------------ */
 typedef struct bikv_stager bikv_stager; /* opaque; owns n_buffers HIP streams, each with a chunk buffer */
@@ -185,7 +186,9 @@ typedef struct bikv_stage_stats {
 
 int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
                         const int64_t* req_pages, int64_t n_requests, int32_t layout,
-                        void* host_dst, int64_t host_bytes, int32_t mode,
+                        void* host_dst, int64_t host_bytes,
+                        void* host_scale_dst /* pinned; NULL iff the pool has no scale class */,
+                        int64_t host_scale_bytes, int32_t mode,
                         bikv_stage_stats* stats /* nullable */);
 
 /* The chunk plan bikv_gather_to_host would use, without touching a GPU: writes up to `cap` chunks

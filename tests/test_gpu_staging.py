@@ -33,6 +33,34 @@ def test_gather_to_host_matches_oracle(lib, oracle, cuda, layout, mode):
         stager.close()
 
 
+@pytest.mark.parametrize("layout", ["layer_major", "page_major"])
+@pytest.mark.parametrize("mode", ["pipelined", "direct"])
+def test_gather_to_host_moves_scales_with_the_payload(lib, oracle, cuda, layout, mode):
+    """fp8-style pool: 16 KiB payload tiles + 32-byte scale tiles go to two pinned images."""
+    import bikv_pagecopy as bk
+    print(f"[case] gather_to_host with scales {layout} {mode}", flush=True)
+    rng = np.random.default_rng(43)
+    n_planes, n_pages, tile, stile = 10, 60, 16384, 32
+    pool_h = rng.integers(0, 256, size=(n_planes, n_pages, tile), dtype=np.uint8)
+    scale_h = rng.integers(0, 256, size=(n_planes, n_pages, stile), dtype=np.uint8)
+    pool = bk.PagedKVPool.from_stacked(torch.from_numpy(pool_h).to(cuda), plane_dims=1,
+                                       scale=torch.from_numpy(scale_h).to(cuda))
+    reqs = [rng.permutation(n_pages)[:m] for m in (5, 31, 1, 0, 12)]
+    batch = pool.make_batch(reqs, layout)
+    want = oracle.gather_layered_c(pool_h, reqs, layout).tobytes()
+    swant = oracle.gather_layered_c(scale_h, reqs, layout).tobytes()
+    for chunk_tiles in (4, 1, 64):
+        stager = bk.HostStager(cuda, chunk_bytes=chunk_tiles * tile, n_buffers=2)
+        host = bk.pinned_empty(batch.n_slots * tile).fill_(0xA5)
+        shost = bk.pinned_empty(batch.n_slots * stile).fill_(0xA5)
+        nbytes, _, _ = stager.gather_to_host(pool, batch, host, mode, host_scale=shost)
+        assert nbytes == batch.n_slots * (tile + stile)
+        assert host.numpy().tobytes() == want and shost.numpy().tobytes() == swant, chunk_tiles
+        stager.close()
+    with pytest.raises(RuntimeError, match="host_scale"):
+        bk.HostStager(cuda).gather_to_host(pool, batch, bk.pinned_empty(batch.n_slots * tile), mode)
+
+
 def test_gather_to_host_argument_checks(lib, cuda):
     import bikv_pagecopy as bk
     print("[case] gather_to_host checks", flush=True)
