@@ -50,6 +50,22 @@ class PageBatchDesc(C.Structure):
     ]
 
 
+class NHDDesc(C.Structure):
+    _fields_ = [
+        ("device", C.c_int32),
+        ("n_layers", C.c_int32),
+        ("kv_heads", C.c_int32),
+        ("head_dim", C.c_int32),
+        ("block_tokens", C.c_int32),
+        ("elem_bytes", C.c_int32),
+        ("n_blocks", C.c_int64),
+        ("block_stride_elems", C.c_int64),
+        ("kv_stride_elems", C.c_int64),
+        ("token_stride_elems", C.c_int64),
+        ("layer_base", C.POINTER(C.c_void_p)),
+    ]
+
+
 class StageStats(C.Structure):
     _fields_ = [("bytes", C.c_int64), ("n_chunks", C.c_int64), ("wall_seconds", C.c_double)]
 
@@ -103,6 +119,12 @@ _SIGNATURES = {
     "bikv_gather_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PageBatchDesc),
                                       C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_void_p,
                                       C.c_int64, C.c_void_p, C.c_int64, C.c_int32, C.POINTER(StageStats)]),
+    "bikv_nhd_create": (C.c_int, [C.POINTER(NHDDesc), C.POINTER(C.c_void_p)]),
+    "bikv_nhd_destroy": (C.c_int, [C.c_void_p]),
+    "bikv_nhd_load_token_major": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
+                                            C.c_int64, C.c_void_p]),
+    "bikv_nhd_store_token_major": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
+                                             C.c_int64, C.c_void_p]),
     "bikv_plan_chunks": (C.c_int64, [C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_int32, C.c_int64,
                                      C.POINTER(C.c_int64), C.c_int64]),
     "bikv_d2h_copy": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,

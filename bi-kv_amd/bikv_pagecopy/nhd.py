@@ -1,0 +1,109 @@
+"""Per-layer paged NHD pool (the layout the model reads) and the fused layout change to and from
+token-major pages (the layout Bi-KV stores and transfers).
+
+The reference has both layouts and no code between them: Worker.receive_kvcache_data_batch stops at
+the received `(token_num,) + token_shape` tensor (Bi-KV/Worker/Worker.py:162-191) and nothing writes
+it into `local_kvcache` (Worker.py:74-78); send_kvcache_data_batch allocates the outgoing tensor and
+never fills it from the pool (Worker.py:193-207). `load_token_major` / `store_token_major` are those
+two missing steps, each one kernel launch over a batch of pages.
+"""
+import ctypes as C
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+
+
+class NHDPool:
+    """L layer tensors addressed (block, kv, token, head, d) with head_dim contiguous."""
+
+    def __init__(self, layers: Sequence[torch.Tensor], block_tokens: int, kv_heads: int, head_dim: int,
+                 n_blocks: int, block_stride: int, kv_stride: int, token_stride: int):
+        t0 = layers[0]
+        for t in layers:
+            if not t.is_cuda:
+                raise RuntimeError("Cache data must be on CUDA")
+            if not t.is_contiguous():
+                raise RuntimeError("Cache data must be contiguous")
+            if t.shape != t0.shape or t.dtype != t0.dtype:
+                raise RuntimeError("all layers must share shape and dtype")
+        self.device = t0.device
+        self.dtype = t0.dtype
+        self.n_layers = len(layers)
+        self.kv_heads, self.head_dim, self.block_tokens, self.n_blocks = kv_heads, head_dim, block_tokens, n_blocks
+        self.token_elems = head_dim * kv_heads * self.n_layers * 2        # one token, token-major
+        self.page_elems = block_tokens * self.token_elems
+        self._layers = list(layers)
+        d = _lib.NHDDesc()
+        d.device = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        d.n_layers, d.kv_heads, d.head_dim, d.block_tokens = self.n_layers, kv_heads, head_dim, block_tokens
+        d.elem_bytes = t0.element_size()
+        d.n_blocks = n_blocks
+        d.block_stride_elems, d.kv_stride_elems, d.token_stride_elems = block_stride, kv_stride, token_stride
+        arr = (C.c_void_p * self.n_layers)(*[t.data_ptr() for t in layers])
+        d.layer_base = C.cast(arr, C.POINTER(C.c_void_p))
+        h = C.c_void_p()
+        _lib.check(_lib.load().bikv_nhd_create(C.byref(d), C.byref(h)))
+        self._h = h
+
+    @classmethod
+    def from_token_kv_layers(cls, layers: Sequence[torch.Tensor], block_tokens: int):
+        """layers[l] is [blocks*block_tokens, 2, heads, dim] (Bi-KV/Worker/Worker.py:74-78)."""
+        slots, two, h, d = layers[0].shape
+        if two != 2 or slots % block_tokens:
+            raise RuntimeError("expected [blocks*block_tokens, 2, heads, dim] per layer")
+        return cls(layers, block_tokens, h, d, slots // block_tokens,
+                   block_stride=block_tokens * 2 * h * d, kv_stride=h * d, token_stride=2 * h * d)
+
+    @classmethod
+    def from_block_kv_layers(cls, layers: Sequence[torch.Tensor]):
+        """layers[l] is [blocks, 2, block_tokens, heads, dim] (Bi-KV/Model/qwen2.py:532-536)."""
+        blocks, two, p, h, d = layers[0].shape
+        if two != 2:
+            raise RuntimeError("expected [blocks, 2, block_tokens, heads, dim] per layer")
+        return cls(layers, p, h, d, blocks, block_stride=2 * p * h * d, kv_stride=p * h * d, token_stride=h * d)
+
+    def _call(self, fn, tm: torch.Tensor, block_ids: torch.Tensor, tm_pages: Optional[torch.Tensor]):
+        if not tm.is_cuda or not tm.is_contiguous():
+            raise RuntimeError("token-major buffer must be a contiguous CUDA tensor")
+        if tm.element_size() != self._layers[0].element_size():
+            raise RuntimeError("token-major buffer and pool differ in element size")
+        if tm_pages is None:
+            tm_pages = torch.arange(block_ids.numel(), dtype=torch.int64, device=self.device)
+        for name, t in (("block_ids", block_ids), ("tm_pages", tm_pages)):
+            if not t.is_cuda or t.dtype != torch.int64 or t.dim() != 1 or not t.is_contiguous():
+                raise RuntimeError(f"{name} must be a contiguous 1-D int64 CUDA tensor")
+        if tm_pages.numel() != block_ids.numel():
+            raise RuntimeError("block_ids and tm_pages differ in length")
+        with torch.cuda.device(self.device):
+            _lib.check(fn(self._h, tm.data_ptr(), tm.numel() * tm.element_size(), block_ids.data_ptr(),
+                          tm_pages.data_ptr(), block_ids.numel(),
+                          C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)))
+
+    def load_token_major(self, tm: torch.Tensor, block_ids: torch.Tensor, tm_pages: Optional[torch.Tensor] = None):
+        """Received token-major pages -> pool blocks (unique block ids). `tm` holds pages of
+        block_tokens tokens, each token [dim][heads][layers][2]; page i of the call is tm page
+        tm_pages[i] (default: i). Asynchronous on the current stream."""
+        self._call(_lib.load().bikv_nhd_load_token_major, tm, block_ids, tm_pages)
+
+    def store_token_major(self, tm: torch.Tensor, block_ids: torch.Tensor, tm_pages: Optional[torch.Tensor] = None):
+        """Pool blocks -> token-major pages (unique tm pages). Asynchronous on the current stream."""
+        self._call(_lib.load().bikv_nhd_store_token_major, tm, block_ids, tm_pages)
+
+    def check(self):
+        idx = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.load().bikv_check_status(
+                idx, C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream), None))
+
+    def close(self):
+        if getattr(self, "_h", None):
+            _lib.load().bikv_nhd_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -627,3 +627,123 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
   }
   return BIKV_OK;
 }
+
+// ---- per-layer paged NHD pool and the fused layout change ------------------------------------
+struct bikv_nhd {
+  int device;
+  int n_layers, kv_heads, head_dim, block_tokens, elem_bytes;
+  int64_t n_blocks;
+  int64_t block_stride, kv_stride, token_stride;   // elements
+  const char** d_layer_base;
+};
+
+extern "C" int bikv_nhd_create(const bikv_nhd_desc* d, bikv_nhd** out) {
+  if (!d || !out) return fail(BIKV_EINVAL, "null argument");
+  *out = nullptr;
+  if (d->n_layers <= 0 || d->n_layers > 65536 || d->kv_heads <= 0 || d->head_dim <= 0 ||
+      d->block_tokens <= 0 || d->n_blocks <= 0)
+    return fail(BIKV_EINVAL, "layers, kv_heads, head_dim, block_tokens and n_blocks must be positive");
+  if (d->elem_bytes != 1 && d->elem_bytes != 2 && d->elem_bytes != 4)
+    return fail(BIKV_EINVAL, "elem_bytes must be 1, 2 or 4");
+  const int ve = 16 / d->elem_bytes;
+  const int64_t cols = (int64_t)d->kv_heads * d->n_layers * 2;
+  if (d->head_dim % ve != 0 || cols % ve != 0)
+    return fail(BIKV_EINVAL, "head_dim (%d) and kv_heads*layers*2 (%lld) must be multiples of %d elements (16 bytes)",
+                d->head_dim, (long long)cols, ve);
+  if (cols >= (int64_t(1) << 24) || (int64_t)d->head_dim * (ve + 4 / d->elem_bytes) * d->elem_bytes > 48 * 1024)
+    return fail(BIKV_EINVAL, "token shape too large for the layout-change kernel");
+  if (!d->layer_base) return fail(BIKV_EINVAL, "layer_base is null");
+  if (d->kv_stride_elems < 0 || d->token_stride_elems < d->kv_heads * (int64_t)d->head_dim ||
+      d->block_stride_elems < (int64_t)d->block_tokens * 2 * d->kv_heads * d->head_dim)
+    return fail(BIKV_EINVAL, "strides are smaller than the data they separate");
+  std::vector<const char*> table((size_t)d->n_layers);
+  for (int l = 0; l < d->n_layers; ++l) {
+    if (!d->layer_base[l]) return fail(BIKV_EINVAL, "layer_base[%d] is null", l);
+    if (((uint64_t)d->layer_base[l]) & 15) return fail(BIKV_EINVAL, "layer_base[%d] is not 16-byte aligned", l);
+    table[l] = static_cast<const char*>(d->layer_base[l]);
+  }
+  if (((d->block_stride_elems | d->kv_stride_elems | d->token_stride_elems) * d->elem_bytes) & 15)
+    return fail(BIKV_EINVAL, "strides must be multiples of 16 bytes");
+  uint32_t* st = nullptr;
+  int rc = device_status(d->device, &st);
+  if (rc) return rc;
+  BIKV_HIP(hipSetDevice(d->device));
+  void* dtab = nullptr;
+  BIKV_HIP(hipMalloc(&dtab, table.size() * sizeof(char*)));
+  hipError_t e = hipMemcpy(dtab, table.data(), table.size() * sizeof(char*), hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    (void)hipFree(dtab);
+    return fail_hip(e, "hipMemcpy(layer table)");
+  }
+  bikv_nhd* p = new bikv_nhd();
+  p->device = d->device;
+  p->n_layers = d->n_layers;
+  p->kv_heads = d->kv_heads;
+  p->head_dim = d->head_dim;
+  p->block_tokens = d->block_tokens;
+  p->elem_bytes = d->elem_bytes;
+  p->n_blocks = d->n_blocks;
+  p->block_stride = d->block_stride_elems;
+  p->kv_stride = d->kv_stride_elems;
+  p->token_stride = d->token_stride_elems;
+  p->d_layer_base = static_cast<const char**>(dtab);
+  *out = p;
+  return BIKV_OK;
+}
+
+extern "C" int bikv_nhd_destroy(bikv_nhd* p) {
+  if (!p) return BIKV_OK;
+  (void)hipSetDevice(p->device);
+  hipError_t e = hipFree((void*)p->d_layer_base);
+  delete p;
+  if (e != hipSuccess) return fail_hip(e, "hipFree(layer table)");
+  return BIKV_OK;
+}
+
+static int transpose_pages(int dir, const bikv_nhd* nhd, void* tm, int64_t tm_bytes,
+                           const int64_t* block_ids, const int64_t* tm_pages, int64_t n_pages,
+                           void* stream) {
+  if (!nhd) return fail(BIKV_EINVAL, "null pool");
+  if (n_pages < 0) return fail(BIKV_EINVAL, "negative n_pages");
+  if (n_pages == 0) return BIKV_OK;
+  if (!tm || !block_ids || !tm_pages) return fail(BIKV_EINVAL, "null pointer argument");
+  if (((uint64_t)tm) & 15) return fail(BIKV_EINVAL, "token-major buffer is not 16-byte aligned");
+  const int64_t cols = (int64_t)nhd->kv_heads * nhd->n_layers * 2;
+  const int64_t page_bytes = (int64_t)nhd->block_tokens * nhd->head_dim * cols * nhd->elem_bytes;
+  if (tm_bytes < page_bytes) return fail(BIKV_EINVAL, "token-major buffer is smaller than one page");
+  TransposeArgs a;
+  memset(&a, 0, sizeof(a));
+  a.layer_base = nhd->d_layer_base;
+  a.tm_base = static_cast<char*>(tm);
+  a.block_ids = block_ids;
+  a.tm_pages = tm_pages;
+  a.n_pages = n_pages;
+  a.n_blocks = nhd->n_blocks;
+  a.n_tm_pages = tm_bytes / page_bytes;
+  a.block_stride = nhd->block_stride;
+  a.kv_stride = nhd->kv_stride;
+  a.token_stride = nhd->token_stride;
+  a.n_layers = nhd->n_layers;
+  a.head_dim = nhd->head_dim;
+  a.n_cols = (int32_t)cols;
+  a.block_tokens = nhd->block_tokens;
+  a.elem_bytes = nhd->elem_bytes;
+  int rc = device_status(nhd->device, &a.status);
+  if (rc) return rc;
+  BIKV_HIP(hipSetDevice(nhd->device));
+  hipError_t e = launch_transpose_pages(dir, a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail_hip(e, "layout-change launch");
+  return BIKV_OK;
+}
+
+extern "C" int bikv_nhd_store_token_major(const bikv_nhd* nhd, void* tm, int64_t tm_bytes,
+                                          const int64_t* block_ids, const int64_t* tm_pages,
+                                          int64_t n_pages, void* stream) {
+  return transpose_pages(0, nhd, tm, tm_bytes, block_ids, tm_pages, n_pages, stream);
+}
+
+extern "C" int bikv_nhd_load_token_major(const bikv_nhd* nhd, const void* tm, int64_t tm_bytes,
+                                         const int64_t* block_ids, const int64_t* tm_pages,
+                                         int64_t n_pages, void* stream) {
+  return transpose_pages(1, nhd, const_cast<void*>(tm), tm_bytes, block_ids, tm_pages, n_pages, stream);
+}

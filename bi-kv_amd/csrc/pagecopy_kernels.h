@@ -75,4 +75,23 @@ struct RunArgs {
 };
 hipError_t launch_copy_runs(const RunArgs& a, hipStream_t stream);
 
+// Fused page move + layout change between token-major pages and a per-layer paged NHD pool.
+struct TransposeArgs {
+  const char* const* layer_base;  // device-resident table, n_layers entries
+  char* tm_base;                  // token-major side: pages of block_tokens tokens
+  const int64_t* block_ids;       // compute-side block of each page
+  const int64_t* tm_pages;        // token-major page index of each page
+  int64_t n_pages;
+  int64_t n_blocks;               // compute-side blocks (bounds check)
+  int64_t n_tm_pages;             // token-major pages available (bounds check)
+  int64_t block_stride, kv_stride, token_stride;  // compute side, in elements
+  int32_t n_layers, head_dim, n_cols;             // n_cols = kv_heads * n_layers * 2
+  int32_t block_tokens, elem_bytes;
+  int32_t chunk_cols, pitch;      // filled by the launcher
+  uint32_t n_chunks, tile_words;
+  uint32_t* status;
+};
+// dir 0: compute -> token-major, dir 1: token-major -> compute.
+hipError_t launch_transpose_pages(int dir, TransposeArgs& a, hipStream_t stream);
+
 }  // namespace bikv

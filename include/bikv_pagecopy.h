@@ -206,6 +206,51 @@ int bikv_host_alloc(int64_t bytes, void** out);
 int bikv_host_free(void* p);
 
 /* --------------------------------------------------------------------------------------------
+ * 3b. Fused page move + layout change: token-major pages <-> per-layer paged NHD pool.
+ *
+ * Bi-KV keeps KV in two layouts and never converts between them: the storage / transfer layout is
+ * token-major, one token = [head_dim][kv_heads][layers][2] elements (Model/qwen2.py:519-522; pools
+ * (tokens,)+token_shape at kvcache.py:38-43, Worker.py:57-62), while the model reads a per-layer
+ * paged pool whose rows are head_dim contiguous elements: [blocks*block, 2, heads, dim] per layer at
+ * Worker.py:74-78, [blocks, 2, block, heads, dim] at Model/qwen2.py:532-536. Worker.receive_kvcache_
+ * data_batch (Worker.py:162-191) stops at the received token-major tensor; these two calls are the
+ * missing step, fused with the page scatter/gather:
+ *   load : compute[l][block_ids[i]][k][t][h][:] = tm[tm_pages[i]][t][:, h, l, k]   (received KV -> pool)
+ *   store: the inverse                                                             (pool -> KV to send)
+ * for every page i < n_pages and every token t < block_tokens of it. The compute side is addressed
+ *   layer_base[l] + (block*block_stride + k*kv_stride + t*token_stride + h*head_dim + d) * elem_bytes
+ * which covers both reference forms (Worker.py form: block_stride = block*2*H*D, kv_stride = H*D,
+ * token_stride = 2*H*D; qwen2.py form: block_stride = 2*block*H*D, kv_stride = block*H*D,
+ * token_stride = H*D). `tm` is an array of token-major pages of block_tokens tokens each; `block_ids`
+ * and `tm_pages` are int64 device arrays. Block ids must be unique in a load, page indices in a store.
+ * Requires head_dim and kv_heads*layers*2 to be multiples of 16 bytes' worth of elements.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct bikv_nhd bikv_nhd; /* opaque; owns a device-resident table of layer base pointers */
+
+typedef struct bikv_nhd_desc {
+  int32_t device;
+  int32_t n_layers;
+  int32_t kv_heads;
+  int32_t head_dim;
+  int32_t block_tokens;
+  int32_t elem_bytes;            /* 1, 2 or 4 */
+  int64_t n_blocks;
+  int64_t block_stride_elems;
+  int64_t kv_stride_elems;
+  int64_t token_stride_elems;
+  const void* const* layer_base; /* HOST array of n_layers device pointers, 16-byte aligned */
+} bikv_nhd_desc;
+
+int bikv_nhd_create(const bikv_nhd_desc* desc, bikv_nhd** out);
+int bikv_nhd_destroy(bikv_nhd* pool);
+int bikv_nhd_load_token_major(const bikv_nhd* pool, const void* tm, int64_t tm_bytes,
+                              const int64_t* block_ids, const int64_t* tm_pages, int64_t n_pages,
+                              void* stream);
+int bikv_nhd_store_token_major(const bikv_nhd* pool, void* tm, int64_t tm_bytes,
+                               const int64_t* block_ids, const int64_t* tm_pages, int64_t n_pages,
+                               void* stream);
+
+/* --------------------------------------------------------------------------------------------
  * 4. Producer/consumer ring — the `ipc_service` roles.
  *
  * The control block lives in POSIX shared memory and is byte-compatible with the reference's

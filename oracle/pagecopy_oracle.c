@@ -14,6 +14,10 @@
  *                           the per-(page, layer, K/V) form of the same copy over the Worker's paged
  *                           pool (Worker/Worker.py:74-78, Model/qwen2.py:532-536); scatter is the
  *                           vectorised form of the disabled host line Worker.py:207
+ *   oracle_transpose_pages  page move fused with the change between the token-major layout
+ *                           (Model/qwen2.py:519-522) and the per-layer paged layout (Worker.py:74-78,
+ *                           qwen2.py:532-536); the reference has no code for it, the index formulas
+ *                           are the two layouts' definitions
  *
  * How each is pinned (tests/test_oracle.py): the two known-answer scenarios the reference's own
  * scripts hold (test_page_ipc.py:41-65,127-150; test_zero_copy.py:30-48,86-103), the library
@@ -158,6 +162,44 @@ int64_t oracle_scatter_layered(uint8_t* const* plane_base, int32_t n_planes, int
       }
     first += m;
     base += m * n_planes;
+  }
+  return bad;
+}
+
+/* Fused page move + layout change between the reference's two KV layouts (it holds both and no
+ * code between them, so there is no reference vector; the index formulas ARE the two layouts):
+ *   token-major page: element (t, d, h, l, k) of page p at ((((p*P + t)*D + d)*H + h)*L + l)*2 + k
+ *     (token_shape = (head_size, num_kv_heads, num_layers, 2), Model/qwen2.py:519-522);
+ *   compute pool, layer l: element (block b, k, t, h, d) at
+ *     b*block_stride + k*kv_stride + t*token_stride + h*D + d
+ *     (Worker/Worker.py:74-78: [blocks*P, 2, H, D] -> strides (P*2*H*D, H*D, 2*H*D);
+ *      Model/qwen2.py:532-536: [blocks, 2, P, H, D] -> strides (2*P*H*D, P*H*D, H*D)).
+ * dir 1: token-major -> compute; dir 0: compute -> token-major. Returns the number of pages whose
+ * block id or token-major page index is out of range (skipped). */
+int64_t oracle_transpose_pages(uint8_t* const* layer_base, int32_t n_layers, int32_t kv_heads,
+                               int32_t head_dim, int32_t block_tokens, int32_t elem_bytes,
+                               int64_t n_blocks, int64_t block_stride, int64_t kv_stride,
+                               int64_t token_stride, uint8_t* tm, int64_t n_tm_pages,
+                               const int64_t* block_ids, const int64_t* tm_pages, int64_t n,
+                               int32_t dir) {
+  const int64_t P = block_tokens, D = head_dim, H = kv_heads, L = n_layers;
+  int64_t bad = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    const int64_t b = block_ids[i], p = tm_pages[i];
+    if (b < 0 || b >= n_blocks || p < 0 || p >= n_tm_pages) { ++bad; continue; }
+    for (int64_t t = 0; t < P; ++t)
+      for (int64_t d = 0; d < D; ++d)
+        for (int64_t h = 0; h < H; ++h)
+          for (int64_t l = 0; l < L; ++l)
+            for (int64_t k = 0; k < 2; ++k) {
+              const int64_t ti = ((((p * P + t) * D + d) * H + h) * L + l) * 2 + k;
+              const int64_t ci = b * block_stride + k * kv_stride + t * token_stride + h * D + d;
+              uint8_t* tp = tm + ti * elem_bytes;
+              uint8_t* cp = layer_base[l] + ci * elem_bytes;
+              for (int32_t e = 0; e < elem_bytes; ++e) {
+                if (dir) cp[e] = tp[e]; else tp[e] = cp[e];
+              }
+            }
   }
   return bad;
 }

@@ -59,6 +59,9 @@ def clib():
             fn.restype = C.c_int64
             fn.argtypes = [C.POINTER(C.c_void_p), C.c_int32, C.c_int64, C.c_int64, C.c_int64, i64p, i64p,
                            C.c_int64, C.c_int32, u8p]
+        lib.oracle_transpose_pages.restype = C.c_int64
+        lib.oracle_transpose_pages.argtypes = [C.POINTER(C.c_void_p)] + [C.c_int32] * 5 + [C.c_int64] * 4 + \
+            [u8p, C.c_int64, i64p, i64p, C.c_int64, C.c_int32]
         _clib = lib
     return _clib
 
@@ -248,6 +251,52 @@ def gather_layered_loops(pool, requests, layout="layer_major"):
                     out[slot * tile + e] = pool[q, int(ids[j]), e]
         base += m * n_planes
     return out
+
+
+# ---------------------------------------------------------------------------------------------
+# fused page move + layout change: token-major pages <-> per-layer paged NHD pool
+#   tm: numpy array [n_tm_pages, P, D, H, L, 2] (token_shape = (D, H, L, 2), Model/qwen2.py:519-522)
+#   layers: list of L numpy arrays, form "token_kv" [blocks*P, 2, H, D] (Worker/Worker.py:74-78) or
+#           "block_kv" [blocks, 2, P, H, D] (Model/qwen2.py:532-536)
+# ---------------------------------------------------------------------------------------------
+def _nhd_strides(layers, form, P):
+    if form == "token_kv":
+        slots, two, H, D = layers[0].shape
+        return slots // P, H, D, (P * 2 * H * D, H * D, 2 * H * D)
+    blocks, two, p, H, D = layers[0].shape
+    assert p == P
+    return blocks, H, D, (2 * P * H * D, P * H * D, H * D)
+
+
+def transpose_pages_c(layers, form, tm, block_ids, tm_pages, direction):
+    """direction "load": tm -> layers; "store": layers -> tm. In place. Returns skipped pages."""
+    P = tm.shape[1]
+    n_blocks, H, D, (bs, ks, ts) = _nhd_strides(layers, form, P)
+    assert tm.shape[2:] == (D, H, len(layers), 2) and tm.flags.c_contiguous
+    assert all(a.flags.c_contiguous for a in layers)
+    ptrs = (C.c_void_p * len(layers))(*[a.ctypes.data for a in layers])
+    b, bp = _i64(block_ids)
+    t, tp = _i64(tm_pages)
+    return clib().oracle_transpose_pages(ptrs, len(layers), H, D, P, tm.dtype.itemsize, n_blocks, bs, ks, ts,
+                                         tm.ctypes.data, tm.shape[0], bp, tp, len(b),
+                                         1 if direction == "load" else 0)
+
+
+def transpose_pages_np(layers, form, tm, block_ids, tm_pages, direction):
+    """The same with numpy's transpose: per page and layer, [P, D, H, 2] <-> [P, 2, H, D]."""
+    P = tm.shape[1]
+    for b, p in zip(block_ids, tm_pages):
+        for l, layer in enumerate(layers):
+            if form == "token_kv":
+                view = layer[b * P:(b + 1) * P]                      # [P, 2, H, D]
+                axes_to, axes_from = (0, 3, 2, 1), (0, 3, 2, 1)      # [P,D,H,2] <-> [P,2,H,D]
+            else:
+                view = layer[b]                                      # [2, P, H, D]
+                axes_to, axes_from = (3, 0, 2, 1), (1, 3, 2, 0)      # [P,D,H,2] -> [2,P,H,D] and back
+            if direction == "load":
+                view[...] = np.transpose(tm[p][:, :, :, l, :], axes_to)
+            else:
+                tm[p][:, :, :, l, :] = np.transpose(view, axes_from)
 
 
 # ---------------------------------------------------------------------------------------------

@@ -1,0 +1,101 @@
+"""Fused page move + layout change (token-major pages <-> per-layer paged NHD pool) on a real GPU,
+bit-exact against the oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+_NP = {1: np.uint8, 2: np.uint16, 4: np.uint32}
+_TORCH = {1: torch.uint8, 2: torch.float16, 4: torch.float32}
+
+
+def _to_np(t):
+    return t.detach().cpu().contiguous().view(torch.uint8).numpy()
+
+
+def _make(rng, form, es, P, D, H, L, blocks, n_tm, cuda):
+    dt = _NP[es]
+    tm_h = rng.integers(0, np.iinfo(dt).max, size=(n_tm, P, D, H, L, 2), dtype=dt)
+    shape = (blocks * P, 2, H, D) if form == "token_kv" else (blocks, 2, P, H, D)
+    layers_h = [rng.integers(0, np.iinfo(dt).max, size=shape, dtype=dt) for _ in range(L)]
+    tm_d = torch.from_numpy(tm_h.view(np.uint8)).to(cuda).view(_TORCH[es]).view(tm_h.shape)
+    layers_d = [torch.from_numpy(a.view(np.uint8)).to(cuda).view(_TORCH[es]).view(a.shape) for a in layers_h]
+    return tm_h, layers_h, tm_d, layers_d
+
+
+@pytest.mark.parametrize("form", ["token_kv", "block_kv"])
+@pytest.mark.parametrize("es,P,D,H,L", [
+    (2, 16, 128, 2, 28),     # the reference's Qwen2-1.5B token shape (Model/qwen2.py:512-522), block of 16
+    (2, 16, 128, 4, 28),     # Qwen2-7B
+    (2, 32, 128, 8, 32),     # Llama-3-8B: 512 columns -> four column chunks per token
+    (1, 16, 128, 8, 80),     # fp8 payload, 1280 columns
+    (4, 4, 64, 2, 6),        # fp32
+    (2, 3, 8, 2, 2),         # the smallest shape the kernel takes (one vector per row)
+    (2, 5, 80, 4, 3),        # head_dim 80: 10 vectors per row, not a multiple of 4
+])
+def test_load_and_store_match_oracle(lib, oracle, cuda, form, es, P, D, H, L):
+    import bikv_pagecopy as bk
+    print(f"[case] layout change {form} es={es} P={P} D={D} H={H} L={L}", flush=True)
+    rng = np.random.default_rng(es * 1000 + D + H + L)
+    blocks, n_tm = 9, 7
+    tm_h, layers_h, tm_d, layers_d = _make(rng, form, es, P, D, H, L, blocks, n_tm, cuda)
+    pool = (bk.NHDPool.from_token_kv_layers(layers_d, P) if form == "token_kv"
+            else bk.NHDPool.from_block_kv_layers(layers_d))
+    block_ids = rng.permutation(blocks)[:5].astype(np.int64)
+    tm_pages = rng.permutation(n_tm)[:5].astype(np.int64)
+    b_d, t_d = torch.from_numpy(block_ids).to(cuda), torch.from_numpy(tm_pages).to(cuda)
+    # load: token-major pages -> pool blocks
+    pool.load_token_major(tm_d, b_d, t_d)
+    pool.check()
+    assert oracle.transpose_pages_c(layers_h, form, tm_h, block_ids, tm_pages, "load") == 0
+    for l in range(L):
+        assert _to_np(layers_d[l]).tobytes() == layers_h[l].tobytes(), f"layer {l}"
+    # store: other pool blocks -> other token-major pages
+    block_ids2 = rng.permutation(blocks)[:4].astype(np.int64)
+    tm_pages2 = rng.permutation(n_tm)[:4].astype(np.int64)
+    pool.store_token_major(tm_d, torch.from_numpy(block_ids2).to(cuda), torch.from_numpy(tm_pages2).to(cuda))
+    pool.check()
+    assert oracle.transpose_pages_c(layers_h, form, tm_h, block_ids2, tm_pages2, "store") == 0
+    assert _to_np(tm_d).tobytes() == tm_h.tobytes()
+
+
+def test_default_tm_pages_is_a_dense_received_buffer(lib, oracle, cuda):
+    """A received tensor (tokens,)+token_shape (Worker.py:166-169) is pages 0..n-1 in order."""
+    import bikv_pagecopy as bk
+    print("[case] layout change dense buffer", flush=True)
+    rng = np.random.default_rng(5)
+    P, D, H, L, blocks = 16, 128, 2, 28, 12
+    tm_h, layers_h, tm_d, layers_d = _make(rng, "token_kv", 2, P, D, H, L, blocks, 6, cuda)
+    pool = bk.NHDPool.from_token_kv_layers(layers_d, P)
+    ids = rng.permutation(blocks)[:6].astype(np.int64)
+    recv = tm_d.view(6 * P, D, H, L, 2)                      # the reference's shape
+    pool.load_token_major(recv, torch.from_numpy(ids).to(cuda))
+    pool.check()
+    oracle.transpose_pages_c(layers_h, "token_kv", tm_h, ids, np.arange(6), "load")
+    for l in range(L):
+        assert _to_np(layers_d[l]).tobytes() == layers_h[l].tobytes()
+    # the model-side view of one element, spelled out
+    t, d, h, l, k = 3, 77, 1, 20, 1
+    assert layers_d[l][ids[2] * P + t, k, h, d].item() == recv[2 * P + t, d, h, l, k].item()
+
+
+def test_bad_ids_are_skipped_and_reported_and_shapes_are_checked(lib, cuda):
+    import bikv_pagecopy as bk
+    print("[case] layout change error paths", flush=True)
+    P, D, H, L, blocks = 4, 64, 2, 4, 5
+    layers = [torch.zeros((blocks * P, 2, H, D), dtype=torch.float16, device=cuda) for _ in range(L)]
+    pool = bk.NHDPool.from_token_kv_layers(layers, P)
+    tm = torch.ones((3, P, D, H, L, 2), dtype=torch.float16, device=cuda)
+    pool.load_token_major(tm, torch.tensor([1, 9, 2], device=cuda), torch.tensor([0, 1, 5], device=cuda))
+    with pytest.raises(RuntimeError, match="page-id"):
+        pool.check()
+    assert torch.all(layers[0][1 * P:2 * P] == 1) and not layers[0][2 * P:3 * P].any()   # page 0 moved, others not
+    with pytest.raises(RuntimeError, match="multiples of"):
+        bk.NHDPool.from_token_kv_layers([torch.zeros((8, 2, 1, 12), dtype=torch.float16, device=cuda)], 4)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        bk.NHDPool.from_token_kv_layers([torch.zeros((8, 2, 2, 64), dtype=torch.float16)], 4)
+    with pytest.raises(RuntimeError, match="element size"):
+        pool.load_token_major(tm.float(), torch.tensor([1], device=cuda))
+    with pytest.raises(RuntimeError, match="int64"):
+        pool.load_token_major(tm, torch.tensor([1], device=cuda, dtype=torch.int32))

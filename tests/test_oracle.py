@@ -248,3 +248,49 @@ def test_config1_golden_digests(oracle):
         p = pool.copy()
         oracle.scatter_layered_c(p, wl["scatter"], st, layout)
         assert _sha(p) == g[layout]["pool_after_scatter_sha256"]
+
+
+# ---- fused page move + layout change -----------------------------------------------------------
+@pytest.mark.parametrize("form", ["token_kv", "block_kv"])
+@pytest.mark.parametrize("dtype", [np.uint8, np.uint16, np.uint32])
+def test_transpose_pages_statements_agree(oracle, form, dtype):
+    rng = np.random.default_rng(14)
+    P, D, H, L, blocks, n_tm = 4, 8, 2, 3, 7, 5
+    tm = rng.integers(0, np.iinfo(dtype).max, size=(n_tm, P, D, H, L, 2), dtype=dtype)
+    shape = (blocks * P, 2, H, D) if form == "token_kv" else (blocks, 2, P, H, D)
+    block_ids, tm_pages = np.array([5, 0, 3]), np.array([4, 1, 2])
+    la = [np.zeros(shape, dtype=dtype) for _ in range(L)]
+    for a in la:
+        a.view(np.uint8)[...] = 0xA5
+    lb = [a.copy() for a in la]
+    assert oracle.transpose_pages_c(la, form, tm, block_ids, tm_pages, "load") == 0
+    oracle.transpose_pages_np(lb, form, tm, block_ids, tm_pages, "load")
+    for a, b in zip(la, lb):
+        assert a.tobytes() == b.tobytes()
+    # one element by hand: page 0 of the call (block 5, tm page 4), token 2, d 6, head 1, layer 2, V
+    want = tm[4, 2, 6, 1, 2, 1]
+    got = la[2][5 * P + 2, 1, 1, 6] if form == "token_kv" else la[2][5, 1, 2, 1, 6]
+    assert got == want
+    # blocks that were not named keep their canary
+    untouched = la[0][1 * P:(1 + 1) * P] if form == "token_kv" else la[0][1]
+    assert np.all(untouched.view(np.uint8) == 0xA5)
+    # store is the inverse of load
+    tm2 = np.zeros_like(tm)
+    tm3 = np.zeros_like(tm)
+    assert oracle.transpose_pages_c(la, form, tm2, block_ids, tm_pages, "store") == 0
+    oracle.transpose_pages_np(la, form, tm3, block_ids, tm_pages, "store")
+    assert tm2.tobytes() == tm3.tobytes()
+    assert np.array_equal(tm2[tm_pages], tm[tm_pages]) and not tm2[[0, 3]].any()
+    # out-of-range ids are skipped and counted
+    assert oracle.transpose_pages_c(la, form, tm, np.array([7, 1]), np.array([0, 9]), "load") == 2
+
+
+def test_transpose_pages_equals_the_flat_token_major_formula(oracle):
+    """The token-major page really is the reference's (tokens,)+token_shape buffer: flat element
+    offset (((t*D + d)*H + h)*L + l)*2 + k with token_shape = (D, H, L, 2)."""
+    P, D, H, L = 2, 8, 2, 4
+    tm = np.arange(1 * P * D * H * L * 2, dtype=np.uint16).reshape(1, P, D, H, L, 2)
+    layers = [np.zeros((3 * P, 2, H, D), dtype=np.uint16) for _ in range(L)]
+    oracle.transpose_pages_c(layers, "token_kv", tm, [2], [0], "load")
+    t, d, h, l, k = 1, 5, 1, 3, 0
+    assert layers[l][2 * P + t, k, h, d] == (((t * D + d) * H + h) * L + l) * 2 + k
