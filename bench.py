@@ -438,6 +438,85 @@ def run_reference_scenario(args, bk, dev):
     }
 
 
+def run_layout_change(args, bk, dev):
+    """Received token-major pages -> the Worker's per-layer paged pool and back, at the reference's own
+    shapes: token_shape (128, 2, 28, 2) fp16 (Model/qwen2.py:512-522), 28 layer tensors of
+    [10240*16, 2, 2, 128] (Worker.py:69-78), 4096 pages of 16 tokens per step and direction."""
+    import numpy as np
+    import torch
+    from oracle import pagecopy_oracle as oracle
+
+    P, D, H, L, blocks, n_pages = 16, 128, 2, 28, 10240, 4096
+    if args.pool_pages:
+        blocks = args.pool_pages
+        n_pages = min(n_pages, blocks)
+    layers = [torch.empty((blocks * P, 2, H, D), dtype=torch.float16, device=dev) for _ in range(L)]
+    for t in layers:
+        fill_random_bytes(t)
+    pool = bk.NHDPool.from_token_kv_layers(layers, P)
+    tm = torch.empty((n_pages, P, D, H, L, 2), dtype=torch.float16, device=dev)
+    fill_random_bytes(tm)
+    tm_out = torch.empty_like(tm)
+    rng = np.random.default_rng(6)
+    ids_h = rng.permutation(blocks)[:n_pages].astype(np.int64)
+    ids = torch.from_numpy(ids_h).to(dev)
+    alg = 2 * tm.numel() * 2                       # bytes read + written per launch
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        pool.load_token_major(tm, ids)             # received pages -> pool blocks
+        if ev:
+            ev[1].record()
+        pool.store_token_major(tm_out, ids)        # the same blocks -> pages to send
+        if ev:
+            ev[2].record()
+
+    for _ in range(args.warmup):
+        step()
+    pool.check()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(evs[k])
+    torch.cuda.synchronize(dev)
+    wall = time.perf_counter() - t0
+    pool.check()
+    if not torch.equal(tm_out.view(torch.int16), tm.view(torch.int16)):
+        raise SystemExit("bench: store(load(x)) != x")
+    # a sample of pages against the CPU oracle
+    sample = np.arange(0, n_pages, max(1, n_pages // 8))[:8]
+    lay_h = [np.zeros((blocks * P, 2, H, D), dtype=np.uint16) for _ in range(L)]
+    tm_h = tm[torch.from_numpy(sample).to(dev)].cpu().view(torch.int16).numpy().view(np.uint16)
+    oracle.transpose_pages_c(lay_h, "token_kv", np.ascontiguousarray(tm_h), ids_h[sample], np.arange(len(sample)), "load")
+    for l in (0, L // 2, L - 1):
+        for b in ids_h[sample]:
+            got = layers[l][b * P:(b + 1) * P].cpu().view(torch.int16).numpy().view(np.uint16)
+            if got.tobytes() != lay_h[l][b * P:(b + 1) * P].tobytes():
+                raise SystemExit("bench: layout change differs from the oracle")
+    l_ms = [e[0].elapsed_time(e[1]) for e in evs]
+    s_ms = [e[1].elapsed_time(e[2]) for e in evs]
+    slow_is_load = np.mean(l_ms) >= np.mean(s_ms)
+    ms_dom = float(np.mean(l_ms if slow_is_load else s_ms))
+    return {
+        "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
+        "value": round(2 * alg / (wall / args.steps) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u16", "data": "synthetic",
+        "config": {"workload": f"layout_change: token-major pages <-> {L} layer tensors [{blocks}*{P}, 2, {H}, {D}] fp16, "
+                               f"{n_pages} pages of {P} tokens loaded then stored per step"},
+        "pct_of_hbm_peak": round(100 * 2 * alg / (wall / args.steps) / 1e9 / HBM_PEAK_GBPS, 2),
+        "pages_per_s": round(2 * n_pages / (wall / args.steps), 1), "bit_exact": True,
+        "roofline": {"bound": "hbm", "kernel": f"bikv::transpose_pages_kernel<{1 if slow_is_load else 0}, 2>",
+                     "achieved": round(alg / (ms_dom * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(alg / (ms_dom * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "alg_bytes_per_launch": alg, "avg_launch_ms": round(ms_dom, 4)},
+        "kernels": {"load": {"GBps": round(alg / (np.mean(l_ms) * 1e-3) / 1e9, 1), "avg_ms": round(float(np.mean(l_ms)), 4)},
+                    "store": {"GBps": round(alg / (np.mean(s_ms) * 1e-3) / 1e9, 1), "avg_ms": round(float(np.mean(s_ms)), 4)}},
+    }
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -460,6 +539,10 @@ def main():
 
     if args.workload == "reference_200x50":
         out = run_reference_scenario(args, bk, dev)
+        print(json.dumps(out), flush=True)
+        return
+    if args.workload == "layout_change":
+        out = run_layout_change(args, bk, dev)
         print(json.dumps(out), flush=True)
         return
     out, shape, wl = run_gather_scatter(args, bk, workloads, dev)

@@ -148,6 +148,12 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
     t.log2_chunk = (int)value;
   } else if (!strcmp(key, "nontemporal")) {
     t.nontemporal = value < 0 ? -1 : (value ? 1 : 0);
+  } else if (!strcmp(key, "transpose_lds_kib")) {
+    if (value < 2 || value > 60) return fail(BIKV_EINVAL, "transpose_lds_kib must be in [2, 60]");
+    t.transpose_lds_kib = (int)value;
+  } else if (!strcmp(key, "transpose_dsplit")) {
+    if (value < 0 || value > 16 || (value & (value - 1))) return fail(BIKV_EINVAL, "transpose_dsplit must be 0 or a power of two <= 16");
+    t.transpose_dsplit = (int)value;
   } else if (!strcmp(key, "run_chunk_kib")) {
     if (value < 0 || value > 1 << 20) return fail(BIKV_EINVAL, "run_chunk_kib out of range");
     t.run_chunk_kib = (int)value;

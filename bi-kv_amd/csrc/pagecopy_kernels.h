@@ -51,6 +51,8 @@ struct Tuning {
   int unroll = 4;       // 16-byte vectors in flight per lane (1, 2, 4 or 8)
   int nontemporal = -1; // nt hint on payload loads and stores: 1 on, 0 off, -1 = chosen
   int run_chunk_kib = 0;  // bytes of a run handled by one workgroup, KiB; 0 = choose
+  int transpose_lds_kib = 60;  // LDS tile budget of the layout-change kernel, KiB
+  int transpose_dsplit = 0;    // slices of head_dim per tile; 0 = default (1: whole compute rows)
 };
 Tuning& tuning();
 
@@ -87,8 +89,8 @@ struct TransposeArgs {
   int64_t block_stride, kv_stride, token_stride;  // compute side, in elements
   int32_t n_layers, head_dim, n_cols;             // n_cols = kv_heads * n_layers * 2
   int32_t block_tokens, elem_bytes;
-  int32_t chunk_cols, pitch;      // filled by the launcher
-  uint32_t n_chunks, tile_words;
+  int32_t chunk_cols, chunk_rows, pitch;      // filled by the launcher
+  uint32_t n_chunks, n_dchunks, tile_words;
   uint32_t* status;
 };
 // dir 0: compute -> token-major, dir 1: token-major -> compute.
