@@ -425,7 +425,32 @@ def run_reference_scenario(args, bk, dev):
         raise SystemExit("bench: reference scenario mismatch")
     alg = 2 * cache.numel() * 2
     ms = e0.elapsed_time(e1) / args.steps
+    # the zero-copy form of the same scenario (test_zero_copy.py:40-56): the pool is pinned host memory
+    # and the kernel reads it over the host link; yardstick = a plain pinned H2D copy of the same bytes
+    pinned = torch.full((n * page_elements,), 7, dtype=torch.float16).pin_memory()
+    out.zero_()
+    bk.copy_runs(pinned, out, offs, offs, page_elements, device=dev)
+    out.copy_(pinned, non_blocking=True)
+    torch.cuda.synchronize(dev)
+    zc, h2d = [], []
+    for _ in range(max(3, args.steps // 4)):
+        e0.record()
+        bk.copy_runs(pinned, out, offs, offs, page_elements, device=dev)
+        e1.record()
+        torch.cuda.synchronize(dev)
+        zc.append(e0.elapsed_time(e1))
+        e0.record()
+        out.copy_(pinned, non_blocking=True)
+        e1.record()
+        torch.cuda.synchronize(dev)
+        h2d.append(e0.elapsed_time(e1))
+    if not torch.equal(out, cache):
+        raise SystemExit("bench: zero-copy scenario mismatch")
+    nbytes = cache.numel() * 2
+    zero_copy = {"GBps": round(nbytes / (min(zc) * 1e-3) / 1e9, 2),
+                 "plain_pinned_h2d_GBps": round(nbytes / (min(h2d) * 1e-3) / 1e9, 2)}
     return {
+        "zero_copy_from_pinned_host": zero_copy,
         "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
         "value": round(alg / (wall / args.steps) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True,

@@ -1,0 +1,70 @@
+"""The cache-side callers of the page copy, as functions.
+
+Mirrors of KVCache.shared_data_batch_pages (Bi-KV/DistributedStorage/kvcache.py:132-239) and
+KVCache.shared_data_batch_pages_cpu2gpu (kvcache.py:241-366): take the coordinator's
+`combined_task_info` (`id_token_pair` = [(item id, tokens)], `cache_pages_list` = [[page ids]]),
+turn the page lists into offset tables, and hand them to `ipc_service.producer_copy_pages` /
+`producer_zero_copy_pages`, which copy into the consumer's ring and publish the shape
+`[pages*page_size, head, kv_heads, layers, 2]`.
+
+Differences from the reference's methods, each for a stated reason:
+  * offsets are in ELEMENTS (the kernel's unit, copy_kernel.cu:22-33; the reference computes tokens,
+    kvcache.py:187-196, which the kernel would misread);
+  * the tables are built vectorised and uploaded once (the reference: two Python loops and two
+    `torch.tensor(list)` uploads per call);
+  * destination offsets are whole pages apart by default, matching the published shape. The
+    reference packs a partial last page tighter (kvcache.py:169-174) while still copying whole
+    pages, so consecutive destinations overlap and the result depends on execution order;
+    `pack_partial_pages=True` reproduces those offsets literally.
+"""
+from typing import Dict, Sequence, Tuple
+
+import torch
+
+import ipc_service
+
+from .offsets import build_run_offsets
+
+# the reference hard-codes these (kvcache.py:198-203, Model/qwen2.py:512-522)
+REFERENCE_DIMS = (128, 2, 28, 2)
+
+
+def _dims(n_pages: int, page_size: int, dims: Sequence[int]):
+    d = ipc_service.TensorDims()
+    d.total_tokens = n_pages * page_size
+    d.head_size, d.num_kv_heads, d.num_layers, d.kv_pair = (int(x) for x in dims)
+    return d
+
+
+def _tables(info: Dict, page_size: int, dims: Sequence[int], pack_partial_pages: bool, device):
+    pages_list = info["cache_pages_list"]
+    tokens = [int(p[1]) for p in info["id_token_pair"]]
+    ept = int(dims[0]) * int(dims[1]) * int(dims[2]) * int(dims[3])
+    off, _ = build_run_offsets(pages_list, tokens, page_size, elements_per_token=ept)
+    n = off.shape[1]
+    if not pack_partial_pages and n:
+        off[1] = range(0, n * page_size * ept, page_size * ept)
+    dev = torch.from_numpy(off).to(device) if n else torch.empty((2, 0), dtype=torch.int64, device=device)
+    return dev, n
+
+
+def shared_data_batch_pages(cuda_cache_data: torch.Tensor, combined_task_info: Dict, page_size: int,
+                            dims: Sequence[int] = REFERENCE_DIMS,
+                            pack_partial_pages: bool = False) -> Tuple[int, int]:
+    """Device pool -> consumer ring. Returns (pages copied, tokens published)."""
+    if not cuda_cache_data.is_cuda:
+        raise RuntimeError("Cache data must be on CUDA")
+    off, n = _tables(combined_task_info, page_size, dims, pack_partial_pages, cuda_cache_data.device)
+    ipc_service.producer_copy_pages(cuda_cache_data, off[0], off[1], page_size, _dims(n, page_size, dims))
+    return n, n * page_size
+
+
+def shared_data_batch_pages_cpu2gpu(cpu_cache_data: torch.Tensor, combined_task_info: Dict, page_size: int,
+                                    device, dims: Sequence[int] = REFERENCE_DIMS,
+                                    pack_partial_pages: bool = False) -> Tuple[int, int]:
+    """Pinned host pool -> consumer ring, the GPU reading host memory directly (kvcache.py:241-366)."""
+    if cpu_cache_data.is_cuda or not cpu_cache_data.is_pinned():
+        raise RuntimeError("CPU data must be pinned memory")
+    off, n = _tables(combined_task_info, page_size, dims, pack_partial_pages, torch.device(device))
+    ipc_service.producer_zero_copy_pages(cpu_cache_data, off[0], off[1], page_size, _dims(n, page_size, dims))
+    return n, n * page_size

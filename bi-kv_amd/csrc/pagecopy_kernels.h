@@ -18,7 +18,9 @@ struct TileClass {
   int64_t tile_bytes;
   int64_t page_stride;
   int32_t vec_width;              // widest power of two (<=16) dividing every address and size
-  int32_t log2_rows;              // fast mover only: tile_bytes == 4096 << log2_rows
+  int32_t log2_rows;              // segment mover: tile_bytes == 4096 << log2_rows; wave mover: pieces
+                                  // per tile == 1 << log2_rows, or -1 when that is not a power of two
+  uint32_t n_parts;               // wave mover: pieces per tile
   int32_t seg;                    // batch pages per workgroup
   uint32_t segs_per_plane;        // ceil(n_batch / seg)
   uint32_t n_blocks;              // plane_count * segs_per_plane

@@ -246,8 +246,11 @@ __device__ __forceinline__ void move_one(uint64_t pool, uint64_t stg) {
 template <int DIR, bool NT, int B>
 __global__ __launch_bounds__(B) void tile_move_wave_kernel(const MoveArgs a) {
   const uint32_t bx = blockIdx.x;
-  const uint32_t lp = (uint32_t)a.payload.log2_rows;
+  // pieces per tile: 2^lp when lp >= 0 (shift and mask), else n_parts (one uniform division per wave)
+  const int32_t lp = a.payload.log2_rows;
+  const uint32_t np = a.payload.n_parts;
   const bool payload = bx < a.payload.n_blocks;
+  const uint32_t bt = payload ? (lp >= 0 ? bx >> lp : bx / np) : 0u;   // x index without the piece
   // Two walks over the same (page, plane, piece) space, chosen by the launcher:
   //   order 0: x = (page, piece), y = plane — one plane at a time, pages in batch order
   //   order 1: x = (plane, page within a chunk of 2^lc pages, piece), (y, z) = chunk — the planes of
@@ -258,17 +261,17 @@ __global__ __launch_bounds__(B) void tile_move_wave_kernel(const MoveArgs a) {
   uint32_t i;
   if (a.order == 0) {
     q = a.plane_begin + (int64_t)blockIdx.y;
-    i = bx >> lp;
+    i = bt;
   } else {
     const uint64_t chunk = (uint64_t)blockIdx.y + (uint64_t)blockIdx.z * gridDim.y;
-    const uint32_t t = (payload ? bx : 0u) >> lp;
+    const uint32_t t = bt;
     const uint64_t page = (chunk << lc) + (t & ((1u << lc) - 1u));
     if (page >= (uint64_t)a.n_batch) return;
     i = (uint32_t)page;
     q = a.plane_begin + (int64_t)(t >> lc);
   }
   if (payload) {
-    const uint32_t part = bx & ((1u << lp) - 1u);
+    const uint32_t part = lp >= 0 ? (bx & ((1u << lp) - 1u)) : bx - bt * np;
     const int64_t pid = cload(a.page_ids + i);
     const int64_t slot = cload(a.slots + i) + q * cload(a.slot_strides + i) - a.slot_bias;
     const uint64_t plane = (uint64_t)cload(a.payload.plane_base + q);  // issued with the others
@@ -284,7 +287,8 @@ __global__ __launch_bounds__(B) void tile_move_wave_kernel(const MoveArgs a) {
     const uint64_t pool = plane + (uint64_t)(pid * a.payload.page_stride);
     const uint64_t stg = (uint64_t)a.payload.staging + (uint64_t)(slot * a.payload.tile_bytes);
     const uint64_t off = (uint64_t)part * (B * 16u) + threadIdx.x * 16u;
-    st<NT, u32x4>((DIR == 0 ? stg : pool) + off, ld<NT, u32x4>((DIR == 0 ? pool : stg) + off));
+    if (off < (uint64_t)a.payload.tile_bytes)   // the last piece of a tile may be ragged
+      st<NT, u32x4>((DIR == 0 ? stg : pool) + off, ld<NT, u32x4>((DIR == 0 ? pool : stg) + off));
   } else {
     // scale class: one lane per vector; order 0 spreads the lanes over the pages of plane q,
     // order 1 over the planes of page i. The launcher keeps (scale workgroups * B) below 2^32.
@@ -372,20 +376,24 @@ static hipError_t launch_wave(const MoveArgs& a, int block, bool nt, dim3 grid, 
   }
 }
 
-// The wave mover takes a payload whose tiles are 2^k pieces of block*16 bytes, all 16-byte aligned.
-// Returns false when the shape does not qualify (the segment movers take it then).
+// The wave mover takes any payload made of 16-byte aligned tiles of at least half a piece
+// (piece = block*16 bytes); smaller or misaligned tiles go to the segment movers.
+// Returns false when the shape does not qualify.
 static bool plan_wave(MoveArgs& a, int block, int order, int log2_chunk, dim3* grid) {
   const int64_t piece = (int64_t)block * 16;
   TileClass& p = a.payload;
-  if (p.vec_width != 16 || p.tile_bytes % piece != 0) return false;
-  const int64_t parts = p.tile_bytes / piece;
-  if ((parts & (parts - 1)) != 0) return false;
-  int lp = 0;
-  while ((int64_t(1) << lp) < parts) ++lp;
+  if (p.vec_width != 16 || p.tile_bytes % 16 != 0 || p.tile_bytes * 2 < piece) return false;
+  const int64_t parts = (p.tile_bytes + piece - 1) / piece;
+  if (parts >= (int64_t(1) << 31)) return false;
+  int lp = -1;
+  if ((parts & (parts - 1)) == 0) {
+    lp = 0;
+    while ((int64_t(1) << lp) < parts) ++lp;
+  }
   // order 0: x walks the batch pages of one plane; order 1: x walks the planes of one page
   if (order == 0) log2_chunk = 0;
   const int64_t walk = order == 0 ? a.n_batch : ((int64_t)a.plane_count << log2_chunk);
-  const int64_t px = walk << lp;
+  const int64_t px = walk * parts;
   int64_t sx = 0;
   if (a.scale.tile_bytes > 0) {
     const int64_t vpt = a.scale.tile_bytes / a.scale.vec_width;
@@ -405,6 +413,7 @@ static bool plan_wave(MoveArgs& a, int block, int order, int log2_chunk, dim3* g
     *grid = dim3((uint32_t)(px + sx), (uint32_t)gy, (uint32_t)gz);
   }
   p.log2_rows = lp;
+  p.n_parts = (uint32_t)parts;
   p.n_blocks = (uint32_t)px;
   a.scale.n_blocks = (uint32_t)sx;
   a.order = order;

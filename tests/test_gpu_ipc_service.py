@@ -185,3 +185,40 @@ def test_error_paths(ipc, cuda):
         ipc.consumer_receive(timeout_ms=50)
     ipc.consumer_cleanup()
     assert not os.path.exists("/dev/shm" + name)        # the consumer unlinks its object
+
+
+@pytest.mark.parametrize("pinned_host_pool", [False, True])
+def test_cache_side_callers_from_task_info(ipc, oracle, cuda, pinned_host_pool):
+    """KVCache.shared_data_batch_pages / _cpu2gpu (kvcache.py:132-366) as functions: the coordinator's
+    task info in, pages in the consumer's ring out."""
+    from bikv_pagecopy import kvcache_calls
+    print(f"[case] cache-side callers, pinned host pool={pinned_host_pool}", flush=True)
+    name = f"/bikv_test_callers_{os.getpid()}"
+    dims, page_size, pool_pages = (64, 2, 3, 2), 16, 50
+    ept = dims[0] * dims[1] * dims[2] * dims[3]
+    page_elems = page_size * ept
+    ipc.consumer_init(0, name, 64 << 20)
+    ipc.producer_init(0, name)
+    rng = np.random.default_rng(23)
+    pool_h = rng.integers(0, 65536, size=pool_pages * page_elems, dtype=np.uint16)
+    pool_t = torch.from_numpy(pool_h.view(np.int16)).view(torch.float16)
+    pool_t = pool_t.pin_memory() if pinned_host_pool else pool_t.to(cuda)
+    info = {"infer_worker": 0, "token_num": 40 + 16 + 33,
+            "id_token_pair": [(11, 40), (12, 16), (13, 33)],            # 3, 1 and 3 pages of 16 tokens
+            "cache_pages_list": [[7, 2, 49], [4], [30, 31, 0]]}
+    if pinned_host_pool:
+        n, tokens = kvcache_calls.shared_data_batch_pages_cpu2gpu(pool_t, info, page_size, cuda, dims)
+    else:
+        n, tokens = kvcache_calls.shared_data_batch_pages(pool_t, info, page_size, dims)
+    assert (n, tokens) == (7, 7 * page_size)
+    got = ipc.consumer_receive(timeout_ms=5000)
+    assert tuple(got.shape) == (7 * page_size,) + dims
+    pages = np.array([7, 2, 49, 4, 30, 31, 0])
+    want = np.zeros(7 * page_elems, dtype=np.uint16)
+    oracle.copy_runs_c(pool_h, want, pages * page_elems, np.arange(7) * page_elems, page_elems)
+    assert got.cpu().contiguous().view(torch.int16).numpy().tobytes() == want.tobytes()
+    # the reference's literal (packed) destination offsets, for the record
+    so, do, total = oracle.build_offsets_loops(info["cache_pages_list"], info["id_token_pair"], page_size, ept)
+    assert total == 89 and do[3] == 40 * ept and so[2] == 49 * page_elems
+    with pytest.raises(RuntimeError):
+        kvcache_calls.shared_data_batch_pages(pool_t.cpu() if not pinned_host_pool else pool_t, info, page_size, dims)

@@ -155,6 +155,37 @@ def test_odd_tile_sizes(bk, oracle, cuda, tile_bytes):
     assert _to_np(staging).tobytes() == oracle.gather_layered_c(pool_h, reqs).tobytes()
 
 
+@pytest.mark.parametrize("tile_bytes", [24576, 40960, 1536, 528, 1008, 4096 + 16, 3 * 1024, 7 * 1024 + 512])
+@pytest.mark.parametrize("order", [0, 1])
+def test_wave_mover_with_piece_counts_that_are_not_powers_of_two(bk, oracle, cuda, tile_bytes, order):
+    """6 KV heads give 24 KiB tiles (24 pieces of 1 KiB); other sizes end in a ragged piece."""
+    _announce(f"wave mover tile {tile_bytes} order {order}")
+    rng = np.random.default_rng(tile_bytes + order)
+    pool_h = _rand_pool(rng, 5, 40, tile_bytes)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    reqs = [rng.permutation(40)[:13], np.array([7, 7]), rng.permutation(40)[:1]]
+    try:
+        bk.set_tuning(order=order, log2_chunk=2 if order else -1)
+        for layout in ("layer_major", "page_major"):
+            batch = pool.make_batch(reqs, layout)
+            st = torch.full((batch.n_slots * tile_bytes + 32,), 0xA5, dtype=torch.uint8, device=cuda)
+            pool.gather(batch, st[: batch.n_slots * tile_bytes])
+            pool.check()
+            assert _to_np(st[: batch.n_slots * tile_bytes]).tobytes() == oracle.gather_layered_c(pool_h, reqs, layout).tobytes()
+            assert torch.all(st[batch.n_slots * tile_bytes:] == 0xA5)      # nothing past the last ragged piece
+        perm = rng.permutation(40)
+        sreqs = [perm[:9], perm[9:12]]
+        sb = pool.make_batch(sreqs)
+        src = torch.from_numpy(rng.integers(0, 256, size=sb.n_slots * tile_bytes, dtype=np.uint8)).to(cuda)
+        pool.scatter(sb, src)
+        pool.check()
+        oracle.scatter_layered_c(pool_h, sreqs, src.cpu().numpy())
+        assert _to_np(pool_d).tobytes() == pool_h.tobytes()
+    finally:
+        bk.set_tuning(order=-1, log2_chunk=-1)
+
+
 def test_misaligned_pool_and_staging(bk, oracle, cuda):
     """Pool planes and staging that start 2 bytes off a 16-byte boundary take the narrow mover."""
     _announce("misaligned")
