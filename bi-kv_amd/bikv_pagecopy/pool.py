@@ -242,6 +242,7 @@ class PagedKVPool:
         if getattr(self, "_h", None):
             _lib.load().bikv_pool_destroy(self._h)
             self._h = None
+        self._keepalive = None
 
     def __del__(self):
         try:
