@@ -48,6 +48,8 @@ def parse_args():
     ap.add_argument("--no-other-layout", dest="no_other_layout", action="store_true",
                     help="skip the second measurement with the other staging layout")
     ap.add_argument("--pool-pages", type=int, default=0, help="override the pool size (pages per plane)")
+    ap.add_argument("--pool-alloc", choices=["planes", "stacked"], default="stacked",
+                    help="one device tensor per (layer, K|V) plane, or one stacked allocation")
     ap.add_argument("--seg", type=int, default=None)
     ap.add_argument("--unroll", type=int, default=None)
     ap.add_argument("--nontemporal", type=int, default=None)
@@ -74,27 +76,35 @@ def fill_random_bytes(t):
         flat[off: off + step].random_(0, 256)
 
 
-def make_pool(shape, dev):
+def make_pool(shape, dev, alloc="planes"):
+    """The pool as the serving engine holds it: one tensor per (layer, K|V) plane ("planes", as
+    Bi-KV/Worker/Worker.py:74-78 keeps a list of per-layer caches), or one stacked allocation
+    ("stacked"). Returns (planes, scale planes or None); both index as planes[q] -> [n_pages, tile]."""
     import torch
-    pool = torch.empty((shape.n_planes, shape.n_pages, shape.tile_bytes), dtype=torch.uint8, device=dev)
-    fill_random_bytes(pool)
-    scale = None
-    if shape.scales:
-        scale = torch.empty((shape.n_planes, shape.n_pages, shape.scale_tile_bytes), dtype=torch.uint8, device=dev)
-        fill_random_bytes(scale)
-    return pool, scale
+
+    def one(tile_bytes):
+        if alloc == "stacked":
+            t = torch.empty((shape.n_planes, shape.n_pages, tile_bytes), dtype=torch.uint8, device=dev)
+            fill_random_bytes(t)
+            return [t[q] for q in range(shape.n_planes)]
+        out = [torch.empty((shape.n_pages, tile_bytes), dtype=torch.uint8, device=dev) for _ in range(shape.n_planes)]
+        for t in out:
+            fill_random_bytes(t)
+        return out
+
+    return one(shape.tile_bytes), (one(shape.scale_tile_bytes) if shape.scales else None)
 
 
 def verify_on_device(pool_t, staging, batch, requests, n_check_planes=3):
     """Independent check at full size: torch.index_select on the device, a few planes per request."""
     import torch
-    n_planes = pool_t.shape[0]
+    n_planes = len(pool_t)
     planes = sorted({0, n_planes // 2, n_planes - 1})[:n_check_planes]
     for r, ids in enumerate(requests):
         if len(ids) == 0:
             continue
         view = batch.request_view(staging, r)
-        idt = torch.from_numpy(ids).to(pool_t.device)
+        idt = torch.from_numpy(ids).to(pool_t[0].device)
         for q in planes:
             want = torch.index_select(pool_t[q], 0, idt)
             got = view[q] if batch.layout == "layer_major" else view[:, q]
@@ -200,8 +210,8 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True):
         shape = shape.scaled(args.pool_pages)
     wl = workloads.named(name, shape)
     log(f"{name}: pool {shape.pool_bytes / 1e9:.2f} GB, tile {shape.tile_bytes} B x {shape.n_planes} planes")
-    pool_t, scale_t = make_pool(shape, dev)
-    pool = bk.PagedKVPool.from_stacked(pool_t, plane_dims=1, scale=scale_t)
+    pool_t, scale_t = make_pool(shape, dev, args.pool_alloc)
+    pool = bk.PagedKVPool.from_planes(pool_t, scale_t)
 
     g_reqs = wl["gather"]
     s_reqs = wl.get("scatter") or []
@@ -324,7 +334,7 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True):
                                f"scatter requests, {n_pages} pages/step in {len(g_groups)}+{len(s_groups)} launches, "
                                f"layout {args.layout}",
                    "pool_GB": round(shape.pool_bytes / 1e9, 2), "tile_bytes": shape.tile_bytes,
-                   "planes": shape.n_planes},
+                   "planes": shape.n_planes, "pool_alloc": args.pool_alloc},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "pages_per_s": round(n_pages / (wall / args.steps), 1),
         "bit_exact": True,
@@ -352,8 +362,8 @@ def run_staging(args, bk, workloads, dev):
     if args.pool_pages:
         shape = shape.scaled(args.pool_pages)
     wl = workloads.named("llama3_8b", shape)
-    pool_t, _ = make_pool(shape, dev)
-    pool = bk.PagedKVPool.from_stacked(pool_t, plane_dims=1)
+    pool_t, _ = make_pool(shape, dev, args.pool_alloc)
+    pool = bk.PagedKVPool.from_planes(pool_t)
     reqs = wl["gather"]
     max_pages = max(len(r) for r in reqs)
     host = bk.pinned_empty(max_pages * shape.page_bytes)
