@@ -379,6 +379,10 @@ def run_staging(args, bk, workloads, dev):
     for _ in range(4):
         link.append(dev_buf.numel() / bk.measure_d2h(dev, host, dev_buf, 0) / 1e9)
     link_gbps = max(link[1:])
+    up = []
+    for _ in range(4):
+        up.append(dev_buf.numel() / bk.measure_h2d(dev, dev_buf, host, 0) / 1e9)
+    up_gbps = max(up[1:])
     results = {}
     for mode in ("pipelined", "direct"):
         stager = bk.HostStager(dev, chunk_bytes=args.chunk_mib << 20, n_buffers=args.buffers)
@@ -406,8 +410,31 @@ def run_staging(args, bk, workloads, dev):
             raise SystemExit(f"bench: staged bytes differ ({mode})")
         results[mode] = {"host_link_GBps": round(tot_b / tot_s / 1e9, 2), "bytes": tot_b, "chunks": chunks,
                          "frac_of_plain_d2h": round(tot_b / tot_s / 1e9 / link_gbps, 4)}
+        # the receiving side: the staged image of a request goes host -> pool, into the pages next to
+        # the ones it came from (a different, still unique id set)
+        rx_b, rx_s = 0, 0.0
+        rx = [(b_, r_) for b_, r_ in zip(batches, reqs) if len(np.unique(r_)) == len(r_)][: max(1, args.steps)]
+        for b_, r_ in rx:
+            stager.gather_to_host(pool, b_, host, mode)
+            shifted = (np.asarray(r_) + 1) % shape.n_pages
+            sb = pool.make_batch([shifted], args.layout)
+            nb, _, sec = stager.scatter_from_host(pool, sb, host, mode)
+            rx_b += nb
+            rx_s += sec
+        if rx:
+            idt = torch.from_numpy(shifted).to(dev)
+            view = host[: sb.n_slots * shape.tile_bytes].view(sb.n_slots, shape.tile_bytes)
+            for q in (0, shape.n_planes - 1):
+                got = torch.index_select(pool_t[q], 0, idt).cpu()
+                want = (view[q * len(shifted): (q + 1) * len(shifted)] if args.layout == "layer_major"
+                        else view[q::shape.n_planes])
+                if not torch.equal(got, want):
+                    raise SystemExit(f"bench: scattered bytes differ ({mode})")
+            results[mode]["scatter_from_host_GBps"] = round(rx_b / rx_s / 1e9, 2)
+            results[mode]["scatter_frac_of_plain_h2d"] = round(rx_b / rx_s / 1e9 / up_gbps, 4)
         stager.close()
-    return {"plain_d2h_GBps": round(link_gbps, 2), "chunk_MiB": args.chunk_mib, "buffers": args.buffers,
+    return {"plain_d2h_GBps": round(link_gbps, 2), "plain_h2d_GBps": round(up_gbps, 2),
+            "chunk_MiB": args.chunk_mib, "buffers": args.buffers,
             "requests": min(len(reqs), max(1, args.steps)), **results}
 
 

@@ -119,6 +119,9 @@ _SIGNATURES = {
     "bikv_gather_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PageBatchDesc),
                                       C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_void_p,
                                       C.c_int64, C.c_void_p, C.c_int64, C.c_int32, C.POINTER(StageStats)]),
+    "bikv_scatter_from_host": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PageBatchDesc),
+                                         C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_void_p,
+                                         C.c_int64, C.c_void_p, C.c_int64, C.c_int32, C.POINTER(StageStats)]),
     "bikv_nhd_create": (C.c_int, [C.POINTER(NHDDesc), C.POINTER(C.c_void_p)]),
     "bikv_nhd_destroy": (C.c_int, [C.c_void_p]),
     "bikv_nhd_load_token_major": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
@@ -128,6 +131,8 @@ _SIGNATURES = {
     "bikv_plan_chunks": (C.c_int64, [C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_int32, C.c_int64,
                                      C.POINTER(C.c_int64), C.c_int64]),
     "bikv_d2h_copy": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
+                                C.POINTER(C.c_double)]),
+    "bikv_h2d_copy": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
                                 C.POINTER(C.c_double)]),
     "bikv_host_alloc": (C.c_int, [C.c_int64, C.POINTER(C.c_void_p)]),
     "bikv_host_free": (C.c_int, [C.c_void_p]),

@@ -34,10 +34,7 @@ class HostStager:
         _lib.check(_lib.load().bikv_stager_create(idx, self.chunk_bytes, self.n_buffers, C.byref(h)))
         self._h = h
 
-    def gather_to_host(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "pipelined",
-                       host_scale: torch.Tensor = None):
-        """Fills `host` (pinned) with the staging image of `batch` (and `host_scale` with the scale
-        image of an fp8 pool); returns (bytes, chunks, seconds)."""
+    def _stage(self, entry: str, pool: PagedKVPool, batch: PageBatch, host, mode, host_scale):
         if mode not in _MODES:
             raise ValueError(f"unknown mode {mode!r}")
         for t in (host, host_scale):
@@ -54,13 +51,25 @@ class HostStager:
         d = batch.desc()
         stats = _lib.StageStats()
         rp = batch.req_pages.ctypes.data_as(C.POINTER(C.c_int64))
-        _lib.check(_lib.load().bikv_gather_to_host(
+        _lib.check(getattr(_lib.load(), entry)(
             self._h, pool._h, C.byref(d), rp, len(batch.req_pages), _LAYOUT_CODE[batch.layout],
             host.data_ptr(), host.numel() * host.element_size(),
             host_scale.data_ptr() if host_scale is not None else None,
             host_scale.numel() * host_scale.element_size() if host_scale is not None else 0,
             _MODES[mode], C.byref(stats)))
         return stats.bytes, stats.n_chunks, stats.wall_seconds
+
+    def gather_to_host(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "pipelined",
+                       host_scale: torch.Tensor = None):
+        """Fills `host` (pinned) with the staging image of `batch` (and `host_scale` with the scale
+        image of an fp8 pool); returns (bytes, chunks, seconds)."""
+        return self._stage("bikv_gather_to_host", pool, batch, host, mode, host_scale)
+
+    def scatter_from_host(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "pipelined",
+                          host_scale: torch.Tensor = None):
+        """Writes the staging image held in `host` (pinned; `host_scale` for an fp8 pool) into the
+        pool pages `batch` names (unique ids); returns (bytes, chunks, seconds)."""
+        return self._stage("bikv_scatter_from_host", pool, batch, host, mode, host_scale)
 
     def close(self):
         if getattr(self, "_h", None):
@@ -94,4 +103,14 @@ def measure_d2h(device, host: torch.Tensor, dev: torch.Tensor, chunk_bytes: int 
     sec = C.c_double()
     torch.cuda.synchronize(device)
     _lib.check(_lib.load().bikv_d2h_copy(idx, host.data_ptr(), dev.data_ptr(), nbytes, chunk_bytes, C.byref(sec)))
+    return sec.value
+
+
+def measure_h2d(device, dev: torch.Tensor, host: torch.Tensor, chunk_bytes: int = 0) -> float:
+    """Seconds for a plain hipMemcpyAsync of host (pinned) -> dev."""
+    idx = torch.device(device).index or 0
+    nbytes = min(host.numel() * host.element_size(), dev.numel() * dev.element_size())
+    sec = C.c_double()
+    torch.cuda.synchronize(device)
+    _lib.check(_lib.load().bikv_h2d_copy(idx, dev.data_ptr(), host.data_ptr(), nbytes, chunk_bytes, C.byref(sec)))
     return sec.value

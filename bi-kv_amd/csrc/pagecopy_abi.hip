@@ -350,9 +350,9 @@ extern "C" int bikv_host_free(void* p) {
   return BIKV_OK;
 }
 
-extern "C" int bikv_d2h_copy(int device, void* host_dst, const void* dev_src, int64_t bytes,
-                             int64_t chunk_bytes, double* seconds_out) {
-  if (!host_dst || !dev_src || bytes <= 0) return fail(BIKV_EINVAL, "bad d2h_copy arguments");
+static int link_copy(int device, void* dst, const void* src, int64_t bytes, int64_t chunk_bytes,
+                     hipMemcpyKind kind, double* seconds_out) {
+  if (!dst || !src || bytes <= 0) return fail(BIKV_EINVAL, "bad host-link copy arguments");
   BIKV_HIP(hipSetDevice(device));
   hipStream_t s;
   BIKV_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
@@ -361,15 +361,25 @@ extern "C" int bikv_d2h_copy(int device, void* host_dst, const void* dev_src, in
   hipError_t e = hipSuccess;
   for (int64_t off = 0; off < bytes && e == hipSuccess; off += chunk_bytes) {
     const int64_t n = bytes - off < chunk_bytes ? bytes - off : chunk_bytes;
-    e = hipMemcpyAsync(static_cast<char*>(host_dst) + off, static_cast<const char*>(dev_src) + off,
-                       (size_t)n, hipMemcpyDeviceToHost, s);
+    e = hipMemcpyAsync(static_cast<char*>(dst) + off, static_cast<const char*>(src) + off,
+                       (size_t)n, kind, s);
   }
   if (e == hipSuccess) e = hipStreamSynchronize(s);
   const auto t1 = std::chrono::steady_clock::now();
   (void)hipStreamDestroy(s);
-  if (e != hipSuccess) return fail_hip(e, "hipMemcpyAsync(D2H)");
+  if (e != hipSuccess) return fail_hip(e, "hipMemcpyAsync(host link)");
   if (seconds_out) *seconds_out = std::chrono::duration<double>(t1 - t0).count();
   return BIKV_OK;
+}
+
+extern "C" int bikv_d2h_copy(int device, void* host_dst, const void* dev_src, int64_t bytes,
+                             int64_t chunk_bytes, double* seconds_out) {
+  return link_copy(device, host_dst, dev_src, bytes, chunk_bytes, hipMemcpyDeviceToHost, seconds_out);
+}
+
+extern "C" int bikv_h2d_copy(int device, void* dev_dst, const void* host_src, int64_t bytes,
+                             int64_t chunk_bytes, double* seconds_out) {
+  return link_copy(device, dev_dst, host_src, bytes, chunk_bytes, hipMemcpyHostToDevice, seconds_out);
 }
 
 // ---- device -> pinned-host staging pipeline -----------------------------------------------
@@ -512,17 +522,20 @@ extern "C" int64_t bikv_plan_chunks(const int64_t* req_pages, int64_t n_requests
   return (int64_t)chunks.size();
 }
 
-extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
-                                   const bikv_page_batch* batch, const int64_t* req_pages,
-                                   int64_t n_requests, int32_t layout, void* host_dst,
-                                   int64_t host_bytes, void* host_scale_dst,
-                                   int64_t host_scale_bytes, int32_t mode,
-                                   bikv_stage_stats* stats) {
+// Both directions of the host staging pipeline. dir 0: pool -> device chunk -> host image;
+// dir 1: host image -> device chunk -> pool. A lane's stream orders the two steps of a chunk and
+// keeps its chunk buffer safe from the lane's next chunk.
+static int stage_between_host(int dir, bikv_stager* st, const bikv_pool* pool,
+                              const bikv_page_batch* batch, const int64_t* req_pages,
+                              int64_t n_requests, int32_t layout, void* host_dst,
+                              int64_t host_bytes, void* host_scale_dst,
+                              int64_t host_scale_bytes, int32_t mode,
+                              bikv_stage_stats* stats) {
   if (!st || !pool || !batch || !req_pages || !host_dst)
     return fail(BIKV_EINVAL, "null argument");
   const bool has_scale = pool->scale_tile_bytes > 0;
   if (has_scale && !host_scale_dst)
-    return fail(BIKV_EINVAL, "pool has a scale class: host_scale_dst must be given");
+    return fail(BIKV_EINVAL, "pool has a scale class: the host scale image must be given");
   if (pool->device != st->device) return fail(BIKV_EINVAL, "pool and stager are on different devices");
   if (layout != BIKV_LAYOUT_LAYER_MAJOR && layout != BIKV_LAYOUT_PAGE_MAJOR)
     return fail(BIKV_EINVAL, "unknown layout %d", layout);
@@ -557,7 +570,9 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
     void* sptr = nullptr;
     BIKV_HIP(hipHostGetDevicePointer(&dptr, host_dst, 0));
     if (has_scale) BIKV_HIP(hipHostGetDevicePointer(&sptr, host_scale_dst, 0));
-    int rc = bikv_gather_pages(pool, batch, dptr, image_bytes, sptr, scale_image_bytes, st->lanes[0]);
+    int rc = dir == 0
+        ? bikv_gather_pages(pool, batch, dptr, image_bytes, sptr, scale_image_bytes, st->lanes[0])
+        : bikv_scatter_pages(pool, batch, dptr, image_bytes, sptr, scale_image_bytes, st->lanes[0]);
     if (rc) return rc;
     rc = sync_and_check(st->device, st->lanes[0]);
     if (rc) return rc;
@@ -598,17 +613,32 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
       sub.plane_begin = ch.plane_begin;
       sub.plane_count = ch.plane_count;
       sub.slot_bias = ch.first_slot;
-      // stream order on the lane keeps the buffer safe: this gather runs after the lane's previous copy
-      rc = bikv_gather_pages(pool, &sub, dev_chunk, ch.n_slots * T, dev_scale, ch.n_slots * S,
-                             st->lanes[lane]);
-      if (rc) break;
-      e = hipMemcpyAsync(static_cast<char*>(host_dst) + ch.first_slot * T, dev_chunk,
-                         (size_t)(ch.n_slots * T), hipMemcpyDeviceToHost, st->lanes[lane]);
-      if (e != hipSuccess) break;
-      if (has_scale) {
-        e = hipMemcpyAsync(static_cast<char*>(host_scale_dst) + ch.first_slot * S, dev_scale,
-                           (size_t)(ch.n_slots * S), hipMemcpyDeviceToHost, st->lanes[lane]);
+      char* host_chunk = static_cast<char*>(host_dst) + ch.first_slot * T;
+      char* host_scale_chunk = has_scale ? static_cast<char*>(host_scale_dst) + ch.first_slot * S : nullptr;
+      if (dir == 0) {
+        rc = bikv_gather_pages(pool, &sub, dev_chunk, ch.n_slots * T, dev_scale, ch.n_slots * S,
+                               st->lanes[lane]);
+        if (rc) break;
+        e = hipMemcpyAsync(host_chunk, dev_chunk, (size_t)(ch.n_slots * T), hipMemcpyDeviceToHost,
+                           st->lanes[lane]);
         if (e != hipSuccess) break;
+        if (has_scale) {
+          e = hipMemcpyAsync(host_scale_chunk, dev_scale, (size_t)(ch.n_slots * S),
+                             hipMemcpyDeviceToHost, st->lanes[lane]);
+          if (e != hipSuccess) break;
+        }
+      } else {
+        e = hipMemcpyAsync(dev_chunk, host_chunk, (size_t)(ch.n_slots * T), hipMemcpyHostToDevice,
+                           st->lanes[lane]);
+        if (e != hipSuccess) break;
+        if (has_scale) {
+          e = hipMemcpyAsync(dev_scale, host_scale_chunk, (size_t)(ch.n_slots * S),
+                             hipMemcpyHostToDevice, st->lanes[lane]);
+          if (e != hipSuccess) break;
+        }
+        rc = bikv_scatter_pages(pool, &sub, dev_chunk, ch.n_slots * T, dev_scale, ch.n_slots * S,
+                                st->lanes[lane]);
+        if (rc) break;
       }
     }
     // Drain every lane whatever happened, so that no work is left in flight on an error path.
@@ -632,6 +662,27 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
     stats->wall_seconds = std::chrono::duration<double>(t1 - t0).count();
   }
   return BIKV_OK;
+}
+
+extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
+                                   const bikv_page_batch* batch, const int64_t* req_pages,
+                                   int64_t n_requests, int32_t layout, void* host_dst,
+                                   int64_t host_bytes, void* host_scale_dst,
+                                   int64_t host_scale_bytes, int32_t mode,
+                                   bikv_stage_stats* stats) {
+  return stage_between_host(0, st, pool, batch, req_pages, n_requests, layout, host_dst, host_bytes,
+                            host_scale_dst, host_scale_bytes, mode, stats);
+}
+
+extern "C" int bikv_scatter_from_host(bikv_stager* st, const bikv_pool* pool,
+                                      const bikv_page_batch* batch, const int64_t* req_pages,
+                                      int64_t n_requests, int32_t layout, const void* host_src,
+                                      int64_t host_bytes, const void* host_scale_src,
+                                      int64_t host_scale_bytes, int32_t mode,
+                                      bikv_stage_stats* stats) {
+  return stage_between_host(1, st, pool, batch, req_pages, n_requests, layout,
+                            const_cast<void*>(host_src), host_bytes,
+                            const_cast<void*>(host_scale_src), host_scale_bytes, mode, stats);
 }
 
 // ---- per-layer paged NHD pool and the fused layout change ------------------------------------

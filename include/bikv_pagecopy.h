@@ -193,7 +193,19 @@ int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool, const bikv_page_
                         int64_t host_scale_bytes, int32_t mode,
                         bikv_stage_stats* stats /* nullable */);
 
-/* The chunk plan bikv_gather_to_host would use, without touching a GPU: writes up to `cap` chunks
+/* The receiving side: the transport has landed a staging image (same layout as above) in pinned
+ * host memory (the reference holds received KV in host tensors, Worker.py:166-169, and reads a
+ * pinned host pool from the GPU in kvcache.py:241-366); chunk c is copied host -> HBM chunk buffer
+ * and scattered from there into the pool on lane c % n_buffers. BIKV_STAGE_DIRECT lets the scatter
+ * kernel read the mapped pinned image itself. Page ids must be unique (a scatter). Synchronous. */
+int bikv_scatter_from_host(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
+                           const int64_t* req_pages, int64_t n_requests, int32_t layout,
+                           const void* host_src, int64_t host_bytes,
+                           const void* host_scale_src /* pinned; NULL iff no scale class */,
+                           int64_t host_scale_bytes, int32_t mode,
+                           bikv_stage_stats* stats /* nullable */);
+
+/* The chunk plan bikv_gather_to_host and bikv_scatter_from_host would use, without touching a GPU: writes up to `cap` chunks
  * as 6 int64 each (first_page, n_pages, plane_begin, plane_count, first_slot, n_slots) into `out`
  * and returns the total number of chunks (which may exceed cap), or a negative code. */
 int64_t bikv_plan_chunks(const int64_t* req_pages, int64_t n_requests, int32_t n_planes,
@@ -201,6 +213,8 @@ int64_t bikv_plan_chunks(const int64_t* req_pages, int64_t n_requests, int32_t n
 
 /* Plain pinned-buffer copy, for measuring the host link on the same box. Synchronous. */
 int bikv_d2h_copy(int device, void* host_dst, const void* dev_src, int64_t bytes,
+                  int64_t chunk_bytes /* 0 = one copy */, double* seconds_out);
+int bikv_h2d_copy(int device, void* dev_dst, const void* host_src, int64_t bytes,
                   int64_t chunk_bytes /* 0 = one copy */, double* seconds_out);
 
 /* Pinned host memory (hipHostMalloc, mapped + portable). */
