@@ -108,6 +108,11 @@ _SIGNATURES = {
     "bikv_set_tuning": (C.c_int, [C.c_char_p, C.c_int64]),
     "bikv_copy_runs": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
                                  C.c_int64, C.c_int64, C.c_int64, C.c_void_p]),
+    "bikv_copy_runs_ragged": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
+                                        C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p]),
+    "bikv_producer_copy_tokens": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                            C.c_int64, C.c_int64, C.c_int64, C.POINTER(TensorDimsC),
+                                            C.c_int64, C.c_int32, C.c_void_p]),
     "bikv_pool_create": (C.c_int, [C.POINTER(PoolDesc), C.POINTER(C.c_void_p)]),
     "bikv_pool_destroy": (C.c_int, [C.c_void_p]),
     "bikv_gather_pages": (C.c_int, [C.c_void_p, C.POINTER(PageBatchDesc), C.c_void_p, C.c_int64,

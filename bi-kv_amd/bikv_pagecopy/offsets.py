@@ -22,9 +22,11 @@ import numpy as np
 
 def build_run_offsets(cache_pages_list: Sequence[Sequence[int]], item_tokens: Sequence[int],
                       page_size: int, elements_per_token: int = 1,
-                      unit: str = "elements") -> Tuple[np.ndarray, int]:
+                      unit: str = "elements", with_sizes: bool = False) -> Tuple[np.ndarray, int]:
     """Returns (offsets, total_tokens): offsets[0] = source offsets, offsets[1] = destination offsets,
-    both int64, one entry per page in list order; total_tokens = sum of the copied page sizes."""
+    both int64, one entry per page in list order; total_tokens = sum of the copied page sizes.
+    with_sizes=True adds a third row, the tokens each run holds (page_size, or the tail of an item's
+    partial last page): the run lengths a packed destination needs (always in tokens)."""
     if unit not in ("elements", "tokens"):
         raise ValueError("unit must be 'elements' or 'tokens'")
     if page_size <= 0:
@@ -33,7 +35,7 @@ def build_run_offsets(cache_pages_list: Sequence[Sequence[int]], item_tokens: Se
         raise ValueError("cache_pages_list and item_tokens differ in length")
     counts = np.fromiter((len(p) for p in cache_pages_list), dtype=np.int64, count=len(cache_pages_list))
     n = int(counts.sum())
-    out = np.empty((2, n), dtype=np.int64)
+    out = np.empty((3 if with_sizes else 2, n), dtype=np.int64)
     if n == 0:
         return out, 0
     pages = np.concatenate([np.asarray(p, dtype=np.int64).reshape(-1) for p in cache_pages_list if len(p)])
@@ -49,4 +51,6 @@ def build_run_offsets(cache_pages_list: Sequence[Sequence[int]], item_tokens: Se
     scale = elements_per_token if unit == "elements" else 1
     out[0] = pages * page_size * scale
     out[1] = dst * scale
+    if with_sizes:
+        out[2] = sizes
     return out, int(sizes.sum())

@@ -211,34 +211,61 @@ extern "C" void bikv_consumer_cleanup(void) {
   g_consumer = Role();
 }
 
-extern "C" int bikv_producer_copy_pages(const void* src, int64_t src_bytes, const int64_t* src_off,
-                                        const int64_t* dst_off, int64_t n_runs, int64_t page_size,
-                                        const bikv_tensor_dims* dims, int64_t elem_bytes,
-                                        int32_t dtype_code, void* stream) {
+static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_off,
+                         const int64_t* dst_off, const int64_t* run_tokens, int64_t n_runs,
+                         int64_t page_size, int64_t total_tokens, const bikv_tensor_dims* dims,
+                         int64_t elem_bytes, int32_t dtype_code, void* stream) {
   if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
   if (!dims) return fail(BIKV_EINVAL, "dims is null");
   if (n_runs < 0 || page_size <= 0 || elem_bytes <= 0) return fail(BIKV_EINVAL, "bad n_runs, page_size or elem_bytes");
   if (dims->head_size <= 0 || dims->num_kv_heads <= 0 || dims->num_layers <= 0 || dims->kv_pair <= 0)
     return fail(BIKV_EINVAL, "TensorDims fields must be positive");
+  if (total_tokens < 0 || total_tokens > n_runs * page_size)
+    return fail(BIKV_EINVAL, "total_tokens %lld is outside [0, n_runs*page_size]", (long long)total_tokens);
   bikv_shared_control* c = g_producer.ctrl;
   const int64_t elems_per_token = dims->head_size * dims->num_kv_heads * dims->num_layers * dims->kv_pair;
-  const int64_t run_bytes = page_size * elems_per_token * elem_bytes;
-  const int64_t data_size = n_runs * run_bytes;
+  const int64_t token_bytes = elems_per_token * elem_bytes;
+  const int64_t run_bytes = page_size * token_bytes;
+  const int64_t data_size = total_tokens * token_bytes;
   if ((size_t)data_size > c->buffer_size)
     return fail(BIKV_ERANGE, "batch of %lld bytes does not fit the %zu-byte ring", (long long)data_size, c->buffer_size);
   BIKV_HIP(hipSetDevice(g_producer.device));
   const size_t at = ring_reserve(c, (size_t)data_size);
   if (n_runs > 0) {
-    int rc = bikv_copy_runs(src, src_bytes, static_cast<char*>(g_producer.mem) + at,
-                            (int64_t)(c->buffer_size - at), src_off, dst_off, n_runs, run_bytes,
-                            elem_bytes, stream);
+    // the window handed to the kernel ends where this transfer ends: a run that would write past
+    // the published bytes is skipped and reported
+    char* window = static_cast<char*>(g_producer.mem) + at;
+    int rc = run_tokens
+        ? bikv_copy_runs_ragged(src, src_bytes, window, data_size, src_off, dst_off, run_tokens, n_runs,
+                                run_bytes, token_bytes, stream)
+        : bikv_copy_runs(src, src_bytes, window, (int64_t)(c->buffer_size - at), src_off, dst_off,
+                         n_runs, run_bytes, elem_bytes, stream);
     if (rc) return rc;
     rc = sync_and_check(g_producer.device, static_cast<hipStream_t>(stream));
     if (rc) return rc;
   }
-  const int64_t shape[5] = {n_runs * page_size, dims->head_size, dims->num_kv_heads, dims->num_layers, dims->kv_pair};
+  const int64_t shape[5] = {total_tokens, dims->head_size, dims->num_kv_heads, dims->num_layers, dims->kv_pair};
   ring_publish(c, (size_t)data_size, shape, 5, dtype_code);
   return BIKV_OK;
+}
+
+extern "C" int bikv_producer_copy_pages(const void* src, int64_t src_bytes, const int64_t* src_off,
+                                        const int64_t* dst_off, int64_t n_runs, int64_t page_size,
+                                        const bikv_tensor_dims* dims, int64_t elem_bytes,
+                                        int32_t dtype_code, void* stream) {
+  if (n_runs < 0 || page_size <= 0) return fail(BIKV_EINVAL, "bad n_runs, page_size or elem_bytes");
+  return producer_copy(src, src_bytes, src_off, dst_off, nullptr, n_runs, page_size, n_runs * page_size,
+                       dims, elem_bytes, dtype_code, stream);
+}
+
+extern "C" int bikv_producer_copy_tokens(const void* src, int64_t src_bytes, const int64_t* src_off,
+                                         const int64_t* dst_off, const int64_t* run_tokens,
+                                         int64_t n_runs, int64_t page_size, int64_t total_tokens,
+                                         const bikv_tensor_dims* dims, int64_t elem_bytes,
+                                         int32_t dtype_code, void* stream) {
+  if (n_runs > 0 && !run_tokens) return fail(BIKV_EINVAL, "run_tokens is null");
+  return producer_copy(src, src_bytes, src_off, dst_off, run_tokens, n_runs, page_size, total_tokens,
+                       dims, elem_bytes, dtype_code, stream);
 }
 
 extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64_t* shape,

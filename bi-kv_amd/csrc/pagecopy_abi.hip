@@ -306,15 +306,15 @@ extern "C" int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* 
   return move_pages(1, pool, batch, staging, staging_bytes, scale_staging, scale_staging_bytes, stream);
 }
 
-extern "C" int bikv_copy_runs(const void* src, int64_t src_bytes, void* dst, int64_t dst_bytes,
-                              const int64_t* src_off, const int64_t* dst_off, int64_t n_runs,
-                              int64_t run_bytes, int64_t unit_bytes, void* stream) {
+static int copy_runs_impl(const void* src, int64_t src_bytes, void* dst, int64_t dst_bytes,
+                          const int64_t* src_off, const int64_t* dst_off, const int64_t* run_len,
+                          int64_t n_runs, int64_t run_bytes, int64_t unit_bytes, void* stream) {
   if (n_runs < 0 || run_bytes < 0) return fail(BIKV_EINVAL, "negative n_runs or run_bytes");
   if (n_runs == 0 || run_bytes == 0) return BIKV_OK;
   if (!src || !dst || !src_off || !dst_off) return fail(BIKV_EINVAL, "null pointer argument");
   if (unit_bytes <= 0) return fail(BIKV_EINVAL, "unit_bytes must be positive");
   if (n_runs >= (int64_t(1) << 31)) return fail(BIKV_EINVAL, "too many runs");
-  if (run_bytes > src_bytes || run_bytes > dst_bytes)
+  if (!run_len && (run_bytes > src_bytes || run_bytes > dst_bytes))
     return fail(BIKV_EINVAL, "run_bytes %lld exceeds a buffer (src %lld, dst %lld bytes)",
                 (long long)run_bytes, (long long)src_bytes, (long long)dst_bytes);
   int dev = 0;
@@ -330,11 +330,28 @@ extern "C" int bikv_copy_runs(const void* src, int64_t src_bytes, void* dst, int
   a.n_runs = n_runs;
   a.run_bytes = run_bytes;
   a.unit_bytes = unit_bytes;
+  a.run_lens = run_len;
   rc = device_status(dev, &a.status);
   if (rc) return rc;
   hipError_t e = launch_copy_runs(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail_hip(e, "copy_runs launch");
   return BIKV_OK;
+}
+
+extern "C" int bikv_copy_runs(const void* src, int64_t src_bytes, void* dst, int64_t dst_bytes,
+                              const int64_t* src_off, const int64_t* dst_off, int64_t n_runs,
+                              int64_t run_bytes, int64_t unit_bytes, void* stream) {
+  return copy_runs_impl(src, src_bytes, dst, dst_bytes, src_off, dst_off, nullptr, n_runs, run_bytes,
+                        unit_bytes, stream);
+}
+
+extern "C" int bikv_copy_runs_ragged(const void* src, int64_t src_bytes, void* dst, int64_t dst_bytes,
+                                     const int64_t* src_off, const int64_t* dst_off,
+                                     const int64_t* run_len, int64_t n_runs, int64_t max_run_bytes,
+                                     int64_t unit_bytes, void* stream) {
+  if (n_runs > 0 && !run_len) return fail(BIKV_EINVAL, "run_len is null");
+  return copy_runs_impl(src, src_bytes, dst, dst_bytes, src_off, dst_off, run_len, n_runs,
+                        max_run_bytes, unit_bytes, stream);
 }
 
 // ---- pinned host memory -------------------------------------------------------------------

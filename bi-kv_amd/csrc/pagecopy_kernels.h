@@ -73,8 +73,9 @@ struct RunArgs {
   const int64_t* src_off;
   const int64_t* dst_off;
   int64_t n_runs;
-  int64_t run_bytes;
+  int64_t run_bytes;              // every run (run_lens null) or the longest run allowed
   int64_t unit_bytes;
+  const int64_t* run_lens;        // nullable, device: length of each run in units (ragged runs)
   uint32_t* status;
 };
 hipError_t launch_copy_runs(const RunArgs& a, hipStream_t stream);

@@ -619,8 +619,18 @@ __global__ __launch_bounds__(B) void copy_runs_wave_kernel(const RunArgs a) {
   const int64_t do_u = cload(a.dst_off + run);
   const int64_t so = so_u * a.unit_bytes;
   const int64_t dof = do_u * a.unit_bytes;
-  const bool bad_src = so_u < 0 || so < 0 || so > a.src_bytes - a.run_bytes;
-  const bool bad_dst = do_u < 0 || dof < 0 || dof > a.dst_bytes - a.run_bytes;
+  // ragged runs: this run's own length (a length outside [0, run_bytes] skips the run and is
+  // reported as a source-range fault)
+  int64_t rb = a.run_bytes;
+  bool bad_len = false;
+  if (a.run_lens) {
+    const int64_t len_u = cload(a.run_lens + run);
+    rb = len_u * a.unit_bytes;
+    bad_len = len_u < 0 || rb < 0 || rb > a.run_bytes;
+    if (bad_len) rb = 0;
+  }
+  const bool bad_src = bad_len || so_u < 0 || so < 0 || so > a.src_bytes - rb;
+  const bool bad_dst = do_u < 0 || dof < 0 || dof > a.dst_bytes - rb;
   if (bad_src || bad_dst) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
       if (bad_src) raise(a.status, ST_SLOT_SRC);
@@ -629,10 +639,10 @@ __global__ __launch_bounds__(B) void copy_runs_wave_kernel(const RunArgs a) {
     return;
   }
   const int64_t lo = (int64_t)blockIdx.x * (B * 16) + threadIdx.x * 16;
-  if (lo >= a.run_bytes) return;
+  if (lo >= rb) return;
   const uint64_t s = (uint64_t)(a.src + so + lo);
   const uint64_t d = (uint64_t)(a.dst + dof + lo);
-  const int64_t left = a.run_bytes - lo;
+  const int64_t left = rb - lo;
   if (left >= 16 && ((s | d) & 15) == 0) {
     st<NT, u32x4>(d, ld<NT, u32x4>(s));
   } else {
@@ -658,7 +668,7 @@ static hipError_t launch_runs_wave(const RunArgs& a, hipStream_t stream) {
 
 hipError_t launch_copy_runs(const RunArgs& a, hipStream_t stream) {
   if (a.n_runs <= 0 || a.run_bytes <= 0) return hipSuccess;
-  if (a.run_bytes > 2048 && tuning().run_chunk_kib == 0) {
+  if (a.run_lens || (a.run_bytes > 2048 && tuning().run_chunk_kib == 0)) {
     switch (tuning().wave_block) {
       case 128: return launch_runs_wave<128>(a, stream);
       case 256: return launch_runs_wave<256>(a, stream);

@@ -34,7 +34,7 @@ from bikv_pagecopy import _lib
 __all__ = [
     "TensorDims", "producer_init", "producer_send", "producer_cleanup", "consumer_init",
     "consumer_receive", "consumer_cleanup", "producer_copy_pages", "cuda_producer_copy_pages",
-    "producer_zero_copy_pages",
+    "producer_zero_copy_pages", "producer_copy_tokens",
 ]
 
 # dtype codes carried in the control block's first spare int (0 = float16, what a reference
@@ -113,6 +113,33 @@ def _copy_pages(data, src_offsets, dest_offsets, page_size, dims):
         _lib.check(_lib.load().bikv_producer_copy_pages(
             data.data_ptr(), data.numel() * es, src_offsets.data_ptr(), dest_offsets.data_ptr(),
             src_offsets.numel(), int(page_size), C.byref(d), es, _CODE_OF[data.dtype], _stream()))
+
+
+def producer_copy_tokens(data, src_token_offsets, dest_token_offsets, run_tokens, page_size, dims):
+    """Not in the reference's module: the packed transfer done right. Offsets and `run_tokens`
+    are in TOKENS, the unit kvcache.py:161-196 computes them in; run i copies run_tokens[i] <=
+    page_size tokens, so the packed destinations of partial last pages (kvcache.py:169-174) do not
+    overlap. `dims.total_tokens` must hold the sum of run_tokens (the host already has it from
+    building the offsets); the published shape is [total_tokens, head, kv_heads, layers, kv].
+    `data` may be a device tensor or a pinned host tensor (read over the link)."""
+    if not data.is_cuda and not data.is_pinned():
+        raise RuntimeError("CPU data must be pinned memory")
+    if not data.is_contiguous():
+        raise RuntimeError("Cache data must be contiguous")
+    for name, t in (("src_offsets", src_token_offsets), ("dest_offsets", dest_token_offsets),
+                    ("run_tokens", run_tokens)):
+        _check_offsets(name, t)
+    if not (src_token_offsets.numel() == dest_token_offsets.numel() == run_tokens.numel()):
+        raise RuntimeError("offset and length tables differ in length")
+    if data.dtype not in _CODE_OF:
+        raise RuntimeError(f"unsupported dtype {data.dtype}")
+    d = dims._c()
+    es = data.element_size()
+    with torch.cuda.device(_producer_device()):
+        _lib.check(_lib.load().bikv_producer_copy_tokens(
+            data.data_ptr(), data.numel() * es, src_token_offsets.data_ptr(), dest_token_offsets.data_ptr(),
+            run_tokens.data_ptr(), run_tokens.numel(), int(page_size), int(dims.total_tokens), C.byref(d), es,
+            _CODE_OF[data.dtype], _stream()))
 
 
 def producer_copy_pages(cache_data, src_offsets, dest_offsets, page_size, dims):

@@ -86,6 +86,17 @@ int bikv_copy_runs(const void* src, int64_t src_bytes,
                    int64_t n_runs, int64_t run_bytes, int64_t unit_bytes,
                    void* stream);
 
+/* Ragged runs: run i moves run_len[i]*unit bytes (int64 device array, 0 <= run_len[i]*unit <=
+ * max_run_bytes; a length outside that range skips the run and sets BIKV_ST_SRC_RANGE). This is what
+ * a packed destination needs: the reference packs the partial last page of an item tighter than a
+ * page (kvcache.py:169-174) but still copies whole pages (copy_kernel.cu:29-35), so its
+ * destinations overlap; with the tail length given per run they do not. */
+int bikv_copy_runs_ragged(const void* src, int64_t src_bytes,
+                          void* dst, int64_t dst_bytes,
+                          const int64_t* src_off, const int64_t* dst_off, const int64_t* run_len,
+                          int64_t n_runs, int64_t max_run_bytes, int64_t unit_bytes,
+                          void* stream);
+
 /* --------------------------------------------------------------------------------------------
  * 2. Layered paged pool — gather/scatter of (page, layer, K/V) tiles.
  *
@@ -340,6 +351,17 @@ int bikv_producer_copy_pages(const void* src, int64_t src_bytes,
                              const int64_t* src_off, const int64_t* dst_off, int64_t n_runs,
                              int64_t page_size, const bikv_tensor_dims* dims,
                              int64_t elem_bytes, int32_t dtype_code, void* stream);
+
+/* The same transfer with offsets and run lengths in TOKENS (one token = head*kv_heads*layers*kv
+ * elements), which is the unit kvcache.py:161-196 computes: run i copies run_tokens[i] <= page_size
+ * tokens from token src_off[i] of the pool to token dst_off[i] of the ring window, so that a packed
+ * destination (partial last pages) holds exactly `total_tokens` tokens with no overlap. Publishes
+ * shape [total_tokens, head, kv_heads, layers, kv]; `total_tokens` is the host-side sum of
+ * run_tokens, and a run that would write past it is skipped and reported (BIKV_EBOUNDS). */
+int bikv_producer_copy_tokens(const void* src, int64_t src_bytes, const int64_t* src_off,
+                              const int64_t* dst_off, const int64_t* run_tokens, int64_t n_runs,
+                              int64_t page_size, int64_t total_tokens, const bikv_tensor_dims* dims,
+                              int64_t elem_bytes, int32_t dtype_code, void* stream);
 
 /* producer_send (ipc_service.cpp:113-143): contiguous device tensor -> ring, publishes the real
  * shape (ndim <= 5). */

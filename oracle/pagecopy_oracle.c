@@ -7,6 +7,8 @@
  * Each function restates one piece of the reference (paths relative to the Bi-KV repository):
  *   oracle_copy_runs        SharedMemory/CUDA_Shared/copy_kernel.cu:9-36 (block_per_page_copy_kernel)
  *                           and :39-66 (zero_copy_page_kernel) — the same formula, host-side source
+ *   oracle_copy_runs_ragged the same copy with a length per run: what the packed destination offsets
+ *                           of kvcache.py:169-174 need (tail tokens of a partial last page)
  *   oracle_ring_step        copy_kernel.cu:84-89,116-127 and ipc_service.cpp:118-138 (ring advance,
  *                           shape publishing)
  *   oracle_build_offsets    DistributedStorage/kvcache.py:161-174,187-196 (page list -> offsets)
@@ -43,6 +45,28 @@ int64_t oracle_copy_runs(const uint8_t* src, int64_t src_bytes, uint8_t* dst, in
       continue;
     }
     for (int64_t e = 0; e < run_bytes; ++e) dst[d0 + e] = src[s0 + e];
+  }
+  return skipped;
+}
+
+/* Ragged form: run p moves run_len[p]*unit bytes. The packed destination of kvcache.py:169-174
+ * (a partial last page takes only `tail` tokens) is consistent only with this: copying a whole page
+ * there, as copy_kernel.cu:29-35 does, overwrites the start of the next item. Runs are applied in
+ * order. Returns the number of runs skipped (length outside [0, max_run_bytes] or out of range). */
+int64_t oracle_copy_runs_ragged(const uint8_t* src, int64_t src_bytes, uint8_t* dst, int64_t dst_bytes,
+                                const int64_t* src_off, const int64_t* dst_off, const int64_t* run_len,
+                                int64_t n_runs, int64_t max_run_bytes, int64_t unit_bytes) {
+  int64_t skipped = 0;
+  for (int64_t p = 0; p < n_runs; ++p) {
+    const int64_t s0 = src_off[p] * unit_bytes;
+    const int64_t d0 = dst_off[p] * unit_bytes;
+    const int64_t n = run_len[p] * unit_bytes;
+    if (run_len[p] < 0 || n > max_run_bytes || s0 < 0 || d0 < 0 || s0 + n > src_bytes ||
+        d0 + n > dst_bytes) {
+      ++skipped;
+      continue;
+    }
+    for (int64_t e = 0; e < n; ++e) dst[d0 + e] = src[s0 + e];
   }
   return skipped;
 }

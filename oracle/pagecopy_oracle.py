@@ -48,6 +48,9 @@ def clib():
         i64p, u8p = C.POINTER(C.c_int64), C.c_void_p
         lib.oracle_copy_runs.restype = C.c_int64
         lib.oracle_copy_runs.argtypes = [u8p, C.c_int64, u8p, C.c_int64, i64p, i64p, C.c_int64, C.c_int64, C.c_int64]
+        lib.oracle_copy_runs_ragged.restype = C.c_int64
+        lib.oracle_copy_runs_ragged.argtypes = [u8p, C.c_int64, u8p, C.c_int64, i64p, i64p, i64p, C.c_int64,
+                                                C.c_int64, C.c_int64]
         lib.oracle_ring_step.restype = C.c_uint64
         lib.oracle_ring_step.argtypes = [C.POINTER(Ring)] + [C.c_int64] * 7
         lib.oracle_ring_send.restype = C.c_uint64
@@ -88,6 +91,37 @@ def copy_runs_c(src: np.ndarray, dst: np.ndarray, src_off, dst_off, run_elems: i
     do, dop = _i64(dst_off)
     return clib().oracle_copy_runs(s.ctypes.data, s.size, d.ctypes.data, d.size, sop, dop, len(so),
                                    int(run_elems) * es, es)
+
+
+def copy_runs_ragged_c(src: np.ndarray, dst: np.ndarray, src_off, dst_off, run_len, max_run_units: int,
+                       unit_elems: int = 1) -> int:
+    """In place on dst. Offsets and lengths in units of `unit_elems` elements. Returns skipped runs."""
+    es = src.dtype.itemsize
+    assert dst.dtype.itemsize == es
+    s, d = _bytes_view(src), _bytes_view(dst)
+    so, sop = _i64(src_off)
+    do, dop = _i64(dst_off)
+    ln, lnp = _i64(run_len)
+    unit = int(unit_elems) * es
+    return clib().oracle_copy_runs_ragged(s.ctypes.data, s.size, d.ctypes.data, d.size, sop, dop, lnp,
+                                          len(so), int(max_run_units) * unit, unit)
+
+
+def packed_items_np(pool_tokens: np.ndarray, cache_pages_list, item_tokens, page_size: int) -> np.ndarray:
+    """What a packed transfer must deliver, stated without offsets: for every item, the rows of its
+    pages in list order, cut to the item's token count, items back to back. pool_tokens is
+    [n_pool_tokens, ...] (token-major pool, kvcache.py:38-43)."""
+    parts = []
+    for pages, tokens in zip(cache_pages_list, item_tokens):
+        if len(pages) == 0:
+            continue
+        rows = np.concatenate([pool_tokens[p * page_size:(p + 1) * page_size] for p in pages])
+        full = (len(pages) - 1) * page_size
+        tail = tokens % page_size or page_size
+        parts.append(rows[: full + tail])
+    if not parts:
+        return pool_tokens[:0]
+    return np.concatenate(parts)
 
 
 def copy_runs_np(src: np.ndarray, dst: np.ndarray, src_off, dst_off, run_elems: int):

@@ -222,3 +222,43 @@ def test_cache_side_callers_from_task_info(ipc, oracle, cuda, pinned_host_pool):
     assert total == 89 and do[3] == 40 * ept and so[2] == 49 * page_elems
     with pytest.raises(RuntimeError):
         kvcache_calls.shared_data_batch_pages(pool_t.cpu() if not pinned_host_pool else pool_t, info, page_size, dims)
+
+
+@pytest.mark.parametrize("pinned_host_pool", [False, True])
+def test_cache_side_callers_pack_partial_pages_exactly(ipc, oracle, cuda, pinned_host_pool):
+    """Packed transfer: the consumer receives each item's tokens, cut to its token count, back to
+    back (what kvcache.py:161-174's destination offsets describe), not whole pages."""
+    from bikv_pagecopy import kvcache_calls
+    print(f"[case] exact packing, pinned host pool={pinned_host_pool}", flush=True)
+    name = f"/bikv_test_packed_{os.getpid()}"
+    dims, page_size, pool_pages = (64, 2, 3, 2), 16, 50
+    ept = dims[0] * dims[1] * dims[2] * dims[3]
+    ipc.consumer_init(0, name, 64 << 20)
+    ipc.producer_init(0, name)
+    try:
+        rng = np.random.default_rng(29)
+        pool_h = rng.integers(0, 65536, size=(pool_pages * page_size, ept), dtype=np.uint16)
+        pool_t = torch.from_numpy(pool_h.view(np.int16)).view(torch.float16)
+        pool_t = pool_t.pin_memory() if pinned_host_pool else pool_t.to(cuda)
+        pages_list = [[7, 2, 49], [4], [], [30, 31, 0], [5]]
+        tokens = [40, 16, 0, 33, 1]
+        info = {"infer_worker": 0, "token_num": sum(tokens),
+                "id_token_pair": [(10 + i, t) for i, t in enumerate(tokens)], "cache_pages_list": pages_list}
+        if pinned_host_pool:
+            n, total = kvcache_calls.shared_data_batch_pages_cpu2gpu(pool_t, info, page_size, cuda, dims, "exact")
+        else:
+            n, total = kvcache_calls.shared_data_batch_pages(pool_t, info, page_size, dims, "exact")
+        assert (n, total) == (8, 90)
+        got = ipc.consumer_receive(timeout_ms=5000)
+        assert tuple(got.shape) == (90,) + dims
+        want = oracle.packed_items_np(pool_h, pages_list, tokens, page_size)
+        assert got.cpu().contiguous().view(torch.int16).numpy().tobytes() == want.tobytes()
+        # a total that is too small makes the last run leave the published window: reported, not written
+        d = ipc.TensorDims()
+        d.total_tokens, d.head_size, d.num_kv_heads, d.num_layers, d.kv_pair = (20,) + dims
+        t = lambda a: torch.tensor(a, dtype=torch.int64, device=cuda)
+        with pytest.raises(RuntimeError, match="destination-range"):
+            ipc.producer_copy_tokens(pool_t, t([0, 16]), t([0, 16]), t([16, 16]), page_size, d)
+    finally:
+        ipc.producer_cleanup()
+        ipc.consumer_cleanup()

@@ -405,6 +405,60 @@ def test_copy_runs_element_offsets_that_break_16_byte_alignment(bk, oracle, cuda
     assert _to_np(dst_d).tobytes() == dst_h.tobytes()
 
 
+@pytest.mark.parametrize("pinned_source", [False, True])
+def test_copy_runs_ragged_lengths(bk, oracle, cuda, pinned_source):
+    """Every run has its own length: zero, one element, around 16-byte and 1-KiB piece boundaries,
+    the maximum; offsets only element-aligned."""
+    _announce(f"copy_runs ragged, pinned source={pinned_source}")
+    from bikv_pagecopy import runs
+    rng = np.random.default_rng(61)
+    max_run = 5000
+    fixed = [0, 1, 7, 8, 9, 511, 512, 513, 1024, 4095, 4096, max_run]
+    lens = np.array(fixed + rng.integers(0, max_run + 1, size=40).tolist(), dtype=np.int64)
+    n = len(lens)
+    src_h = rng.integers(0, 65536, size=60000, dtype=np.uint16)
+    so = rng.integers(0, 60000 - max_run, size=n).astype(np.int64)
+    do = np.concatenate([[0], np.cumsum(lens + rng.integers(0, 3, size=n))[:-1]]).astype(np.int64)
+    total = int(do[-1] + lens[-1]) + 5
+    dst_h = np.full(total, 0xA5A5, dtype=np.uint16)
+    assert oracle.copy_runs_ragged_c(src_h, dst_h, so, do, lens, max_run) == 0
+    src_t = torch.from_numpy(src_h.view(np.int16)).view(torch.float16)
+    src_t = src_t.pin_memory() if pinned_source else src_t.to(cuda)
+    dst_d = torch.from_numpy(np.full(total, 0xA5A5, dtype=np.uint16).view(np.int16)).to(cuda).view(torch.float16)
+    bk.copy_runs(src_t, dst_d, torch.from_numpy(so).to(cuda), torch.from_numpy(do).to(cuda), max_run,
+                 device=cuda, run_lens=torch.from_numpy(lens).to(cuda))
+    runs.check(cuda)
+    assert _to_np(dst_d).tobytes() == dst_h.tobytes()
+    # token units: offsets and lengths count blocks of 24 elements
+    unit, max_units = 24, 16
+    lens_u = rng.integers(0, max_units + 1, size=30).astype(np.int64)
+    so_u = rng.integers(0, 60000 // unit - max_units, size=30).astype(np.int64)
+    do_u = np.concatenate([[0], np.cumsum(lens_u)[:-1]]).astype(np.int64)
+    want = np.full(int(lens_u.sum()) * unit, 0xA5A5, dtype=np.uint16)
+    assert oracle.copy_runs_ragged_c(src_h, want, so_u, do_u, lens_u, max_units, unit_elems=unit) == 0
+    got = torch.from_numpy(np.full(want.size, 0xA5A5, dtype=np.uint16).view(np.int16)).to(cuda).view(torch.float16)
+    bk.copy_runs(src_t, got, torch.from_numpy(so_u).to(cuda), torch.from_numpy(do_u).to(cuda), max_units * unit,
+                 device=cuda, run_lens=torch.from_numpy(lens_u).to(cuda), unit_elems=unit)
+    runs.check(cuda)
+    assert _to_np(got).tobytes() == want.tobytes()
+
+
+def test_copy_runs_ragged_reports_bad_lengths(bk, cuda):
+    _announce("copy_runs ragged bounds")
+    from bikv_pagecopy import runs
+    src = torch.arange(0, 4096, dtype=torch.int16, device=cuda)
+    dst = torch.zeros(4096, dtype=torch.int16, device=cuda)
+    so = torch.tensor([0, 100, 200, 4090], dtype=torch.int64, device=cuda)
+    do = torch.tensor([0, 100, 200, 300], dtype=torch.int64, device=cuda)
+    lens = torch.tensor([50, -3, 65, 10], dtype=torch.int64, device=cuda)     # ok, negative, above max, src overrun
+    bk.copy_runs(src, dst, so, do, 64, run_lens=lens)
+    with pytest.raises(RuntimeError, match="source-range"):
+        runs.check(cuda)
+    assert torch.equal(dst[:50], src[:50]) and not dst[50:].any()
+    with pytest.raises(RuntimeError, match="differ in length"):
+        bk.copy_runs(src, dst, so, do, 64, run_lens=lens[:2].contiguous())
+
+
 def test_copy_runs_rejects_offsets_outside_the_buffers(bk, cuda):
     _announce("copy_runs bounds")
     from bikv_pagecopy import runs

@@ -282,3 +282,18 @@ def test_workload_generators_have_the_stated_properties():
 
     small = w.mixed_gather_scatter(w.SHAPES["qwen2_7b"].scaled(512), 8, 1024, 8192, seed=3)
     assert sum(len(r) for r in small["gather"]) + sum(len(r) for r in small["scatter"]) <= 512
+
+
+def test_build_run_offsets_can_return_the_tokens_of_each_run():
+    from bikv_pagecopy.offsets import build_run_offsets
+    pages_list = [[7, 2, 39], [4], [], [30, 31, 0], [5, 6]]
+    tokens = [40, 16, 0, 33, 17]
+    off, total = build_run_offsets(pages_list, tokens, 16, unit="tokens", with_sizes=True)
+    assert off.shape == (3, 9) and total == 106
+    assert off[2].tolist() == [16, 16, 8, 16, 16, 16, 1, 16, 1]
+    assert off[1].tolist() == np.concatenate([[0], np.cumsum(off[2])[:-1]]).tolist()
+    assert off[0].tolist() == [p * 16 for p in (7, 2, 39, 4, 30, 31, 0, 5, 6)]
+    off2, total2 = build_run_offsets(pages_list, tokens, 16, unit="tokens")
+    assert total2 == total and np.array_equal(off2, off[:2])
+    e, t0 = build_run_offsets([], [], 16, with_sizes=True)
+    assert e.shape == (3, 0) and t0 == 0

@@ -294,3 +294,70 @@ def test_transpose_pages_equals_the_flat_token_major_formula(oracle):
     oracle.transpose_pages_c(layers, "token_kv", tm, [2], [0], "load")
     t, d, h, l, k = 1, 5, 1, 3, 0
     assert layers[l][2 * P + t, k, h, d] == (((t * D + d) * H + h) * L + l) * 2 + k
+
+
+# ---- ragged runs (packed destinations of partial last pages) -----------------------------------
+def test_ragged_copy_reduces_to_the_uniform_copy_and_to_brute_force(oracle):
+    rng = np.random.default_rng(51)
+    src = rng.integers(0, 65536, size=4000, dtype=np.uint16)
+    n, run = 23, 96
+    so = rng.integers(0, 4000 - run, size=n)
+    do = rng.permutation(n) * run
+    a = np.full(n * run, 0xA5A5, dtype=np.uint16)
+    b = a.copy()
+    assert oracle.copy_runs_ragged_c(src, a, so, do, np.full(n, run), run) == 0
+    assert oracle.copy_runs_c(src, b, so, do, run) == 0
+    assert a.tobytes() == b.tobytes()                      # all lengths equal -> the uniform copy
+    lens = rng.integers(0, run + 1, size=n)
+    lens[:2] = (0, run)
+    c = np.full(n * run, 0xA5A5, dtype=np.uint16)
+    assert oracle.copy_runs_ragged_c(src, c, so, do, lens, run) == 0
+    want = np.full(n * run, 0xA5A5, dtype=np.uint16)
+    for p in range(n):                                      # brute force, element by element
+        for e in range(int(lens[p])):
+            want[do[p] + e] = src[so[p] + e]
+    assert c.tobytes() == want.tobytes()
+    # units: offsets and lengths in blocks of 8 elements
+    d = np.full(n * run, 0xA5A5, dtype=np.uint16)
+    lens8 = rng.integers(0, run // 8 + 1, size=n)
+    so8 = rng.integers(0, (4000 - run) // 8, size=n)
+    do8 = rng.permutation(n) * (run // 8)
+    assert oracle.copy_runs_ragged_c(src, d, so8, do8, lens8, run // 8, unit_elems=8) == 0
+    want = np.full(n * run, 0xA5A5, dtype=np.uint16)
+    for p in range(n):
+        want[do8[p] * 8: do8[p] * 8 + lens8[p] * 8] = src[so8[p] * 8: so8[p] * 8 + lens8[p] * 8]
+    assert d.tobytes() == want.tobytes()
+
+
+def test_ragged_copy_skips_bad_lengths_and_ranges(oracle):
+    src = np.arange(100, dtype=np.uint16)
+    dst = np.zeros(100, dtype=np.uint16)
+    so = np.array([0, 10, 20, 95, 40])
+    do = np.array([0, 10, 20, 30, 96])
+    lens = np.array([5, -1, 11, 6, 5])                      # ok, negative, above max, src overrun, dst overrun
+    assert oracle.copy_runs_ragged_c(src, dst, so, do, lens, 10) == 4
+    assert dst[:5].tolist() == [0, 1, 2, 3, 4] and not dst[5:].any()
+
+
+def test_packed_offsets_with_tail_lengths_deliver_exactly_each_items_tokens(oracle):
+    """The reference's packed destination offsets (kvcache.py:161-174), restated by build_offsets_loops,
+    are consistent with ONE thing only: copying `tail` tokens of a partial last page. Stated without
+    any offsets, the transfer is 'each item's rows, cut to its token count, back to back'."""
+    rng = np.random.default_rng(52)
+    page_size, ept, pool_pages = 16, 12, 40
+    pool = rng.integers(0, 65536, size=(pool_pages * page_size, ept), dtype=np.uint16)
+    pages_list = [[7, 2, 39], [4], [], [30, 31, 0], [5, 6]]
+    tokens = [40, 16, 0, 33, 17]
+    so, do, total = oracle.build_offsets_loops(pages_list, [(0, t) for t in tokens], page_size)   # token units
+    sizes = []
+    for pages, t in zip(pages_list, tokens):
+        sizes += [page_size] * (len(pages) - 1) + ([t % page_size or page_size] if pages else [])
+    assert total == sum(sizes) == 40 + 16 + 33 + 17
+    dst = np.full((total, ept), 0xA5A5, dtype=np.uint16)
+    assert oracle.copy_runs_ragged_c(pool, dst, so, do, sizes, page_size, unit_elems=ept) == 0
+    want = oracle.packed_items_np(pool, pages_list, tokens, page_size)
+    assert want.shape == dst.shape and dst.tobytes() == want.tobytes()
+    # whole-page copies into the same packed offsets write past an item's end: the last run alone
+    # already leaves the buffer
+    over = np.full((total, ept), 0xA5A5, dtype=np.uint16)
+    assert oracle.copy_runs_c(pool, over, np.asarray(so) * ept, np.asarray(do) * ept, page_size * ept) >= 1
