@@ -17,6 +17,8 @@
 #include <cerrno>
 #include <cstring>
 #include <ctime>
+#include <deque>
+#include <utility>
 #include <fcntl.h>
 #include <semaphore.h>
 #include <sys/mman.h>
@@ -37,6 +39,11 @@ struct Role {
   int device = 0;
   bool ipc_mapped = false;  // producer only: mem came from hipIpcOpenMemHandle
   char shm_name[256] = "";
+  // producer only, back-pressure: transfers published and not yet released by the consumer, oldest
+  // first, as (ring offset, bytes)
+  bool backpressure = false;
+  int64_t bp_timeout_ms = -1;
+  std::deque<std::pair<size_t, size_t>> in_flight;
 };
 
 Role g_producer, g_consumer;
@@ -59,6 +66,56 @@ void unmap_role(Role& r) {
 size_t ring_reserve(bikv_shared_control* c, size_t data_size) {
   if (c->current_offset + data_size > c->buffer_size) c->current_offset = 0;
   return c->current_offset;
+}
+
+int wait_ms(sem_t* s, int64_t timeout_ms) {
+  int rc;
+  if (timeout_ms < 0) {
+    do { rc = sem_wait(s); } while (rc == -1 && errno == EINTR);
+    return rc;
+  }
+  struct timespec ts;
+  clock_gettime(CLOCK_REALTIME, &ts);
+  ts.tv_sec += timeout_ms / 1000;
+  ts.tv_nsec += (timeout_ms % 1000) * 1000000L;
+  if (ts.tv_nsec >= 1000000000L) {
+    ts.tv_sec += 1;
+    ts.tv_nsec -= 1000000000L;
+  }
+  do { rc = sem_timedwait(s, &ts); } while (rc == -1 && errno == EINTR);
+  return rc;
+}
+
+// Ring advance for the producer. Without back-pressure this is ring_reserve. With it, the write
+// window [at, at+data_size) must not touch a transfer the consumer still holds: the consumer posts
+// sem_complete once per transfer it is done with, in order, and the producer blocks here until
+// every overlapping transfer has been released (the reference declares sem_complete,
+// ipc_wrapper.h:16, initialises it, ipc_service.cpp:47, and never uses it: a wrapping producer
+// overwrites tensors the consumer may still read).
+int producer_reserve(Role& p, size_t data_size, size_t* at_out) {
+  bikv_shared_control* c = p.ctrl;
+  const size_t at = ring_reserve(c, data_size);
+  *at_out = at;
+  if (!p.backpressure) return BIKV_OK;
+  sem_t* done = sem_of(c->sem_complete);
+  while (!p.in_flight.empty() && sem_trywait(done) == 0) p.in_flight.pop_front();
+  for (;;) {
+    bool overlap = false;
+    for (const auto& t : p.in_flight)
+      if (t.second > 0 && data_size > 0 && t.first < at + data_size && at < t.first + t.second) overlap = true;
+    if (!overlap) return BIKV_OK;
+    if (wait_ms(done, p.bp_timeout_ms) != 0) {
+      if (errno == ETIMEDOUT)
+        return fail(BIKV_ESTATE, "producer timed out after %lld ms waiting for the consumer to release ring space",
+                    (long long)p.bp_timeout_ms);
+      return fail(BIKV_ESYS, "sem_wait(sem_complete) failed: %s", strerror(errno));
+    }
+    p.in_flight.pop_front();
+  }
+}
+
+void producer_published(Role& p, size_t at, size_t data_size) {
+  if (p.backpressure) p.in_flight.emplace_back(at, data_size);
 }
 
 // The reference's publish step (copy_kernel.cu:116-128, ipc_service.cpp:130-142).
@@ -230,7 +287,11 @@ static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_
   if ((size_t)data_size > c->buffer_size)
     return fail(BIKV_ERANGE, "batch of %lld bytes does not fit the %zu-byte ring", (long long)data_size, c->buffer_size);
   BIKV_HIP(hipSetDevice(g_producer.device));
-  const size_t at = ring_reserve(c, (size_t)data_size);
+  size_t at = 0;
+  {
+    const int rc = producer_reserve(g_producer, (size_t)data_size, &at);
+    if (rc) return rc;
+  }
   if (n_runs > 0) {
     // the window handed to the kernel ends where this transfer ends: a run that would write past
     // the published bytes is skipped and reported
@@ -246,6 +307,7 @@ static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_
   }
   const int64_t shape[5] = {total_tokens, dims->head_size, dims->num_kv_heads, dims->num_layers, dims->kv_pair};
   ring_publish(c, (size_t)data_size, shape, 5, dtype_code);
+  producer_published(g_producer, at, (size_t)data_size);
   return BIKV_OK;
 }
 
@@ -277,13 +339,33 @@ extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64
   if (bytes > c->buffer_size)
     return fail(BIKV_ERANGE, "tensor of %zu bytes does not fit the %zu-byte ring", bytes, c->buffer_size);
   BIKV_HIP(hipSetDevice(g_producer.device));
-  const size_t at = ring_reserve(c, bytes);
+  size_t at = 0;
+  {
+    const int rc = producer_reserve(g_producer, bytes, &at);
+    if (rc) return rc;
+  }
   if (bytes > 0) {
     BIKV_HIP(hipMemcpyAsync(static_cast<char*>(g_producer.mem) + at, dev_src, bytes,
                             hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
     BIKV_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   }
   ring_publish(c, bytes, shape, ndim, dtype_code);
+  producer_published(g_producer, at, bytes);
+  return BIKV_OK;
+}
+
+extern "C" int bikv_producer_set_backpressure(int enabled, int64_t timeout_ms) {
+  if (!g_producer.ctrl) return fail(BIKV_ESTATE, "producer is not initialised");
+  g_producer.backpressure = enabled != 0;
+  g_producer.bp_timeout_ms = timeout_ms;
+  if (!enabled) g_producer.in_flight.clear();
+  return BIKV_OK;
+}
+
+extern "C" int bikv_consumer_release(void) {
+  if (!g_consumer.ctrl) return fail(BIKV_ESTATE, "consumer is not initialised");
+  if (sem_post(sem_of(g_consumer.ctrl->sem_complete)) != 0)
+    return fail(BIKV_ESYS, "sem_post(sem_complete) failed: %s", strerror(errno));
   return BIKV_OK;
 }
 
@@ -294,17 +376,7 @@ extern "C" int bikv_consumer_receive(int64_t timeout_ms, void** ptr, int64_t sha
   if (!ptr || !shape || !ndim) return fail(BIKV_EINVAL, "null pointer argument");
   bikv_shared_control* c = g_consumer.ctrl;
   sem_t* s = sem_of(c->sem_start);
-  int rc;
-  if (timeout_ms < 0) {
-    do { rc = sem_wait(s); } while (rc == -1 && errno == EINTR);
-  } else {
-    struct timespec ts;
-    clock_gettime(CLOCK_REALTIME, &ts);
-    ts.tv_sec += timeout_ms / 1000;
-    ts.tv_nsec += (timeout_ms % 1000) * 1000000L;
-    if (ts.tv_nsec >= 1000000000L) { ts.tv_sec += 1; ts.tv_nsec -= 1000000000L; }
-    do { rc = sem_timedwait(s, &ts); } while (rc == -1 && errno == EINTR);
-  }
+  const int rc = wait_ms(s, timeout_ms);
   if (rc == -1) {
     if (errno == ETIMEDOUT) return fail(BIKV_ESTATE, "consumer_receive timed out after %lld ms", (long long)timeout_ms);
     return fail(BIKV_ESYS, "consumer_receive sem_wait failed: %s", strerror(errno));

@@ -23,7 +23,8 @@ Differences a caller can observe (all extensions; fp16 callers see the reference
     ipc_service.cpp:157);
   * a batch larger than the whole ring raises instead of overrunning the buffer;
   * offsets that would leave the source tensor or the ring raise instead of faulting the GPU;
-  * consumer_receive(timeout_ms=...) may be given a timeout (default: wait forever, as the reference).
+  * consumer_receive(timeout_ms=...) may be given a timeout (default: wait forever, as the reference);
+  * producer_copy_tokens, producer_set_backpressure and consumer_release are additions (see each).
 """
 import ctypes as C
 
@@ -34,7 +35,7 @@ from bikv_pagecopy import _lib
 __all__ = [
     "TensorDims", "producer_init", "producer_send", "producer_cleanup", "consumer_init",
     "consumer_receive", "consumer_cleanup", "producer_copy_pages", "cuda_producer_copy_pages",
-    "producer_zero_copy_pages", "producer_copy_tokens",
+    "producer_zero_copy_pages", "producer_copy_tokens", "producer_set_backpressure", "consumer_release",
 ]
 
 # dtype codes carried in the control block's first spare int (0 = float16, what a reference
@@ -86,6 +87,20 @@ def producer_cleanup():
 
 def consumer_cleanup():
     _lib.load().bikv_consumer_cleanup()
+
+
+def producer_set_backpressure(enabled, timeout_ms=-1):
+    """Not in the reference's module. When enabled, a producer call that would overwrite a tensor the
+    consumer has not released yet blocks (RuntimeError after timeout_ms); the consumer must then call
+    consumer_release() once per received tensor, in order. Uses SharedControl.sem_complete, which the
+    reference declares (ipc_wrapper.h:16) and never posts or waits on."""
+    _lib.check(_lib.load().bikv_producer_set_backpressure(1 if enabled else 0, int(timeout_ms)))
+
+
+def consumer_release():
+    """Tells a back-pressured producer that the oldest tensor handed out by consumer_receive is no
+    longer needed."""
+    _lib.check(_lib.load().bikv_consumer_release())
 
 
 def _producer_device():

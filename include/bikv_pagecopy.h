@@ -375,6 +375,17 @@ int bikv_consumer_receive(int64_t timeout_ms, void** ptr, int64_t shape[BIKV_MAX
                           size_t* ndim, size_t* data_bytes, int32_t* device_id,
                           int32_t* dtype_code);
 
+/* Back-pressure (off by default: a reference consumer never posts sem_complete). The reference
+ * declares and initialises SharedControl.sem_complete (ipc_wrapper.h:16, ipc_service.cpp:47) but
+ * never uses it, so a producer that wraps overwrites tensors the consumer may still be reading
+ * (ipc_service.cpp:146-168 hands out non-owning views). With back-pressure enabled on the
+ * producer, every transfer stays "in flight" until the consumer calls bikv_consumer_release()
+ * (once per received transfer, in order); a producer call whose ring window overlaps an in-flight
+ * transfer blocks until that transfer is released, or fails with BIKV_ESTATE after timeout_ms
+ * (< 0 = wait forever) with nothing copied or published. */
+int bikv_producer_set_backpressure(int enabled, int64_t timeout_ms);
+int bikv_consumer_release(void);
+
 /* Read-only views for tests and diagnostics (NULL when the role is not initialised). */
 const bikv_shared_control* bikv_producer_control(void);
 const bikv_shared_control* bikv_consumer_control(void);

@@ -262,3 +262,50 @@ def test_cache_side_callers_pack_partial_pages_exactly(ipc, oracle, cuda, pinned
     finally:
         ipc.producer_cleanup()
         ipc.consumer_cleanup()
+
+
+def test_backpressure_blocks_a_wrapping_producer_until_release(ipc, cuda):
+    """sem_complete in use: with back-pressure on, the producer may not wrap over a tensor the consumer
+    still holds. Ring of 2.5 transfers: the third transfer would land on the first."""
+    print("[case] ring back-pressure", flush=True)
+    name = f"/bikv_test_bp_{os.getpid()}"
+    n = 1 << 16
+    ipc.consumer_init(0, name, 5 * n * 2 // 2)          # 2.5 tensors of n fp16
+    ipc.producer_init(0, name)
+    try:
+        ipc.producer_set_backpressure(True, timeout_ms=200)
+        tensors = [torch.full((n,), float(i + 1), dtype=torch.float16, device=cuda) for i in range(4)]
+        ipc.producer_send(tensors[0])
+        first = ipc.consumer_receive(timeout_ms=5000)
+        ipc.producer_send(tensors[1])
+        second = ipc.consumer_receive(timeout_ms=5000)
+        ctrl = ipc._lib.load().bikv_producer_control().contents
+        before = (ctrl.current_offset, ctrl.last_valid_offset)
+        with pytest.raises(RuntimeError, match="release ring space"):
+            ipc.producer_send(tensors[2])               # would wrap onto `first`, still held
+        torch.cuda.synchronize()
+        assert bool((first == 1).all()) and bool((second == 2).all())
+        assert (ctrl.last_valid_offset, ctrl.data_size) == (before[1], n * 2)     # nothing was published
+        ipc.consumer_release()                          # done with `first`
+        ipc.producer_send(tensors[2])                   # now lands at offset 0
+        third = ipc.consumer_receive(timeout_ms=5000)
+        assert third.data_ptr() == first.data_ptr() and bool((third == 3).all()) and bool((second == 2).all())
+        # the fourth goes behind the third, onto `second`: blocked until that is released too
+        with pytest.raises(RuntimeError, match="release ring space"):
+            ipc.producer_send(tensors[3])
+        ipc.consumer_release()
+        ipc.producer_send(tensors[3])
+        fourth = ipc.consumer_receive(timeout_ms=5000)
+        assert bool((fourth == 4).all()) and bool((third == 3).all())
+        # switched off again: the reference's behaviour (overwrites without asking)
+        ipc.producer_set_backpressure(False)
+        ipc.producer_send(tensors[0])
+        ipc.producer_send(tensors[1])
+        assert ipc.consumer_receive(timeout_ms=5000) is not None
+    finally:
+        ipc.producer_cleanup()
+        ipc.consumer_cleanup()
+    with pytest.raises(RuntimeError, match="not initialised"):
+        ipc.consumer_release()
+    with pytest.raises(RuntimeError, match="not initialised"):
+        ipc.producer_set_backpressure(True)
