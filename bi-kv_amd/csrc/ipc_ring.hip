@@ -106,12 +106,30 @@ int producer_reserve(Role& p, size_t data_size, size_t* at_out) {
     if (!overlap) return BIKV_OK;
     if (wait_ms(done, p.bp_timeout_ms) != 0) {
       if (errno == ETIMEDOUT)
-        return fail(BIKV_ESTATE, "producer timed out after %lld ms waiting for the consumer to release ring space",
+        return fail(BIKV_ESTATE, "producer timed out after %lld ms waiting for the consumer to release the ring space it needs",
                     (long long)p.bp_timeout_ms);
       return fail(BIKV_ESYS, "sem_wait(sem_complete) failed: %s", strerror(errno));
     }
     p.in_flight.pop_front();
   }
+}
+
+// The control block has ONE slot for the published offset and shape (ipc_wrapper.h:21-27), so with
+// back-pressure a transfer is published only once the consumer has released the previous one: the
+// copy of transfer k+1 overlaps the consumer's use of transfer k, its publication does not.
+int producer_wait_slot(Role& p) {
+  if (!p.backpressure) return BIKV_OK;
+  sem_t* done = sem_of(p.ctrl->sem_complete);
+  while (!p.in_flight.empty()) {
+    if (wait_ms(done, p.bp_timeout_ms) != 0) {
+      if (errno == ETIMEDOUT)
+        return fail(BIKV_ESTATE, "producer timed out after %lld ms waiting for the consumer to release the previous transfer",
+                    (long long)p.bp_timeout_ms);
+      return fail(BIKV_ESYS, "sem_wait(sem_complete) failed: %s", strerror(errno));
+    }
+    p.in_flight.pop_front();
+  }
+  return BIKV_OK;
 }
 
 void producer_published(Role& p, size_t at, size_t data_size) {
@@ -306,6 +324,10 @@ static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_
     if (rc) return rc;
   }
   const int64_t shape[5] = {total_tokens, dims->head_size, dims->num_kv_heads, dims->num_layers, dims->kv_pair};
+  {
+    const int rc = producer_wait_slot(g_producer);
+    if (rc) return rc;
+  }
   ring_publish(c, (size_t)data_size, shape, 5, dtype_code);
   producer_published(g_producer, at, (size_t)data_size);
   return BIKV_OK;
@@ -348,6 +370,10 @@ extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64
     BIKV_HIP(hipMemcpyAsync(static_cast<char*>(g_producer.mem) + at, dev_src, bytes,
                             hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
     BIKV_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  }
+  {
+    const int rc = producer_wait_slot(g_producer);
+    if (rc) return rc;
   }
   ring_publish(c, bytes, shape, ndim, dtype_code);
   producer_published(g_producer, at, bytes);

@@ -377,12 +377,14 @@ int bikv_consumer_receive(int64_t timeout_ms, void** ptr, int64_t shape[BIKV_MAX
 
 /* Back-pressure (off by default: a reference consumer never posts sem_complete). The reference
  * declares and initialises SharedControl.sem_complete (ipc_wrapper.h:16, ipc_service.cpp:47) but
- * never uses it, so a producer that wraps overwrites tensors the consumer may still be reading
- * (ipc_service.cpp:146-168 hands out non-owning views). With back-pressure enabled on the
- * producer, every transfer stays "in flight" until the consumer calls bikv_consumer_release()
- * (once per received transfer, in order); a producer call whose ring window overlaps an in-flight
- * transfer blocks until that transfer is released, or fails with BIKV_ESTATE after timeout_ms
- * (< 0 = wait forever) with nothing copied or published. */
+ * never uses it, so a producer that runs ahead overwrites the single published offset/shape slot,
+ * and one that wraps overwrites tensors the consumer may still be reading (ipc_service.cpp:146-168
+ * hands out non-owning views). With back-pressure enabled on the producer, a transfer stays "in
+ * flight" until the consumer calls bikv_consumer_release() (once per received transfer). A producer
+ * call (i) blocks before copying while its ring window overlaps the in-flight transfer, (ii) copies,
+ * then (iii) blocks before publishing until the in-flight transfer is released: the copy of the next
+ * transfer overlaps the consumer's use of the current one. Either wait fails with BIKV_ESTATE after
+ * timeout_ms (< 0 = wait forever) with nothing published. */
 int bikv_producer_set_backpressure(int enabled, int64_t timeout_ms);
 int bikv_consumer_release(void);
 

@@ -264,9 +264,9 @@ def test_cache_side_callers_pack_partial_pages_exactly(ipc, oracle, cuda, pinned
         ipc.consumer_cleanup()
 
 
-def test_backpressure_blocks_a_wrapping_producer_until_release(ipc, cuda):
-    """sem_complete in use: with back-pressure on, the producer may not wrap over a tensor the consumer
-    still holds. Ring of 2.5 transfers: the third transfer would land on the first."""
+def test_backpressure_holds_the_producer_until_release(ipc, cuda):
+    """sem_complete in use. With back-pressure on, the producer copies ahead into free ring space but
+    publishes only after the consumer released the previous tensor, and never copies over a held one."""
     print("[case] ring back-pressure", flush=True)
     name = f"/bikv_test_bp_{os.getpid()}"
     n = 1 << 16
@@ -274,30 +274,35 @@ def test_backpressure_blocks_a_wrapping_producer_until_release(ipc, cuda):
     ipc.producer_init(0, name)
     try:
         ipc.producer_set_backpressure(True, timeout_ms=200)
-        tensors = [torch.full((n,), float(i + 1), dtype=torch.float16, device=cuda) for i in range(4)]
+        tensors = [torch.full((n,), float(i + 1), dtype=torch.float16, device=cuda) for i in range(3)]
+        big = torch.full((2 * n,), 9.0, dtype=torch.float16, device=cuda)
+        ctrl = ipc._lib.load().bikv_producer_control().contents
         ipc.producer_send(tensors[0])
         first = ipc.consumer_receive(timeout_ms=5000)
+        with pytest.raises(RuntimeError, match="release the previous transfer"):
+            ipc.producer_send(tensors[1])               # copied behind `first`, but not published
+        assert (ctrl.last_valid_offset, ctrl.data_size) == (0, n * 2) and bool((first == 1).all())
+        with pytest.raises(RuntimeError, match="timed out"):
+            ipc.consumer_receive(timeout_ms=50)         # nothing new to receive
+        ipc.consumer_release()
         ipc.producer_send(tensors[1])
         second = ipc.consumer_receive(timeout_ms=5000)
-        ctrl = ipc._lib.load().bikv_producer_control().contents
-        before = (ctrl.current_offset, ctrl.last_valid_offset)
-        with pytest.raises(RuntimeError, match="release ring space"):
-            ipc.producer_send(tensors[2])               # would wrap onto `first`, still held
+        assert second.data_ptr() == first.data_ptr() + n * 2 and bool((second == 2).all())
+        # a transfer of 2n elements has to wrap to offset 0 and would reach into `second`: the producer
+        # blocks BEFORE copying
+        with pytest.raises(RuntimeError, match="release the ring space"):
+            ipc.producer_send(big)
         torch.cuda.synchronize()
-        assert bool((first == 1).all()) and bool((second == 2).all())
-        assert (ctrl.last_valid_offset, ctrl.data_size) == (before[1], n * 2)     # nothing was published
-        ipc.consumer_release()                          # done with `first`
-        ipc.producer_send(tensors[2])                   # now lands at offset 0
-        third = ipc.consumer_receive(timeout_ms=5000)
-        assert third.data_ptr() == first.data_ptr() and bool((third == 3).all()) and bool((second == 2).all())
-        # the fourth goes behind the third, onto `second`: blocked until that is released too
-        with pytest.raises(RuntimeError, match="release ring space"):
-            ipc.producer_send(tensors[3])
+        assert bool((second == 2).all())
         ipc.consumer_release()
-        ipc.producer_send(tensors[3])
+        ipc.producer_send(big)
+        third = ipc.consumer_receive(timeout_ms=5000)
+        assert third.data_ptr() == first.data_ptr() and third.numel() == 2 * n and bool((third == 9).all())
+        ipc.consumer_release()
+        ipc.producer_send(tensors[2])                   # 2n + n > 2.5n: wraps again
         fourth = ipc.consumer_receive(timeout_ms=5000)
-        assert bool((fourth == 4).all()) and bool((third == 3).all())
-        # switched off again: the reference's behaviour (overwrites without asking)
+        assert fourth.data_ptr() == first.data_ptr() and bool((fourth == 3).all())
+        # switched off again: the reference's behaviour (publishes without asking)
         ipc.producer_set_backpressure(False)
         ipc.producer_send(tensors[0])
         ipc.producer_send(tensors[1])

@@ -7,6 +7,7 @@ are kept far below 2 GiB)."""
 import multiprocessing as mp
 import os
 import sys
+import time
 
 import numpy as np
 import pytest
@@ -36,7 +37,7 @@ def _pool():
     return np.random.default_rng(99).integers(0, 65536, size=POOL_PAGES * PAGE_ELEMS, dtype=np.uint16)
 
 
-def _consumer(name, ready, go, out):
+def _consumer(name, ready, go, out, backpressure=False):
     try:
         _paths()
         import torch
@@ -47,8 +48,13 @@ def _consumer(name, ready, go, out):
         for k in range(TRANSFERS):
             t = ipc_service.consumer_receive(timeout_ms=60000)
             assert tuple(t.shape) == (N_RUNS * PAGE_SIZE,) + DIMS and t.dtype == torch.float16
+            if backpressure:
+                time.sleep(0.05)          # a slow consumer: the producer has time to run ahead
             digests.append(t.cpu().contiguous().view(torch.int16).numpy().tobytes())
-            go.set()                      # the producer may overwrite the ring from here on
+            if backpressure:
+                ipc_service.consumer_release()
+            else:
+                go.set()                  # the producer may overwrite the ring from here on
         ipc_service.consumer_cleanup()
         out.put(("consumer", "ok", digests))
     except Exception as e:  # noqa: BLE001
@@ -56,7 +62,7 @@ def _consumer(name, ready, go, out):
         go.set()
 
 
-def _producer(name, ready, go, out):
+def _producer(name, ready, go, out, backpressure=False):
     try:
         _paths()
         import torch
@@ -64,6 +70,8 @@ def _producer(name, ready, go, out):
         if not ready.wait(120):
             raise RuntimeError("consumer did not come up")
         ipc_service.producer_init(0, name.encode())
+        if backpressure:
+            ipc_service.producer_set_backpressure(True, timeout_ms=60000)
         pool = torch.from_numpy(_pool().view(np.int16)).cuda().view(torch.float16)
         d = ipc_service.TensorDims()
         d.head_size, d.num_kv_heads, d.num_layers, d.kv_pair = DIMS
@@ -71,6 +79,8 @@ def _producer(name, ready, go, out):
             so, do = _transfer(k)
             ipc_service.producer_copy_pages(pool, torch.from_numpy(so).cuda(), torch.from_numpy(do).cuda(),
                                             PAGE_SIZE, d)
+            if backpressure:
+                continue                  # no handshake outside the ring: sem_complete paces the producer
             if not go.wait(120):
                 raise RuntimeError("consumer did not acknowledge")
             go.clear()
@@ -80,13 +90,17 @@ def _producer(name, ready, go, out):
         out.put(("producer", f"{type(e).__name__}: {e}", None))
 
 
-def test_two_process_page_copy_over_hip_ipc(oracle, cuda):
-    print("[case] ipc_service two processes", flush=True)
+@pytest.mark.parametrize("backpressure", [False, True])
+def test_two_process_page_copy_over_hip_ipc(oracle, cuda, backpressure):
+    """backpressure=False: the reference's protocol, paced by an event outside the ring (its scripts
+    sleep instead). backpressure=True: a free-running producer and a slow consumer, paced only by
+    sem_complete."""
+    print(f"[case] ipc_service two processes, backpressure={backpressure}", flush=True)
     ctx = mp.get_context("spawn")
-    name = f"/bikv_test_2proc_{os.getpid()}"
+    name = f"/bikv_test_2proc_{os.getpid()}_{int(backpressure)}"
     ready, go, out = ctx.Event(), ctx.Event(), ctx.Queue()
-    procs = [ctx.Process(target=_consumer, args=(name, ready, go, out)),
-             ctx.Process(target=_producer, args=(name, ready, go, out))]
+    procs = [ctx.Process(target=_consumer, args=(name, ready, go, out, backpressure)),
+             ctx.Process(target=_producer, args=(name, ready, go, out, backpressure))]
     for p in procs:
         p.start()
     results = {}
