@@ -154,6 +154,12 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
   } else if (!strcmp(key, "transpose_dsplit")) {
     if (value < 0 || value > 16 || (value & (value - 1))) return fail(BIKV_EINVAL, "transpose_dsplit must be 0 or a power of two <= 16");
     t.transpose_dsplit = (int)value;
+  } else if (!strcmp(key, "transpose_block")) {
+    if (value != 128 && value != 256 && value != 512 && value != 1024)
+      return fail(BIKV_EINVAL, "transpose_block must be 128, 256, 512 or 1024");
+    t.transpose_block = (int)value;
+  } else if (!strcmp(key, "transpose_pairs")) {
+    t.transpose_pairs = value ? 1 : 0;
   } else if (!strcmp(key, "run_chunk_kib")) {
     if (value < 0 || value > 1 << 20) return fail(BIKV_EINVAL, "run_chunk_kib out of range");
     t.run_chunk_kib = (int)value;

@@ -55,6 +55,8 @@ struct Tuning {
   int run_chunk_kib = 0;  // bytes of a run handled by one workgroup, KiB; 0 = choose
   int transpose_lds_kib = 60;  // LDS tile budget of the layout-change kernel, KiB
   int transpose_dsplit = 0;    // slices of head_dim per tile; 0 = default (1: whole compute rows)
+  int transpose_pairs = 1;  // 2-byte elements: the word-pair kernel (0 = element-wise kernel)
+  int transpose_block = 512; // lanes per workgroup of the word-pair kernel: 128, 256, 512, 1024
 };
 Tuning& tuning();
 

@@ -154,6 +154,197 @@ __global__ __launch_bounds__(kBlock) void transpose_pages_kernel(const Transpose
   }
 }
 
+// ---- 2-byte elements, K/V pairs as 32-bit words -----------------------------------------------
+// Column c = (h*L + l)*2 + k puts the K and the V element of one (head, layer) next to each other,
+// so a token row is a sequence of 32-bit words {K[d], V[d]} and the layout change is a transpose
+// of WORDS ([D][C/2] -> [C/2][D]) followed by a de-interleave of 16-bit halves in registers.
+// LDS holds the tile transposed, [column pair][d] words, no padding; the 4-word groups of a row
+// are permuted by XOR with (pair/4 mod 8), which keeps 16-byte LDS accesses along d intact and
+// spreads the word-wise accesses of the other side (lanes walk a token-major row: pair index steps
+// by 4) over all banks. Per 16-byte vector moved this takes 5 LDS instructions and ~30 VALU
+// instructions; the element-wise kernel above takes 11 and ~100 (three integer divisions).
+// Needs head_dim % 32 == 0 (XOR closure over the groups of a row).
+struct Walk {        // (outer, inner) of a linear index that advances by kBlock per step
+  int outer, inner;
+};
+__device__ __forceinline__ Walk walk_start(int idx, int n_inner) {
+  Walk w;
+  w.outer = idx / n_inner;
+  w.inner = idx - w.outer * n_inner;
+  return w;
+}
+__device__ __forceinline__ void walk_step(Walk& w, int q, int r, int n_inner) {
+  w.outer += q;
+  w.inner += r;
+  if (w.inner >= n_inner) {
+    w.inner -= n_inner;
+    w.outer += 1;
+  }
+}
+
+template <int DIR, int B>
+__global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs a) {
+  extern __shared__ uint32_t lds_words[];
+  u32x4* lds_vec = reinterpret_cast<u32x4*>(lds_words);
+  uint64_t* row_addr = reinterpret_cast<uint64_t*>(lds_words + a.tile_words);  // K row of each pair
+
+  const uint32_t chunk = blockIdx.x % a.n_chunks;              // column chunk
+  const uint32_t t = blockIdx.x / a.n_chunks;                  // token within the page
+  const uint64_t i = (uint64_t)blockIdx.y + (uint64_t)blockIdx.z * gridDim.y;
+  if (i >= (uint64_t)a.n_pages) return;
+  const int64_t blk = tload(a.block_ids + i);
+  const int64_t tmp = tload(a.tm_pages + i);
+  const bool bad_blk = (uint64_t)blk >= (uint64_t)a.n_blocks;
+  const bool bad_tm = (uint64_t)tmp >= (uint64_t)a.n_tm_pages;
+  if (bad_blk || bad_tm) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+      if (bad_blk) *reinterpret_cast<volatile uint32_t*>(a.status + ST_SLOT_PAGE) = 1u;
+      if (bad_tm) *reinterpret_cast<volatile uint32_t*>(a.status + (DIR == 0 ? ST_SLOT_DST : ST_SLOT_SRC)) = 1u;
+    }
+    return;
+  }
+  const int D = a.head_dim, C = a.n_cols;
+  const int Cw = a.chunk_cols >> 1;        // column pairs in the tile
+  const int vpr = a.chunk_cols >> 3;       // 16-byte vectors per token-major row piece
+  const int dgs = D >> 3;                  // 16-byte vectors per compute row
+  const int cp0 = (int)chunk * Cw;
+  // The compute side is walked layer by layer (all heads of a layer, K rows then V rows, are
+  // neighbours in memory), the LDS tile is indexed by column pair (head-major): entry j of the table
+  // holds the K row address of the j-th pair in walking order and, in its top 16 bits, that pair's
+  // index in the tile. A tile that is only a column chunk of the token is walked in column order.
+  const int n_heads = C / (2 * a.n_layers);
+  for (int j = threadIdx.x; j < Cw; j += B) {
+    int h, l, cp;
+    if (a.n_chunks == 1) {
+      l = j / n_heads;
+      h = j - l * n_heads;
+      cp = h * a.n_layers + l;
+    } else {
+      cp = j;
+      h = (cp0 + cp) / a.n_layers;
+      l = (cp0 + cp) - h * a.n_layers;
+    }
+    const int64_t off = blk * a.block_stride + (int64_t)t * a.token_stride + (int64_t)h * a.head_dim;
+    row_addr[j] = ((uint64_t)a.layer_base[l] + (uint64_t)off * 2) | ((uint64_t)cp << 48);
+  }
+  const uint64_t kv_bytes = (uint64_t)a.kv_stride * 2;
+  const uint64_t tm_tok = (uint64_t)a.tm_base +
+                          (((uint64_t)(tmp * a.block_tokens + t) * D) * C + (uint64_t)cp0 * 2) * 2;
+  const uint64_t tm_row_bytes = (uint64_t)C * 2;
+  const int n_tm = D * vpr;                // vectors on the token-major side
+  const int n_cp = Cw * dgs;               // (pair, 8 d) items on the compute side
+  // LDS word index of (pair cp, d): cp*D + (d ^ (((cp >> 2) & 7) << 2))
+
+  if (DIR == 1) {
+    // token-major rows -> LDS, four words of a vector to four pair rows
+    constexpr int U = 8;
+    const int q = B / vpr, r = B - q * vpr;
+    Walk w = walk_start(threadIdx.x, vpr);                     // (d, vector within the row piece)
+    for (int base = 0; base < n_tm; base += B * U) {
+      u32x4 x[U];
+      Walk wu = w;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const bool ok = wu.outer < D;                          // a lane past the end re-reads row 0
+        const int d = ok ? wu.outer : 0;
+        x[u] = __builtin_nontemporal_load(
+            (const BIKV_GLOBAL u32x4*)(tm_tok + (uint64_t)d * tm_row_bytes + (uint64_t)wu.inner * 16));
+        walk_step(wu, q, r, vpr);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (w.outer < D) {
+          const int cv = w.inner;
+          uint32_t* row = lds_words + (cv * 4) * D + (w.outer ^ ((cv & 7) << 2));
+          row[0] = x[u].x;
+          row[D] = x[u].y;
+          row[2 * D] = x[u].z;
+          row[3 * D] = x[u].w;
+        }
+        walk_step(w, q, r, vpr);
+      }
+    }
+    __syncthreads();
+    // LDS -> compute rows: 8 words {K[d],V[d]} become one K vector and one V vector
+    const int q2 = B / dgs, r2 = B - q2 * dgs;
+    Walk o = walk_start(threadIdx.x, dgs);                     // (pair, 8-d group)
+    for (int base = 0; base < n_cp; base += B) {
+      if (o.outer < Cw) {
+        const uint64_t entry = row_addr[o.outer];
+        const int cp = (int)(entry >> 48), dg = o.inner;
+        const int s = (cp >> 2) & 7;
+        const int flip = (dg >> 2) & 1;                        // lanes 0-3 and 4-7 start on different halves
+        const u32x4 lo = lds_vec[(cp * D >> 2) + ((2 * dg + flip) ^ s)];
+        const u32x4 hi = lds_vec[(cp * D >> 2) + ((2 * dg + 1 - flip) ^ s)];
+        const u32x4 g0 = flip ? hi : lo, g1 = flip ? lo : hi;  // words d..d+3, d+4..d+7
+        u32x4 kx, vx;
+        kx.x = __builtin_amdgcn_perm(g0.y, g0.x, 0x05040100u);
+        kx.y = __builtin_amdgcn_perm(g0.w, g0.z, 0x05040100u);
+        kx.z = __builtin_amdgcn_perm(g1.y, g1.x, 0x05040100u);
+        kx.w = __builtin_amdgcn_perm(g1.w, g1.z, 0x05040100u);
+        vx.x = __builtin_amdgcn_perm(g0.y, g0.x, 0x07060302u);
+        vx.y = __builtin_amdgcn_perm(g0.w, g0.z, 0x07060302u);
+        vx.z = __builtin_amdgcn_perm(g1.y, g1.x, 0x07060302u);
+        vx.w = __builtin_amdgcn_perm(g1.w, g1.z, 0x07060302u);
+        const uint64_t ra = (entry & 0xFFFFFFFFFFFFull) + (uint64_t)dg * 16;
+        __builtin_nontemporal_store(kx, (BIKV_GLOBAL u32x4*)ra);
+        __builtin_nontemporal_store(vx, (BIKV_GLOBAL u32x4*)(ra + kv_bytes));
+      }
+      walk_step(o, q2, r2, dgs);
+    }
+  } else {
+    // compute rows -> LDS: a K vector and a V vector interleave into 8 words
+    __syncthreads();                                            // row_addr
+    constexpr int U = 4;
+    const int q2 = B / dgs, r2 = B - q2 * dgs;
+    Walk o = walk_start(threadIdx.x, dgs);
+    for (int base = 0; base < n_cp; base += B * U) {
+      u32x4 kx[U], vx[U];
+      Walk ou = o;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const bool ok = ou.outer < Cw;
+        const uint64_t ra = (row_addr[ok ? ou.outer : 0] & 0xFFFFFFFFFFFFull) + (uint64_t)ou.inner * 16;
+        kx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)ra);
+        vx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(ra + kv_bytes));
+        walk_step(ou, q2, r2, dgs);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (o.outer < Cw) {
+          const int cp = (int)(row_addr[o.outer] >> 48), dg = o.inner;
+          const int s = (cp >> 2) & 7;
+          u32x4 g0, g1;
+          g0.x = __builtin_amdgcn_perm(vx[u].x, kx[u].x, 0x05040100u);
+          g0.y = __builtin_amdgcn_perm(vx[u].x, kx[u].x, 0x07060302u);
+          g0.z = __builtin_amdgcn_perm(vx[u].y, kx[u].y, 0x05040100u);
+          g0.w = __builtin_amdgcn_perm(vx[u].y, kx[u].y, 0x07060302u);
+          g1.x = __builtin_amdgcn_perm(vx[u].z, kx[u].z, 0x05040100u);
+          g1.y = __builtin_amdgcn_perm(vx[u].z, kx[u].z, 0x07060302u);
+          g1.z = __builtin_amdgcn_perm(vx[u].w, kx[u].w, 0x05040100u);
+          g1.w = __builtin_amdgcn_perm(vx[u].w, kx[u].w, 0x07060302u);
+          lds_vec[(cp * D >> 2) + ((2 * dg) ^ s)] = g0;
+          lds_vec[(cp * D >> 2) + ((2 * dg + 1) ^ s)] = g1;
+        }
+        walk_step(o, q2, r2, dgs);
+      }
+    }
+    __syncthreads();
+    const int q = B / vpr, r = B - q * vpr;
+    Walk w = walk_start(threadIdx.x, vpr);
+    for (int base = 0; base < n_tm; base += B) {
+      if (w.outer < D) {
+        const int cv = w.inner;
+        const uint32_t* row = lds_words + (cv * 4) * D + (w.outer ^ ((cv & 7) << 2));
+        u32x4 x = {row[0], row[D], row[2 * D], row[3 * D]};
+        __builtin_nontemporal_store(
+            x, (BIKV_GLOBAL u32x4*)(tm_tok + (uint64_t)w.outer * tm_row_bytes + (uint64_t)cv * 16));
+      }
+      walk_step(w, q, r, vpr);
+    }
+  }
+}
+
 template <int DIR>
 static hipError_t launch_transpose_dir(const TransposeArgs& a, dim3 grid, size_t lds, hipStream_t s) {
   switch (a.elem_bytes) {
@@ -180,6 +371,43 @@ hipError_t launch_transpose_pages(int dir, TransposeArgs& a, hipStream_t stream)
   // compute rows (Dd = head_dim) and the widest column chunk that fits LDS. Cutting head_dim to make
   // room for wider chunks lost 10-25 %, a 16 KiB tile lost 30-60 %, so the default is the full
   // head_dim with a ~60 KiB tile (two workgroups per CU).
+  if (ES == 2 && D % 32 == 0 && tuning().transpose_pairs != 0 && tuning().transpose_dsplit <= 1) {
+    // the word-pair kernel: unpadded tile [Cc/2 pairs][D] words, the widest column chunk that fits
+    const int64_t budget = (int64_t)tuning().transpose_lds_kib * 1024;
+    int best = 0;
+    for (int cc = VE; cc <= C; cc += VE)
+      if (C % cc == 0 && (int64_t)D * cc * 2 + (cc / 2) * 8 <= budget) best = cc;
+    if (best > 0) {
+      a.chunk_rows = D;
+      a.n_dchunks = 1;
+      a.chunk_cols = best;
+      a.pitch = 0;
+      a.n_chunks = (uint32_t)(C / best);
+      a.tile_words = (uint32_t)((int64_t)D * best / 2);
+      const size_t lds = (size_t)a.tile_words * 4 + (size_t)(best / 2) * 8;
+      const int64_t gx = (int64_t)a.n_chunks * a.block_tokens;
+      const int64_t gy = a.n_pages < 32768 ? a.n_pages : 32768;
+      const int64_t gz = (a.n_pages + gy - 1) / gy;
+      if (gx >= (int64_t(1) << 24) || gz > 65535) return hipErrorInvalidValue;
+      const dim3 grid((uint32_t)gx, (uint32_t)gy, (uint32_t)gz);
+      const int block = tuning().transpose_block;
+#define BIKV_LAUNCH_PAIRS(DIR_, B_) \
+  hipLaunchKernelGGL((transpose_pairs_kernel<DIR_, B_>), grid, dim3(B_), lds, stream, a)
+      if (dir == 0) {
+        if (block == 512) BIKV_LAUNCH_PAIRS(0, 512);
+        else if (block == 1024) BIKV_LAUNCH_PAIRS(0, 1024);
+        else if (block == 128) BIKV_LAUNCH_PAIRS(0, 128);
+        else BIKV_LAUNCH_PAIRS(0, 256);
+      } else {
+        if (block == 512) BIKV_LAUNCH_PAIRS(1, 512);
+        else if (block == 1024) BIKV_LAUNCH_PAIRS(1, 1024);
+        else if (block == 128) BIKV_LAUNCH_PAIRS(1, 128);
+        else BIKV_LAUNCH_PAIRS(1, 256);
+      }
+#undef BIKV_LAUNCH_PAIRS
+      return hipGetLastError();
+    }
+  }
   const int budget_elems = (tuning().transpose_lds_kib * 1024) / ES;
   int dsplit = tuning().transpose_dsplit;
   if (dsplit <= 0) dsplit = 1;

@@ -63,7 +63,9 @@ int bikv_check_status(int device, void* stream, uint32_t* bits_out);
  * "unroll" (segment mover: 16-byte vectors in flight per lane: 1, 2, 4, 8), "nontemporal" (nt hint on
  * payload accesses: 1 on, 0 off, -1 = default: chosen per direction and layout),
  * "run_chunk_kib" (bytes of a run per workgroup, KiB; 0 = automatic), "transpose_lds_kib" and
- * "transpose_dsplit" (LDS tile budget and head_dim slices of the layout-change kernel).
+ * "transpose_dsplit" (LDS tile budget and head_dim slices of the layout-change kernel),
+ * "transpose_pairs" (2-byte elements with head_dim % 32 == 0: 1 = the word-pair kernel, default;
+ * 0 = the element-wise kernel) and "transpose_block" (its lanes per workgroup: 128, 256, 512, 1024).
  * Process-wide. */
 int bikv_set_tuning(const char* key, int64_t value);
 

@@ -33,10 +33,17 @@ def _make(rng, form, es, P, D, H, L, blocks, n_tm, cuda):
     (4, 4, 64, 2, 6),        # fp32
     (2, 3, 8, 2, 2),         # the smallest shape the kernel takes (one vector per row)
     (2, 5, 80, 4, 3),        # head_dim 80: 10 vectors per row, not a multiple of 4
+    (2, 4, 96, 4, 5),        # head_dim 96: word-pair kernel with 12 vectors per compute row
+    (2, 2, 32, 1, 4),        # the smallest shape of the word-pair kernel: one vector per token-major row
+    (2, 3, 256, 2, 36),      # head_dim 256, 144 columns: the tile is cut into column chunks
 ])
-def test_load_and_store_match_oracle(lib, oracle, cuda, form, es, P, D, H, L):
+@pytest.mark.parametrize("pairs", [1, 0])
+def test_load_and_store_match_oracle(lib, oracle, cuda, form, es, P, D, H, L, pairs):
     import bikv_pagecopy as bk
-    print(f"[case] layout change {form} es={es} P={P} D={D} H={H} L={L}", flush=True)
+    if pairs == 0 and (es != 2 or D % 32):
+        pytest.skip("only 2-byte elements with head_dim % 32 == 0 have two kernels to choose from")
+    print(f"[case] layout change {form} es={es} P={P} D={D} H={H} L={L} pairs={pairs}", flush=True)
+    bk.set_tuning(transpose_pairs=pairs)
     rng = np.random.default_rng(es * 1000 + D + H + L)
     blocks, n_tm = 9, 7
     tm_h, layers_h, tm_d, layers_d = _make(rng, form, es, P, D, H, L, blocks, n_tm, cuda)
@@ -56,8 +63,36 @@ def test_load_and_store_match_oracle(lib, oracle, cuda, form, es, P, D, H, L):
     tm_pages2 = rng.permutation(n_tm)[:4].astype(np.int64)
     pool.store_token_major(tm_d, torch.from_numpy(block_ids2).to(cuda), torch.from_numpy(tm_pages2).to(cuda))
     pool.check()
+    bk.set_tuning(transpose_pairs=1)
     assert oracle.transpose_pages_c(layers_h, form, tm_h, block_ids2, tm_pages2, "store") == 0
     assert _to_np(tm_d).tobytes() == tm_h.tobytes()
+
+
+@pytest.mark.parametrize("block", [128, 256, 1024])
+def test_word_pair_kernel_at_other_workgroup_sizes(lib, oracle, cuda, block):
+    import bikv_pagecopy as bk
+    print(f"[case] layout change, word-pair kernel with {block} lanes", flush=True)
+    rng = np.random.default_rng(block)
+    P, D, H, L, blocks, n_tm = 5, 64, 3, 4, 8, 6
+    tm_h, layers_h, tm_d, layers_d = _make(rng, "block_kv", 2, P, D, H, L, blocks, n_tm, cuda)
+    pool = bk.NHDPool.from_block_kv_layers(layers_d)
+    ids = rng.permutation(blocks)[:5].astype(np.int64)
+    pages = rng.permutation(n_tm)[:5].astype(np.int64)
+    bk.set_tuning(transpose_block=block)
+    try:
+        pool.load_token_major(tm_d, torch.from_numpy(ids).to(cuda), torch.from_numpy(pages).to(cuda))
+        pool.check()
+        oracle.transpose_pages_c(layers_h, "block_kv", tm_h, ids, pages, "load")
+        for l in range(L):
+            assert _to_np(layers_d[l]).tobytes() == layers_h[l].tobytes(), f"layer {l}"
+        ids2 = rng.permutation(blocks)[:4].astype(np.int64)
+        pages2 = rng.permutation(n_tm)[:4].astype(np.int64)
+        pool.store_token_major(tm_d, torch.from_numpy(ids2).to(cuda), torch.from_numpy(pages2).to(cuda))
+        pool.check()
+        oracle.transpose_pages_c(layers_h, "block_kv", tm_h, ids2, pages2, "store")
+        assert _to_np(tm_d).tobytes() == tm_h.tobytes()
+    finally:
+        bk.set_tuning(transpose_block=512)
 
 
 def test_default_tm_pages_is_a_dense_received_buffer(lib, oracle, cuda):
