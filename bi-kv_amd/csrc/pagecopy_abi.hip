@@ -147,13 +147,19 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
     if (value < -1 || value > 16) return fail(BIKV_EINVAL, "log2_chunk must be in [-1, 16]");
     t.log2_chunk = (int)value;
   } else if (!strcmp(key, "nontemporal")) {
-    t.nontemporal = value < 0 ? -1 : (value ? 1 : 0);
+    if (value > 3) return fail(BIKV_EINVAL, "nontemporal must be -1, 0, 1, 2 (loads only) or 3 (stores only)");
+    t.nontemporal = value < 0 ? -1 : (int)value;
   } else if (!strcmp(key, "transpose_lds_kib")) {
     if (value < 2 || value > 60) return fail(BIKV_EINVAL, "transpose_lds_kib must be in [2, 60]");
     t.transpose_lds_kib = (int)value;
   } else if (!strcmp(key, "transpose_dsplit")) {
     if (value < 0 || value > 16 || (value & (value - 1))) return fail(BIKV_EINVAL, "transpose_dsplit must be 0 or a power of two <= 16");
     t.transpose_dsplit = (int)value;
+  } else if (!strcmp(key, "run_group")) {
+    t.run_group = value ? 1 : 0;
+  } else if (!strcmp(key, "small_run_max")) {
+    if (value < 16 || value > (1 << 20)) return fail(BIKV_EINVAL, "small_run_max must be in [16, 1 MiB]");
+    t.small_run_max = (int)value;
   } else if (!strcmp(key, "transpose_block")) {
     if (value != 128 && value != 256 && value != 512 && value != 1024)
       return fail(BIKV_EINVAL, "transpose_block must be 128, 256, 512 or 1024");

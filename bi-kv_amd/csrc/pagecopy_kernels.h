@@ -55,7 +55,9 @@ struct Tuning {
   int run_chunk_kib = 0;  // bytes of a run handled by one workgroup, KiB; 0 = choose
   int transpose_lds_kib = 60;  // LDS tile budget of the layout-change kernel, KiB
   int transpose_dsplit = 0;    // slices of head_dim per tile; 0 = default (1: whole compute rows)
-  int transpose_pairs = 1;  // 2-byte elements: the word-pair kernel (0 = element-wise kernel)
+int run_group = 1;         // wave run kernel: pack several short runs into one grid row (0 = off)
+  int small_run_max = 1023;  // runs up to this many bytes go to the one-lane-per-piece kernel
+    int transpose_pairs = 1;  // 2-byte elements: the word-pair kernel (0 = element-wise kernel)
   int transpose_block = 512; // lanes per workgroup of the word-pair kernel: 128, 256, 512, 1024
 };
 Tuning& tuning();

@@ -564,7 +564,8 @@ __global__ __launch_bounds__(kBlock) void copy_runs_kernel(const RunArgs a, int6
   }
 }
 
-// Small runs (<= 2 KiB): one lane per 16-byte piece, many runs per workgroup.
+// Small runs (below 1 KiB by default): one lane per 16-byte piece, many runs per workgroup.
+template <bool NT>
 __global__ __launch_bounds__(kBlock) void copy_small_runs_kernel(const RunArgs a,
                                                                  uint32_t pieces_per_run,
                                                                  int64_t total_pieces) {
@@ -586,7 +587,7 @@ __global__ __launch_bounds__(kBlock) void copy_small_runs_kernel(const RunArgs a
   const uint64_t s = (uint64_t)(a.src + so + lo);
   const uint64_t d = (uint64_t)(a.dst + dof + lo);
   if (n == 16 && (((s | d) & 15) == 0)) {
-    st<false, u32x4>(d, ld<false, u32x4>(s));
+    st<NT, u32x4>(d, ld<NT, u32x4>(s));
   } else {
     for (int64_t i = 0; i < n; ++i)
       st<false, uint8_t>(d + (uint64_t)i, ld<false, uint8_t>(s + (uint64_t)i));
@@ -611,9 +612,18 @@ __device__ __forceinline__ void move_upto16(uint64_t s, uint64_t d, int n) {
 // (y, z) = run; one 16-byte vector per lane; the run's two offsets come in through scalar loads.
 // A run whose addresses are not 16-byte aligned, and the ragged end of a run, fall back to narrower
 // accesses lane by lane.
-template <bool NT, int B>
-__global__ __launch_bounds__(B) void copy_runs_wave_kernel(const RunArgs a) {
-  const uint64_t run = (uint64_t)blockIdx.y + (uint64_t)blockIdx.z * gridDim.y;
+// `group_shift` >= 0 packs 2^group_shift runs into one row of the grid (x = run in group, piece;
+// pieces per run = 2^piece_shift): rows of only a few workgroups dispatch slowly (runs of 2-8 pieces
+// were capped near 4.85 TB/s whatever the kernel did).
+template <bool NTL, bool NTS, int B>
+__global__ __launch_bounds__(B) void copy_runs_wave_kernel(const RunArgs a, int piece_shift,
+                                                           int group_shift) {
+  uint64_t run = (uint64_t)blockIdx.y + (uint64_t)blockIdx.z * gridDim.y;
+  uint32_t piece = blockIdx.x;
+  if (group_shift >= 0) {
+    run = (run << group_shift) + (blockIdx.x >> piece_shift);
+    piece = blockIdx.x & ((1u << piece_shift) - 1u);
+  }
   if (run >= (uint64_t)a.n_runs) return;
   const int64_t so_u = cload(a.src_off + run);
   const int64_t do_u = cload(a.dst_off + run);
@@ -632,19 +642,19 @@ __global__ __launch_bounds__(B) void copy_runs_wave_kernel(const RunArgs a) {
   const bool bad_src = bad_len || so_u < 0 || so < 0 || so > a.src_bytes - rb;
   const bool bad_dst = do_u < 0 || dof < 0 || dof > a.dst_bytes - rb;
   if (bad_src || bad_dst) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
+    if (threadIdx.x == 0 && piece == 0) {
       if (bad_src) raise(a.status, ST_SLOT_SRC);
       if (bad_dst) raise(a.status, ST_SLOT_DST);
     }
     return;
   }
-  const int64_t lo = (int64_t)blockIdx.x * (B * 16) + threadIdx.x * 16;
+  const int64_t lo = (int64_t)piece * (B * 16) + threadIdx.x * 16;
   if (lo >= rb) return;
   const uint64_t s = (uint64_t)(a.src + so + lo);
   const uint64_t d = (uint64_t)(a.dst + dof + lo);
   const int64_t left = rb - lo;
   if (left >= 16 && ((s | d) & 15) == 0) {
-    st<NT, u32x4>(d, ld<NT, u32x4>(s));
+    st<NTS, u32x4>(d, ld<NTL, u32x4>(s));
   } else {
     move_upto16(s, d, left < 16 ? (int)left : 16);
   }
@@ -653,35 +663,54 @@ __global__ __launch_bounds__(B) void copy_runs_wave_kernel(const RunArgs a) {
 template <int B>
 static hipError_t launch_runs_wave(const RunArgs& a, hipStream_t stream) {
   const int64_t piece = (int64_t)B * 16;
-  const int64_t gx = (a.run_bytes + piece - 1) / piece;
+  int64_t gx = (a.run_bytes + piece - 1) / piece;
   if (gx >= (int64_t(1) << 32) / B) return hipErrorInvalidValue;
-  const int64_t gy = a.n_runs < 32768 ? a.n_runs : 32768;
-  const int64_t gz = (a.n_runs + gy - 1) / gy;
+  int64_t rows = a.n_runs;
+  int piece_shift = 0, group_shift = -1;
+  if (gx < 256 && (gx & (gx - 1)) == 0 && tuning().run_group != 0) {
+    while ((int64_t(1) << piece_shift) < gx) ++piece_shift;
+    group_shift = 0;
+    while ((gx << group_shift) < 1024 && (int64_t(1) << group_shift) < a.n_runs) ++group_shift;
+    rows = (a.n_runs + (int64_t(1) << group_shift) - 1) >> group_shift;
+    gx <<= group_shift;
+  }
+  const int64_t gy = rows < 32768 ? rows : 32768;
+  const int64_t gz = (rows + gy - 1) / gy;
   if (gz > 65535) return hipErrorInvalidValue;
   const dim3 grid((uint32_t)gx, (uint32_t)gy, (uint32_t)gz);
-  if (tuning().nontemporal != 0)
-    hipLaunchKernelGGL((copy_runs_wave_kernel<true, B>), grid, dim3(B), 0, stream, a);
+  const int nt = tuning().nontemporal;   // -1/1 both sides, 0 none, 2 loads only, 3 stores only
+  if (nt == 0)
+    hipLaunchKernelGGL((copy_runs_wave_kernel<false, false, B>), grid, dim3(B), 0, stream, a, piece_shift, group_shift);
+  else if (nt == 2)
+    hipLaunchKernelGGL((copy_runs_wave_kernel<true, false, B>), grid, dim3(B), 0, stream, a, piece_shift, group_shift);
+  else if (nt == 3)
+    hipLaunchKernelGGL((copy_runs_wave_kernel<false, true, B>), grid, dim3(B), 0, stream, a, piece_shift, group_shift);
   else
-    hipLaunchKernelGGL((copy_runs_wave_kernel<false, B>), grid, dim3(B), 0, stream, a);
+    hipLaunchKernelGGL((copy_runs_wave_kernel<true, true, B>), grid, dim3(B), 0, stream, a, piece_shift, group_shift);
   return hipGetLastError();
 }
 
 hipError_t launch_copy_runs(const RunArgs& a, hipStream_t stream) {
   if (a.n_runs <= 0 || a.run_bytes <= 0) return hipSuccess;
-  if (a.run_lens || (a.run_bytes > 2048 && tuning().run_chunk_kib == 0)) {
+  const int64_t small_max = tuning().small_run_max;
+  if (a.run_lens || (a.run_bytes > small_max && tuning().run_chunk_kib == 0)) {
     switch (tuning().wave_block) {
       case 128: return launch_runs_wave<128>(a, stream);
       case 256: return launch_runs_wave<256>(a, stream);
       default: return launch_runs_wave<64>(a, stream);
     }
   }
-  if (a.run_bytes <= 2048) {
+  if (a.run_bytes <= small_max) {
     const int64_t ppr = (a.run_bytes + 15) >> 4;
     const int64_t total = ppr * a.n_runs;
     const int64_t grid = (total + kBlock - 1) / kBlock;
     if (grid >= (int64_t(1) << 24)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(copy_small_runs_kernel, dim3((uint32_t)grid), dim3(kBlock), 0, stream, a,
-                       (uint32_t)ppr, total);
+    if (tuning().nontemporal != 0)
+      hipLaunchKernelGGL(copy_small_runs_kernel<true>, dim3((uint32_t)grid), dim3(kBlock), 0, stream, a,
+                         (uint32_t)ppr, total);
+    else
+      hipLaunchKernelGGL(copy_small_runs_kernel<false>, dim3((uint32_t)grid), dim3(kBlock), 0, stream, a,
+                         (uint32_t)ppr, total);
     return hipGetLastError();
   }
   int64_t chunk = (int64_t)tuning().run_chunk_kib * 1024;

@@ -61,8 +61,11 @@ int bikv_check_status(int device, void* stream, uint32_t* bits_out);
  * -1 = default: chosen from the batch's layout hint), "log2_chunk" (order 1: pages per chunk,
  * -1 = chosen),
  * "unroll" (segment mover: 16-byte vectors in flight per lane: 1, 2, 4, 8), "nontemporal" (nt hint on
- * payload accesses: 1 on, 0 off, -1 = default: chosen per direction and layout),
- * "run_chunk_kib" (bytes of a run per workgroup, KiB; 0 = automatic), "transpose_lds_kib" and
+ * payload accesses: 1 on, 0 off, -1 = default: chosen per direction and layout; the run copy also
+ * takes 2 = loads only, 3 = stores only),
+ * "run_chunk_kib" (bytes of a run per workgroup, KiB; 0 = automatic), "small_run_max" (runs up to this
+ * many bytes use one lane per 16-byte piece instead of one wave per KiB), "run_group" (1 = several
+ * short runs share a row of the launch grid, default; 0 = one row per run), "transpose_lds_kib" and
  * "transpose_dsplit" (LDS tile budget and head_dim slices of the layout-change kernel),
  * "transpose_pairs" (2-byte elements with head_dim % 32 == 0: 1 = the word-pair kernel, default;
  * 0 = the element-wise kernel) and "transpose_block" (its lanes per workgroup: 128, 256, 512, 1024).

@@ -358,9 +358,12 @@ def test_tuning_knobs_do_not_change_results(bk, oracle, cuda):
 # ---- run copy (reference API) -------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,run_elems", [
     (torch.float16, 14336 * 16), (torch.bfloat16, 4096), (torch.float32, 1000), (torch.float64, 33),
-    (torch.uint8, 5), (torch.uint8, 2049), (torch.float16, 8), (torch.float16, 1029)])
-def test_copy_runs_gather_and_scatter(bk, oracle, cuda, dtype, run_elems):
-    _announce(f"copy_runs {dtype} run_elems={run_elems}")
+    (torch.uint8, 5), (torch.uint8, 2049), (torch.float16, 8), (torch.float16, 1029),
+    (torch.float16, 512), (torch.uint8, 1023), (torch.uint8, 16384)])
+@pytest.mark.parametrize("run_group", [1, 0])
+def test_copy_runs_gather_and_scatter(bk, oracle, cuda, dtype, run_elems, run_group):
+    _announce(f"copy_runs {dtype} run_elems={run_elems} run_group={run_group}")
+    bk.set_tuning(run_group=run_group)
     rng = np.random.default_rng(run_elems)
     es = torch.empty((), dtype=dtype).element_size()
     n_pages, n = 37, 19
@@ -385,6 +388,7 @@ def test_copy_runs_gather_and_scatter(bk, oracle, cuda, dtype, run_elems):
     pool2_h = np.zeros_like(src_h)
     oracle.copy_runs_c(dst_h.view(np_dt), pool2_h.view(np_dt), do, back_ids, run_elems)
     assert _to_np(pool2_d).tobytes() == pool2_h.tobytes()
+    bk.set_tuning(run_group=1)
 
 
 def test_copy_runs_element_offsets_that_break_16_byte_alignment(bk, oracle, cuda):
