@@ -34,7 +34,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch as a multiple of the algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this file, each scaled by the same counter's reading for the plain-copy
 # calibration launch below (summaries under profiles/). None = not measured for that workload.
-MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9954, "scatter": 1.0001}}
+MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9949, "scatter": 1.0003}}
 
 
 def parse_args():

@@ -147,7 +147,7 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
     if (value < -1 || value > 16) return fail(BIKV_EINVAL, "log2_chunk must be in [-1, 16]");
     t.log2_chunk = (int)value;
   } else if (!strcmp(key, "nontemporal")) {
-    if (value > 3) return fail(BIKV_EINVAL, "nontemporal must be -1, 0, 1, 2 (loads only) or 3 (stores only)");
+    if (value > 4) return fail(BIKV_EINVAL, "nontemporal must be -1, 0, 1, 2 (loads only), 3 (stores only) or 4 (nt + sc1)");
     t.nontemporal = value < 0 ? -1 : (int)value;
   } else if (!strcmp(key, "transpose_lds_kib")) {
     if (value < 2 || value > 60) return fail(BIKV_EINVAL, "transpose_lds_kib must be in [2, 60]");

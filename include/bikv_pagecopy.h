@@ -61,8 +61,8 @@ int bikv_check_status(int device, void* stream, uint32_t* bits_out);
  * -1 = default: chosen from the batch's layout hint), "log2_chunk" (order 1: pages per chunk,
  * -1 = chosen),
  * "unroll" (segment mover: 16-byte vectors in flight per lane: 1, 2, 4, 8), "nontemporal" (nt hint on
- * payload accesses: 1 on, 0 off, -1 = default: chosen per direction and layout; the run copy also
- * takes 2 = loads only, 3 = stores only),
+ * payload accesses: 1 on, 0 off, 4 = nt with system scope, -1 = default: chosen per direction and
+ * layout; the run copy also takes 2 = loads only, 3 = stores only),
  * "run_chunk_kib" (bytes of a run per workgroup, KiB; 0 = automatic), "small_run_max" (runs up to this
  * many bytes use one lane per 16-byte piece instead of one wave per KiB), "run_group" (1 = several
  * short runs share a row of the launch grid, default; 0 = one row per run), "transpose_lds_kib" and

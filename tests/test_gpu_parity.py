@@ -335,7 +335,7 @@ def test_tuning_knobs_do_not_change_results(bk, oracle, cuda):
     oracle.scatter_layered_c(want_pool, sreqs, src.cpu().numpy())
     try:
         # seg 0 = wave mover (wave_block lanes per workgroup); seg > 0 = LDS-staged segment mover
-        cases = [dict(seg=0, wave_block=wb, nontemporal=nt) for wb in (64, 128, 256) for nt in (-1, 0, 1)]
+        cases = [dict(seg=0, wave_block=wb, nontemporal=nt) for wb in (64, 128, 256) for nt in (-1, 0, 1, 4)]
         # wave mover walks: plane by plane, or chunks of 2^k pages with their planes together
         cases += [dict(seg=0, wave_block=64, order=o, log2_chunk=lc) for o in (0, 1) for lc in (-1, 0, 1, 3, 6, 10)]
         cases += [dict(seg=seg, unroll=u, nontemporal=nt) for seg in (1, 3, 16, 256) for u in (1, 2, 4, 8)
