@@ -58,7 +58,7 @@ def parse_args():
     ap.add_argument("--log2-chunk", dest="log2_chunk", type=int, default=None)
     ap.add_argument("--staging-cap-gb", dest="staging_cap_gb", type=float, default=32.0,
                     help="largest staging buffer of one launch; bigger batches take several launches")
-    ap.add_argument("--chunk-mib", type=int, default=8, help="staging pipeline chunk (llama3_8b)")
+    ap.add_argument("--chunk-mib", type=int, default=32, help="staging pipeline chunk (llama3_8b)")
     ap.add_argument("--buffers", type=int, default=2, help="staging pipeline lanes (stream + HBM chunk each)")
     return ap.parse_args()
 

@@ -24,7 +24,7 @@ def pinned_empty(nbytes: int) -> torch.Tensor:
 
 
 class HostStager:
-    def __init__(self, device, chunk_bytes: int = 8 << 20, n_buffers: int = 2):
+    def __init__(self, device, chunk_bytes: int = 32 << 20, n_buffers: int = 2):
         self.device = torch.device(device)
         self.chunk_bytes = int(chunk_bytes)
         self.n_buffers = int(n_buffers)
