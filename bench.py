@@ -486,8 +486,27 @@ def run_reference_scenario(args, bk, dev):
     nbytes = cache.numel() * 2
     zero_copy = {"GBps": round(nbytes / (min(zc) * 1e-3) / 1e9, 2),
                  "plain_pinned_h2d_GBps": round(nbytes / (min(h2d) * 1e-3) / 1e9, 2)}
+    # the same launches captured once in a HIP graph and replayed: what a serving loop pays per transfer
+    # once the Python and launch overhead is taken out of the loop
+    out.zero_()
+    side = torch.cuda.Stream(device=dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(args.steps):
+                bk.copy_runs(cache, out, offs, offs, page_elements)
+    graph.replay()
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize(dev)
+    graph_wall = time.perf_counter() - t0
+    if not torch.equal(out, cache):
+        raise SystemExit("bench: graph replay mismatch")
     return {
         "zero_copy_from_pinned_host": zero_copy,
+        "graph_replay": {"GBps": round(alg / (graph_wall / args.steps) / 1e9, 1),
+                         "ms_per_launch": round(graph_wall * 1e3 / args.steps, 4)},
         "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
         "value": round(alg / (wall / args.steps) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True,

@@ -496,3 +496,55 @@ def test_copy_runs_zero_copy_from_pinned_host(bk, oracle, cuda):
     want = np.zeros(7 * run, dtype=np.uint16)
     oracle.copy_runs_c(src_h, want, so, do, run)
     assert _to_np(dst).tobytes() == want.tobytes()
+
+
+# ---- HIP graph capture --------------------------------------------------------------------------
+def test_gather_scatter_and_run_copy_replay_from_a_hip_graph(bk, oracle, cuda):
+    """The asynchronous entry points only launch kernels (no allocation, no memset, no synchronisation),
+    so a serving loop can capture them once and replay: every replay is checked against the oracle with
+    different pool contents, with eager work and synchronisations between the replays."""
+    _announce("graph capture: gather + scatter + copy_runs")
+    from bikv_pagecopy import runs
+    rng = np.random.default_rng(71)
+    n_planes, n_pages, tile = 6, 64, 8192
+    pool_h = rng.integers(0, 256, size=(n_planes, n_pages, tile), dtype=np.uint8)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    perm = rng.permutation(n_pages)
+    g_reqs = [perm[:9], perm[5:20]]                       # overlapping requests: duplicate reads
+    s_reqs = [perm[30:39], perm[40:55]]                   # unique, disjoint from the gathered pages
+    gb, sb = pool.make_batch(g_reqs, "layer_major"), pool.make_batch(s_reqs, "layer_major")
+    st, _ = pool.empty_staging(gb)
+    run = tile // 2
+    so = torch.from_numpy(np.arange(0, 4 * run, run, dtype=np.int64)).to(cuda)
+    do = torch.from_numpy(np.array([3, 1, 0, 2], dtype=np.int64) * run).to(cuda)
+    copy_out = torch.zeros(4 * run, dtype=torch.float16, device=cuda)
+    # one eager pass first: per-device set-up (the status block) happens outside the capture
+    pool.gather(gb, st)
+    pool.check()
+    stream = torch.cuda.Stream(device=cuda)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            pool.gather(gb, st)
+            pool.scatter(sb, st)
+            bk.copy_runs(st.view(torch.float16), copy_out, so, do, run)
+    for rep in range(3):
+        pool_h = rng.integers(0, 256, size=(n_planes, n_pages, tile), dtype=np.uint8)
+        pool_d.copy_(torch.from_numpy(pool_h))            # eager work between replays
+        st.fill_(0xA5)
+        copy_out.zero_()
+        torch.cuda.synchronize(cuda)
+        graph.replay()
+        torch.cuda.synchronize(cuda)
+        pool.check()
+        staged = oracle.gather_layered_c(pool_h, g_reqs, "layer_major")
+        want_pool = pool_h.copy()
+        oracle.scatter_layered_c(want_pool, s_reqs, staged, "layer_major")
+        assert _to_np(st).tobytes() == staged.tobytes(), rep
+        assert _to_np(pool_d).tobytes() == want_pool.tobytes(), rep
+        want_copy = np.zeros(4 * run, dtype=np.uint16)
+        oracle.copy_runs_c(staged.view(np.uint16).reshape(-1), want_copy, so.cpu().numpy(), do.cpu().numpy(), run)
+        assert _to_np(copy_out).tobytes() == want_copy.tobytes(), rep
+    runs.check(cuda)
+    pool.close()
