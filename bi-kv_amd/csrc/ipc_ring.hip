@@ -272,7 +272,7 @@ extern "C" void bikv_consumer_cleanup(void) {
     bikv_producer_cleanup();
   }
   if (g_consumer.mem) {
-    (void)hipSetDevice(g_consumer.device);
+    DeviceGuard guard_(g_consumer.device);
     (void)hipFree(g_consumer.mem);
     g_consumer.mem = nullptr;
   }
@@ -304,7 +304,7 @@ static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_
   const int64_t data_size = total_tokens * token_bytes;
   if ((size_t)data_size > c->buffer_size)
     return fail(BIKV_ERANGE, "batch of %lld bytes does not fit the %zu-byte ring", (long long)data_size, c->buffer_size);
-  BIKV_HIP(hipSetDevice(g_producer.device));
+  BIKV_DEVICE(g_producer.device);
   size_t at = 0;
   {
     const int rc = producer_reserve(g_producer, (size_t)data_size, &at);
@@ -360,7 +360,7 @@ extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64
   bikv_shared_control* c = g_producer.ctrl;
   if (bytes > c->buffer_size)
     return fail(BIKV_ERANGE, "tensor of %zu bytes does not fit the %zu-byte ring", bytes, c->buffer_size);
-  BIKV_HIP(hipSetDevice(g_producer.device));
+  BIKV_DEVICE(g_producer.device);
   size_t at = 0;
   {
     const int rc = producer_reserve(g_producer, bytes, &at);

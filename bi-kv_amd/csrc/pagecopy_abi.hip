@@ -42,7 +42,7 @@ int device_status(int device, uint32_t** dev_ptr) {
   std::lock_guard<std::mutex> lk(g_ctx_mu);
   DevCtx& c = g_ctx[device];
   if (!c.status_host) {
-    BIKV_HIP(hipSetDevice(device));
+    BIKV_DEVICE(device);
     void* h = nullptr;
     BIKV_HIP(hipHostMalloc(&h, ST_SLOTS * sizeof(uint32_t) * 8, hipHostMallocMapped | hipHostMallocPortable));
     memset(h, 0, ST_SLOTS * sizeof(uint32_t) * 8);
@@ -119,7 +119,7 @@ extern "C" const char* bikv_last_error(void) { return g_err; }
 
 extern "C" int bikv_check_status(int device, void* stream, uint32_t* bits_out) {
   if (device < 0 || device >= 64) return fail(BIKV_EINVAL, "device index %d out of range", device);
-  BIKV_HIP(hipSetDevice(device));
+  BIKV_DEVICE(device);
   BIKV_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   const uint32_t bits = take_status(device);
   if (bits_out) *bits_out = bits;
@@ -207,7 +207,7 @@ extern "C" int bikv_pool_create(const bikv_pool_desc* d, bikv_pool** out) {
   uint32_t* st = nullptr;
   int rc = device_status(d->device, &st);
   if (rc) return rc;
-  BIKV_HIP(hipSetDevice(d->device));
+  BIKV_DEVICE(d->device);
   void* dtab = nullptr;
   BIKV_HIP(hipMalloc(&dtab, table.size() * sizeof(char*)));
   hipError_t e = hipMemcpy(dtab, table.data(), table.size() * sizeof(char*), hipMemcpyHostToDevice);
@@ -232,7 +232,7 @@ extern "C" int bikv_pool_create(const bikv_pool_desc* d, bikv_pool** out) {
 
 extern "C" int bikv_pool_destroy(bikv_pool* p) {
   if (!p) return BIKV_OK;
-  (void)hipSetDevice(p->device);
+  DeviceGuard guard_(p->device);
   hipError_t e = hipFree((void*)p->d_plane_base);
   delete p;
   if (e != hipSuccess) return fail_hip(e, "hipFree(plane table)");
@@ -297,7 +297,7 @@ static int move_pages(int dir, const bikv_pool* pool, const bikv_page_batch* b, 
   int rc = build_move(pool, b, staging, staging_bytes, scale_staging, scale_bytes, &m);
   if (rc) return rc;
   if (m.n_batch == 0) return BIKV_OK;
-  BIKV_HIP(hipSetDevice(pool->device));
+  BIKV_DEVICE(pool->device);
   hipError_t e = launch_tile_move(dir, m, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail_hip(e, dir == 0 ? "gather launch" : "scatter launch");
   return BIKV_OK;
@@ -382,7 +382,7 @@ extern "C" int bikv_host_free(void* p) {
 static int link_copy(int device, void* dst, const void* src, int64_t bytes, int64_t chunk_bytes,
                      hipMemcpyKind kind, double* seconds_out) {
   if (!dst || !src || bytes <= 0) return fail(BIKV_EINVAL, "bad host-link copy arguments");
-  BIKV_HIP(hipSetDevice(device));
+  BIKV_DEVICE(device);
   hipStream_t s;
   BIKV_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
   if (chunk_bytes <= 0) chunk_bytes = bytes;
@@ -437,7 +437,7 @@ extern "C" int bikv_stager_create(int device, int64_t chunk_bytes, int32_t n_buf
   uint32_t* st_ptr = nullptr;
   int rc = device_status(device, &st_ptr);
   if (rc) return rc;
-  BIKV_HIP(hipSetDevice(device));
+  BIKV_DEVICE(device);
   bikv_stager* st = new bikv_stager();
   st->device = device;
   st->chunk_bytes = chunk_bytes;
@@ -461,7 +461,7 @@ extern "C" int bikv_stager_create(int device, int64_t chunk_bytes, int32_t n_buf
 
 extern "C" int bikv_stager_destroy(bikv_stager* st) {
   if (!st) return BIKV_OK;
-  (void)hipSetDevice(st->device);
+  DeviceGuard guard_(st->device);
   for (hipStream_t s : st->lanes) {
     (void)hipStreamSynchronize(s);
     (void)hipStreamDestroy(s);
@@ -591,7 +591,7 @@ static int stage_between_host(int dir, bikv_stager* st, const bikv_pool* pool,
                 (long long)host_scale_bytes, (long long)scale_image_bytes);
   if (stats) { stats->bytes = 0; stats->n_chunks = 0; stats->wall_seconds = 0.0; }
   if (total_pages == 0) return BIKV_OK;
-  BIKV_HIP(hipSetDevice(st->device));
+  BIKV_DEVICE(st->device);
   const auto t0 = std::chrono::steady_clock::now();
 
   if (mode == BIKV_STAGE_DIRECT) {
@@ -753,7 +753,7 @@ extern "C" int bikv_nhd_create(const bikv_nhd_desc* d, bikv_nhd** out) {
   uint32_t* st = nullptr;
   int rc = device_status(d->device, &st);
   if (rc) return rc;
-  BIKV_HIP(hipSetDevice(d->device));
+  BIKV_DEVICE(d->device);
   void* dtab = nullptr;
   BIKV_HIP(hipMalloc(&dtab, table.size() * sizeof(char*)));
   hipError_t e = hipMemcpy(dtab, table.data(), table.size() * sizeof(char*), hipMemcpyHostToDevice);
@@ -779,7 +779,7 @@ extern "C" int bikv_nhd_create(const bikv_nhd_desc* d, bikv_nhd** out) {
 
 extern "C" int bikv_nhd_destroy(bikv_nhd* p) {
   if (!p) return BIKV_OK;
-  (void)hipSetDevice(p->device);
+  DeviceGuard guard_(p->device);
   hipError_t e = hipFree((void*)p->d_layer_base);
   delete p;
   if (e != hipSuccess) return fail_hip(e, "hipFree(layer table)");
@@ -816,7 +816,7 @@ static int transpose_pages(int dir, const bikv_nhd* nhd, void* tm, int64_t tm_by
   a.elem_bytes = nhd->elem_bytes;
   int rc = device_status(nhd->device, &a.status);
   if (rc) return rc;
-  BIKV_HIP(hipSetDevice(nhd->device));
+  BIKV_DEVICE(nhd->device);
   hipError_t e = launch_transpose_pages(dir, a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail_hip(e, "layout-change launch");
   return BIKV_OK;
