@@ -548,3 +548,15 @@ def test_gather_scatter_and_run_copy_replay_from_a_hip_graph(bk, oracle, cuda):
         assert _to_np(copy_out).tobytes() == want_copy.tobytes(), rep
     runs.check(cuda)
     pool.close()
+
+
+def test_plain_c_program_drives_the_library(bk, cuda):
+    """tests/c_client/abi_client.c: gcc-built, includes only include/bikv_pagecopy.h, links only the
+    shared library. Run copy, ragged run copy, layered gather/scatter and a rejected page id."""
+    import os
+    import subprocess
+    _announce("plain-C client of the ABI")
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_client", "abi_client")
+    assert os.path.exists(exe), "tests/c_client/abi_client is not built (make -C tests/c_client)"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0 and "abi_client: ok" in r.stdout, (r.returncode, r.stdout, r.stderr)

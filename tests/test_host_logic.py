@@ -297,3 +297,16 @@ def test_build_run_offsets_can_return_the_tokens_of_each_run():
     assert total2 == total and np.array_equal(off2, off[:2])
     e, t0 = build_run_offsets([], [], 16, with_sizes=True)
     assert e.shape == (3, 0) and t0 == 0
+
+
+def test_plain_c_client_compiles_against_the_header_alone():
+    """The C client used by the GPU suite must build with gcc -std=c99 -pedantic from the public header
+    (no HIP headers on the include path)."""
+    import subprocess
+    import tempfile
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with tempfile.TemporaryDirectory() as tmp:
+        r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(root, "include"),
+                            "-c", os.path.join(root, "tests", "c_client", "abi_client.c"), "-o", os.path.join(tmp, "c.o")],
+                           capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr
