@@ -57,7 +57,7 @@ struct Tuning {
   int transpose_dsplit = 0;    // slices of head_dim per tile; 0 = default (1: whole compute rows)
 int run_group = 1;         // wave run kernel: pack several short runs into one grid row (0 = off)
   int small_run_max = 1023;  // runs up to this many bytes go to the one-lane-per-piece kernel
-    int transpose_pairs = 1;  // 2-byte elements: the word-pair kernel (0 = element-wise kernel)
+    int transpose_pairs = 1;  // the K/V-pair kernel where the shape allows (0 = element-wise kernel)
   int transpose_block = 512; // lanes per workgroup of the word-pair kernel: 128, 256, 512, 1024
 };
 Tuning& tuning();

@@ -154,17 +154,20 @@ __global__ __launch_bounds__(kBlock) void transpose_pages_kernel(const Transpose
   }
 }
 
-// ---- 2-byte elements, K/V pairs as 32-bit words -----------------------------------------------
+// ---- K/V pairs as units -------------------------------------------------------------------------
 // Column c = (h*L + l)*2 + k puts the K and the V element of one (head, layer) next to each other,
-// so a token row is a sequence of 32-bit words {K[d], V[d]} and the layout change is a transpose
-// of WORDS ([D][C/2] -> [C/2][D]) followed by a de-interleave of 16-bit halves in registers.
-// LDS holds the tile transposed, [column pair][d] words, no padding; the 4-word groups of a row
-// are permuted by XOR with (pair/4 mod 8), which keeps 16-byte LDS accesses along d intact and
-// spreads the word-wise accesses of the other side (lanes walk a token-major row: pair index steps
-// by 4) over all banks. Per 16-byte vector moved this takes 5 LDS instructions and ~30 VALU
-// instructions; the element-wise kernel above takes 11 and ~100 (three integer divisions).
-// Needs head_dim % 32 == 0 (XOR closure over the groups of a row).
-struct Walk {        // (outer, inner) of a linear index that advances by kBlock per step
+// so a token row is a sequence of UNITS {K[d], V[d]} of 2*ES bytes and the layout change is a
+// transpose of units ([D][C/2] -> [C/2][D]) followed by a split of each unit in registers.
+// LDS holds the tile transposed, [column pair][d] units, no padding. A lane on the compute side
+// reads 32 contiguous bytes of a pair's row (16/ES values of d) and turns them into one K vector and
+// one V vector; a lane on the token-major side moves the 16/(2*ES) units of one vector to or from as
+// many pair rows. The 16-byte groups of a row are permuted by XOR with (vector index mod 8), which
+// keeps the 16-byte accesses along d intact and spreads the unit-wise accesses of the other side
+// (consecutive lanes = consecutive vectors of a token-major row) over all banks. For 2-byte elements
+// this takes 5.5 LDS and ~60 VALU instructions per 16-byte vector moved; the element-wise kernel
+// above takes 11 and ~105 (three integer divisions per vector).
+// Needs head_dim * ES % 64 == 0 (XOR closure over the 16-byte groups of a row).
+struct Walk {        // (outer, inner) of a linear index that advances by the block size per step
   int outer, inner;
 };
 __device__ __forceinline__ Walk walk_start(int idx, int n_inner) {
@@ -182,10 +185,60 @@ __device__ __forceinline__ void walk_step(Walk& w, int q, int r, int n_inner) {
   }
 }
 
-template <int DIR, int B>
+// 32 bytes of units {K,V} (g0 = the first 16, g1 = the next 16) -> a K vector and a V vector.
+template <int ES>
+__device__ __forceinline__ void split_kv(const u32x4& g0, const u32x4& g1, u32x4& kx, u32x4& vx) {
+  if constexpr (ES == 4) {
+    kx = u32x4{g0.x, g0.z, g1.x, g1.z};
+    vx = u32x4{g0.y, g0.w, g1.y, g1.w};
+  } else {
+    constexpr uint32_t SK = ES == 2 ? 0x05040100u : 0x06040200u;   // K halves / K bytes of two words
+    constexpr uint32_t SV = ES == 2 ? 0x07060302u : 0x07050301u;
+    kx.x = __builtin_amdgcn_perm(g0.y, g0.x, SK);
+    kx.y = __builtin_amdgcn_perm(g0.w, g0.z, SK);
+    kx.z = __builtin_amdgcn_perm(g1.y, g1.x, SK);
+    kx.w = __builtin_amdgcn_perm(g1.w, g1.z, SK);
+    vx.x = __builtin_amdgcn_perm(g0.y, g0.x, SV);
+    vx.y = __builtin_amdgcn_perm(g0.w, g0.z, SV);
+    vx.z = __builtin_amdgcn_perm(g1.y, g1.x, SV);
+    vx.w = __builtin_amdgcn_perm(g1.w, g1.z, SV);
+  }
+}
+// The inverse: a K vector and a V vector -> 32 bytes of units.
+template <int ES>
+__device__ __forceinline__ void join_kv(const u32x4& kx, const u32x4& vx, u32x4& g0, u32x4& g1) {
+  if constexpr (ES == 4) {
+    g0 = u32x4{kx.x, vx.x, kx.y, vx.y};
+    g1 = u32x4{kx.z, vx.z, kx.w, vx.w};
+  } else {
+    constexpr uint32_t SL = ES == 2 ? 0x05040100u : 0x05010400u;   // units from the low / high half of
+    constexpr uint32_t SH = ES == 2 ? 0x07060302u : 0x07030602u;   // a K word and a V word
+    g0.x = __builtin_amdgcn_perm(vx.x, kx.x, SL);
+    g0.y = __builtin_amdgcn_perm(vx.x, kx.x, SH);
+    g0.z = __builtin_amdgcn_perm(vx.y, kx.y, SL);
+    g0.w = __builtin_amdgcn_perm(vx.y, kx.y, SH);
+    g1.x = __builtin_amdgcn_perm(vx.z, kx.z, SL);
+    g1.y = __builtin_amdgcn_perm(vx.z, kx.z, SH);
+    g1.z = __builtin_amdgcn_perm(vx.w, kx.w, SL);
+    g1.w = __builtin_amdgcn_perm(vx.w, kx.w, SH);
+  }
+}
+
+template <int ES> struct UnitOf;
+template <> struct UnitOf<1> { using T = uint16_t; };
+template <> struct UnitOf<2> { using T = uint32_t; };
+template <> struct UnitOf<4> { using T = uint64_t; };
+
+template <int DIR, int ES, int B>
 __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs a) {
+  using Unit = typename UnitOf<ES>::T;
+  constexpr int UB = 2 * ES;               // bytes of a unit
+  constexpr int UPV = 16 / UB;             // units in a 16-byte vector
+  constexpr int UPV_SHIFT = ES == 1 ? 3 : (ES == 2 ? 2 : 1);
+  constexpr int DPV = 16 / ES;             // values of d in a compute-side vector
   extern __shared__ uint32_t lds_words[];
   u32x4* lds_vec = reinterpret_cast<u32x4*>(lds_words);
+  Unit* lds_unit = reinterpret_cast<Unit*>(lds_words);
   uint64_t* row_addr = reinterpret_cast<uint64_t*>(lds_words + a.tile_words);  // K row of each pair
 
   const uint32_t chunk = blockIdx.x % a.n_chunks;              // column chunk
@@ -205,8 +258,9 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
   }
   const int D = a.head_dim, C = a.n_cols;
   const int Cw = a.chunk_cols >> 1;        // column pairs in the tile
-  const int vpr = a.chunk_cols >> 3;       // 16-byte vectors per token-major row piece
-  const int dgs = D >> 3;                  // 16-byte vectors per compute row
+  const int vpr = Cw >> UPV_SHIFT;         // 16-byte vectors per token-major row piece
+  const int dgs = D / DPV;                 // 16-byte vectors per compute row
+  const int gpr = (D * UB) >> 4;           // 16-byte groups per LDS row (a multiple of 8)
   const int cp0 = (int)chunk * Cw;
   // The compute side is walked layer by layer (all heads of a layer, K rows then V rows, are
   // neighbours in memory), the LDS tile is indexed by column pair (head-major): entry j of the table
@@ -225,18 +279,19 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
       l = (cp0 + cp) - h * a.n_layers;
     }
     const int64_t off = blk * a.block_stride + (int64_t)t * a.token_stride + (int64_t)h * a.head_dim;
-    row_addr[j] = ((uint64_t)a.layer_base[l] + (uint64_t)off * 2) | ((uint64_t)cp << 48);
+    row_addr[j] = ((uint64_t)a.layer_base[l] + (uint64_t)off * ES) | ((uint64_t)cp << 48);
   }
-  const uint64_t kv_bytes = (uint64_t)a.kv_stride * 2;
+  const uint64_t kv_bytes = (uint64_t)a.kv_stride * ES;
   const uint64_t tm_tok = (uint64_t)a.tm_base +
-                          (((uint64_t)(tmp * a.block_tokens + t) * D) * C + (uint64_t)cp0 * 2) * 2;
-  const uint64_t tm_row_bytes = (uint64_t)C * 2;
+                          (((uint64_t)(tmp * a.block_tokens + t) * D) * C + (uint64_t)cp0 * 2) * ES;
+  const uint64_t tm_row_bytes = (uint64_t)C * ES;
   const int n_tm = D * vpr;                // vectors on the token-major side
-  const int n_cp = Cw * dgs;               // (pair, 8 d) items on the compute side
-  // LDS word index of (pair cp, d): cp*D + (d ^ (((cp >> 2) & 7) << 2))
+  const int n_cp = Cw * dgs;               // (pair, 16/ES values of d) items on the compute side
+  // Unit (pair cp, d) sits in group (d / (UPV)) ^ s of row cp, s = (cp / UPV) & 7 = the index of the
+  // token-major vector the pair belongs to, mod 8.
 
   if (DIR == 1) {
-    // token-major rows -> LDS, four words of a vector to four pair rows
+    // token-major rows -> LDS, the units of a vector to as many pair rows
     constexpr int U = 8;
     const int q = B / vpr, r = B - q * vpr;
     Walk w = walk_start(threadIdx.x, vpr);                     // (d, vector within the row piece)
@@ -254,38 +309,32 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         if (w.outer < D) {
-          const int cv = w.inner;
-          uint32_t* row = lds_words + (cv * 4) * D + (w.outer ^ ((cv & 7) << 2));
-          row[0] = x[u].x;
-          row[D] = x[u].y;
-          row[2 * D] = x[u].z;
-          row[3 * D] = x[u].w;
+          const int cv = w.inner, d = w.outer;
+          // unit index inside row (cv*UPV + j): group (d/UPV ^ s) * UPV + d % UPV
+          Unit* row = lds_unit + (cv * UPV) * D + ((((d >> UPV_SHIFT) ^ (cv & 7)) << UPV_SHIFT) | (d & (UPV - 1)));
+          Unit e[UPV];
+          __builtin_memcpy(e, &x[u], 16);
+#pragma unroll
+          for (int j = 0; j < UPV; ++j) row[j * D] = e[j];
         }
         walk_step(w, q, r, vpr);
       }
     }
     __syncthreads();
-    // LDS -> compute rows: 8 words {K[d],V[d]} become one K vector and one V vector
+    // LDS -> compute rows: 32 bytes of units become one K vector and one V vector
     const int q2 = B / dgs, r2 = B - q2 * dgs;
-    Walk o = walk_start(threadIdx.x, dgs);                     // (pair, 8-d group)
+    Walk o = walk_start(threadIdx.x, dgs);                     // (pair, group of d)
     for (int base = 0; base < n_cp; base += B) {
       if (o.outer < Cw) {
         const uint64_t entry = row_addr[o.outer];
         const int cp = (int)(entry >> 48), dg = o.inner;
-        const int s = (cp >> 2) & 7;
+        const int s = (cp >> UPV_SHIFT) & 7;
         const int flip = (dg >> 2) & 1;                        // lanes 0-3 and 4-7 start on different halves
-        const u32x4 lo = lds_vec[(cp * D >> 2) + ((2 * dg + flip) ^ s)];
-        const u32x4 hi = lds_vec[(cp * D >> 2) + ((2 * dg + 1 - flip) ^ s)];
-        const u32x4 g0 = flip ? hi : lo, g1 = flip ? lo : hi;  // words d..d+3, d+4..d+7
+        const u32x4 lo = lds_vec[cp * gpr + ((2 * dg + flip) ^ s)];
+        const u32x4 hi = lds_vec[cp * gpr + ((2 * dg + 1 - flip) ^ s)];
+        const u32x4 g0 = flip ? hi : lo, g1 = flip ? lo : hi;
         u32x4 kx, vx;
-        kx.x = __builtin_amdgcn_perm(g0.y, g0.x, 0x05040100u);
-        kx.y = __builtin_amdgcn_perm(g0.w, g0.z, 0x05040100u);
-        kx.z = __builtin_amdgcn_perm(g1.y, g1.x, 0x05040100u);
-        kx.w = __builtin_amdgcn_perm(g1.w, g1.z, 0x05040100u);
-        vx.x = __builtin_amdgcn_perm(g0.y, g0.x, 0x07060302u);
-        vx.y = __builtin_amdgcn_perm(g0.w, g0.z, 0x07060302u);
-        vx.z = __builtin_amdgcn_perm(g1.y, g1.x, 0x07060302u);
-        vx.w = __builtin_amdgcn_perm(g1.w, g1.z, 0x07060302u);
+        split_kv<ES>(g0, g1, kx, vx);
         const uint64_t ra = (entry & 0xFFFFFFFFFFFFull) + (uint64_t)dg * 16;
         __builtin_nontemporal_store(kx, (BIKV_GLOBAL u32x4*)ra);
         __builtin_nontemporal_store(vx, (BIKV_GLOBAL u32x4*)(ra + kv_bytes));
@@ -293,7 +342,7 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
       walk_step(o, q2, r2, dgs);
     }
   } else {
-    // compute rows -> LDS: a K vector and a V vector interleave into 8 words
+    // compute rows -> LDS: a K vector and a V vector interleave into 32 bytes of units
     __syncthreads();                                            // row_addr
     constexpr int U = 4;
     const int q2 = B / dgs, r2 = B - q2 * dgs;
@@ -313,18 +362,11 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
       for (int u = 0; u < U; ++u) {
         if (o.outer < Cw) {
           const int cp = (int)(row_addr[o.outer] >> 48), dg = o.inner;
-          const int s = (cp >> 2) & 7;
+          const int s = (cp >> UPV_SHIFT) & 7;
           u32x4 g0, g1;
-          g0.x = __builtin_amdgcn_perm(vx[u].x, kx[u].x, 0x05040100u);
-          g0.y = __builtin_amdgcn_perm(vx[u].x, kx[u].x, 0x07060302u);
-          g0.z = __builtin_amdgcn_perm(vx[u].y, kx[u].y, 0x05040100u);
-          g0.w = __builtin_amdgcn_perm(vx[u].y, kx[u].y, 0x07060302u);
-          g1.x = __builtin_amdgcn_perm(vx[u].z, kx[u].z, 0x05040100u);
-          g1.y = __builtin_amdgcn_perm(vx[u].z, kx[u].z, 0x07060302u);
-          g1.z = __builtin_amdgcn_perm(vx[u].w, kx[u].w, 0x05040100u);
-          g1.w = __builtin_amdgcn_perm(vx[u].w, kx[u].w, 0x07060302u);
-          lds_vec[(cp * D >> 2) + ((2 * dg) ^ s)] = g0;
-          lds_vec[(cp * D >> 2) + ((2 * dg + 1) ^ s)] = g1;
+          join_kv<ES>(kx[u], vx[u], g0, g1);
+          lds_vec[cp * gpr + ((2 * dg) ^ s)] = g0;
+          lds_vec[cp * gpr + ((2 * dg + 1) ^ s)] = g1;
         }
         walk_step(o, q2, r2, dgs);
       }
@@ -334,11 +376,15 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
     Walk w = walk_start(threadIdx.x, vpr);
     for (int base = 0; base < n_tm; base += B) {
       if (w.outer < D) {
-        const int cv = w.inner;
-        const uint32_t* row = lds_words + (cv * 4) * D + (w.outer ^ ((cv & 7) << 2));
-        u32x4 x = {row[0], row[D], row[2 * D], row[3 * D]};
+        const int cv = w.inner, d = w.outer;
+        const Unit* row = lds_unit + (cv * UPV) * D + ((((d >> UPV_SHIFT) ^ (cv & 7)) << UPV_SHIFT) | (d & (UPV - 1)));
+        Unit e[UPV];
+#pragma unroll
+        for (int j = 0; j < UPV; ++j) e[j] = row[j * D];
+        u32x4 x;
+        __builtin_memcpy(&x, e, 16);
         __builtin_nontemporal_store(
-            x, (BIKV_GLOBAL u32x4*)(tm_tok + (uint64_t)w.outer * tm_row_bytes + (uint64_t)cv * 16));
+            x, (BIKV_GLOBAL u32x4*)(tm_tok + (uint64_t)d * tm_row_bytes + (uint64_t)cv * 16));
       }
       walk_step(w, q, r, vpr);
     }
@@ -371,19 +417,19 @@ hipError_t launch_transpose_pages(int dir, TransposeArgs& a, hipStream_t stream)
   // compute rows (Dd = head_dim) and the widest column chunk that fits LDS. Cutting head_dim to make
   // room for wider chunks lost 10-25 %, a 16 KiB tile lost 30-60 %, so the default is the full
   // head_dim with a ~60 KiB tile (two workgroups per CU).
-  if (ES == 2 && D % 32 == 0 && tuning().transpose_pairs != 0 && tuning().transpose_dsplit <= 1) {
-    // the word-pair kernel: unpadded tile [Cc/2 pairs][D] words, the widest column chunk that fits
+  if ((D * ES) % 64 == 0 && tuning().transpose_pairs != 0 && tuning().transpose_dsplit <= 1) {
+    // the pair kernel: unpadded tile [Cc/2 pairs][D] units, the widest column chunk that fits
     const int64_t budget = (int64_t)tuning().transpose_lds_kib * 1024;
     int best = 0;
     for (int cc = VE; cc <= C; cc += VE)
-      if (C % cc == 0 && (int64_t)D * cc * 2 + (cc / 2) * 8 <= budget) best = cc;
+      if (C % cc == 0 && (int64_t)D * cc * ES + (cc / 2) * 8 <= budget) best = cc;
     if (best > 0) {
       a.chunk_rows = D;
       a.n_dchunks = 1;
       a.chunk_cols = best;
       a.pitch = 0;
       a.n_chunks = (uint32_t)(C / best);
-      a.tile_words = (uint32_t)((int64_t)D * best / 2);
+      a.tile_words = (uint32_t)((int64_t)D * best * ES / 4);
       const size_t lds = (size_t)a.tile_words * 4 + (size_t)(best / 2) * 8;
       const int64_t gx = (int64_t)a.n_chunks * a.block_tokens;
       const int64_t gy = a.n_pages < 32768 ? a.n_pages : 32768;
@@ -391,19 +437,25 @@ hipError_t launch_transpose_pages(int dir, TransposeArgs& a, hipStream_t stream)
       if (gx >= (int64_t(1) << 24) || gz > 65535) return hipErrorInvalidValue;
       const dim3 grid((uint32_t)gx, (uint32_t)gy, (uint32_t)gz);
       const int block = tuning().transpose_block;
-#define BIKV_LAUNCH_PAIRS(DIR_, B_) \
-  hipLaunchKernelGGL((transpose_pairs_kernel<DIR_, B_>), grid, dim3(B_), lds, stream, a)
+#define BIKV_LAUNCH_PAIRS(DIR_, ES_, B_) \
+  hipLaunchKernelGGL((transpose_pairs_kernel<DIR_, ES_, B_>), grid, dim3(B_), lds, stream, a)
+#define BIKV_LAUNCH_PAIRS_B(DIR_, ES_)                         \
+  do {                                                         \
+    if (block == 256) BIKV_LAUNCH_PAIRS(DIR_, ES_, 256);       \
+    else if (block == 1024) BIKV_LAUNCH_PAIRS(DIR_, ES_, 1024); \
+    else if (block == 128) BIKV_LAUNCH_PAIRS(DIR_, ES_, 128);  \
+    else BIKV_LAUNCH_PAIRS(DIR_, ES_, 512);                    \
+  } while (0)
       if (dir == 0) {
-        if (block == 512) BIKV_LAUNCH_PAIRS(0, 512);
-        else if (block == 1024) BIKV_LAUNCH_PAIRS(0, 1024);
-        else if (block == 128) BIKV_LAUNCH_PAIRS(0, 128);
-        else BIKV_LAUNCH_PAIRS(0, 256);
+        if (ES == 1) BIKV_LAUNCH_PAIRS_B(0, 1);
+        else if (ES == 2) BIKV_LAUNCH_PAIRS_B(0, 2);
+        else BIKV_LAUNCH_PAIRS_B(0, 4);
       } else {
-        if (block == 512) BIKV_LAUNCH_PAIRS(1, 512);
-        else if (block == 1024) BIKV_LAUNCH_PAIRS(1, 1024);
-        else if (block == 128) BIKV_LAUNCH_PAIRS(1, 128);
-        else BIKV_LAUNCH_PAIRS(1, 256);
+        if (ES == 1) BIKV_LAUNCH_PAIRS_B(1, 1);
+        else if (ES == 2) BIKV_LAUNCH_PAIRS_B(1, 2);
+        else BIKV_LAUNCH_PAIRS_B(1, 4);
       }
+#undef BIKV_LAUNCH_PAIRS_B
 #undef BIKV_LAUNCH_PAIRS
       return hipGetLastError();
     }

@@ -36,12 +36,15 @@ def _make(rng, form, es, P, D, H, L, blocks, n_tm, cuda):
     (2, 4, 96, 4, 5),        # head_dim 96: word-pair kernel with 12 vectors per compute row
     (2, 2, 32, 1, 4),        # the smallest shape of the word-pair kernel: one vector per token-major row
     (2, 3, 256, 2, 36),      # head_dim 256, 144 columns: the tile is cut into column chunks
+    (1, 3, 64, 2, 4),        # 1-byte elements, the smallest pair-kernel shape (one vector per row)
+    (4, 2, 16, 3, 2),        # 4-byte elements, head_dim 16
+    (4, 3, 128, 4, 16),      # fp32, 128 columns: chunked
 ])
 @pytest.mark.parametrize("pairs", [1, 0])
 def test_load_and_store_match_oracle(lib, oracle, cuda, form, es, P, D, H, L, pairs):
     import bikv_pagecopy as bk
-    if pairs == 0 and (es != 2 or D % 32):
-        pytest.skip("only 2-byte elements with head_dim % 32 == 0 have two kernels to choose from")
+    if pairs == 0 and (D * es) % 64:
+        pytest.skip("only shapes with head_dim * element size % 64 == 0 have two kernels to choose from")
     print(f"[case] layout change {form} es={es} P={P} D={D} H={H} L={L} pairs={pairs}", flush=True)
     bk.set_tuning(transpose_pairs=pairs)
     rng = np.random.default_rng(es * 1000 + D + H + L)
