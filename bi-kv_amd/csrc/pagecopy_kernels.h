@@ -51,14 +51,15 @@ struct Tuning {
                         // -1 = chosen from the batch's layout hint
   int log2_chunk = -1;  // order 1: 2^log2_chunk pages per chunk; -1 = chosen
   int unroll = 4;       // 16-byte vectors in flight per lane (1, 2, 4 or 8)
-  int nontemporal = -1; // nt hint on payload loads and stores: 1 on, 0 off, -1 = chosen
-  int run_chunk_kib = 0;  // bytes of a run handled by one workgroup, KiB; 0 = choose
-  int transpose_lds_kib = 60;  // LDS tile budget of the layout-change kernel, KiB
+  int nontemporal = -1; // cache policy of payload accesses: 0 none, 1 nt, 4 nt + system scope,
+                        // -1 = chosen per direction and layout (run copy also: 2 loads, 3 stores only)
+  int run_chunk_kib = 0;       // bytes of a run handled by one workgroup, KiB; 0 = choose
+  int run_group = 1;           // wave run kernel: several short runs share one grid row (0 = off)
+  int small_run_max = 1023;    // runs up to this many bytes go to the one-lane-per-piece kernel
+  int transpose_lds_kib = 60;  // LDS tile budget of the layout-change kernels, KiB
   int transpose_dsplit = 0;    // slices of head_dim per tile; 0 = default (1: whole compute rows)
-int run_group = 1;         // wave run kernel: pack several short runs into one grid row (0 = off)
-  int small_run_max = 1023;  // runs up to this many bytes go to the one-lane-per-piece kernel
-    int transpose_pairs = 1;  // the K/V-pair kernel where the shape allows (0 = element-wise kernel)
-  int transpose_block = 512; // lanes per workgroup of the word-pair kernel: 128, 256, 512, 1024
+  int transpose_pairs = 1;     // the K/V-pair kernel where the shape allows (0 = element-wise kernel)
+  int transpose_block = 512;   // lanes per workgroup of the K/V-pair kernel: 128, 256, 512, 1024
 };
 Tuning& tuning();
 
