@@ -24,8 +24,10 @@
  * How each is pinned (tests/test_oracle.py): the two known-answer scenarios the reference's own
  * scripts hold (test_page_ipc.py:41-65,127-150; test_zero_copy.py:30-48,86-103), the library
  * routines the formula reduces to (numpy fancy indexing, torch.index_select / index_copy_),
- * per-byte brute force on tiny inputs, and permutation / duplicate / canary invariants.
- * No function here is "parity unpinned".
+ * per-byte brute force on tiny inputs, and permutation / duplicate / canary invariants. The ragged
+ * copy is pinned by its reduction to the uniform copy, by brute force, and by an offset-free
+ * statement of the packed transfer ("each item's rows, cut to its token count, back to back") reached
+ * through the reference's own packed offsets. No function here is "parity unpinned".
  */
 #include <stdint.h>
 #include <string.h>
