@@ -519,6 +519,87 @@ def run_reference_scenario(args, bk, dev):
     }
 
 
+def run_token_major(args, bk, workloads, dev):
+    """The Qwen2-7B request stream in the REFERENCE'S layout: a token-major pool of 131072 pages of
+    16 tokens x (128, 4, 28, 2) bf16 = 917 504 bytes each (kvcache.py:38-43 at this shape), one run per
+    page through the run copy (block_per_page_copy_kernel's role, copy_kernel.cu:9-36): gather the 32
+    gather requests into a dense buffer, scatter the 32 scatter requests back from it."""
+    import numpy as np
+    import torch
+    shape = workloads.SHAPES["qwen2_7b"]
+    if args.pool_pages:
+        shape = shape.scaled(args.pool_pages)
+    wl = workloads.named("qwen2_7b", shape)
+    page_elems = shape.page_bytes // 2
+    pool = torch.empty(shape.n_pages * page_elems, dtype=torch.bfloat16, device=dev)
+    fill_random_bytes(pool)
+    g_ids = np.concatenate(wl["gather"]).astype(np.int64)
+    s_ids = np.concatenate(wl["scatter"]).astype(np.int64)
+    n_g, n_s = len(g_ids), len(s_ids)
+    dense = torch.empty(max(n_g, n_s) * page_elems, dtype=torch.bfloat16, device=dev)
+    g_src = torch.from_numpy(g_ids * page_elems).to(dev)
+    s_dst = torch.from_numpy(s_ids * page_elems).to(dev)
+    g_dst = torch.arange(n_g, dtype=torch.int64, device=dev) * page_elems
+    s_src = torch.arange(n_s, dtype=torch.int64, device=dev) * page_elems
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        bk.copy_runs(pool, dense, g_src, g_dst, page_elems)
+        if ev:
+            ev[1].record()
+        bk.copy_runs(dense, pool, s_src, s_dst, page_elems)
+        if ev:
+            ev[2].record()
+
+    # parity of the gather at full size: torch.index_select over the page view
+    bk.copy_runs(pool, dense, g_src, g_dst, page_elems)
+    from bikv_pagecopy import runs
+    runs.check(dev)
+    view = pool.view(torch.int16).view(shape.n_pages, page_elems)
+    sample = np.arange(0, n_g, max(1, n_g // 64))
+    want = torch.index_select(view, 0, torch.from_numpy(g_ids[sample]).to(dev))
+    got = dense.view(torch.int16).view(-1, page_elems)[torch.from_numpy(sample).to(dev)]
+    if not torch.equal(got, want):
+        raise SystemExit("bench: token-major gather differs from torch.index_select")
+    for _ in range(args.warmup):
+        step()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(evs[k])
+    torch.cuda.synchronize(dev)
+    wall = time.perf_counter() - t0
+    runs.check(dev)
+    # the scatter wrote the dense buffer's first n_s pages into the scatter ids
+    got = torch.index_select(view, 0, torch.from_numpy(s_ids[:64]).to(dev))
+    if not torch.equal(got, dense.view(torch.int16).view(-1, page_elems)[:64]):
+        raise SystemExit("bench: token-major scatter differs")
+    g_ms = float(np.mean([e[0].elapsed_time(e[1]) for e in evs]))
+    s_ms = float(np.mean([e[1].elapsed_time(e[2]) for e in evs]))
+    alg_g, alg_s = 2 * n_g * shape.page_bytes, 2 * n_s * shape.page_bytes
+    slow_g = alg_g / g_ms <= alg_s / s_ms
+    alg, ms = (alg_g, g_ms) if slow_g else (alg_s, s_ms)
+    value = (alg_g + alg_s) / (wall / args.steps) / 1e9
+    return {
+        "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"qwen2_7b_token_major: {shape.n_pages} pages x {shape.page_bytes} B (16 tok x (128,4,28,2) bf16), "
+                               f"{n_g} pages gathered + {n_s} scattered per step, one run per page",
+                   "pool_GB": round(shape.pool_bytes / 1e9, 2)},
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "pages_per_s": round((n_g + n_s) / (wall / args.steps), 1), "bit_exact": True,
+        "kernels": {"gather": {"GBps": round(alg_g / g_ms / 1e6, 1), "avg_ms": round(g_ms, 4)},
+                    "scatter": {"GBps": round(alg_s / s_ms / 1e6, 1), "avg_ms": round(s_ms, 4)}},
+        "roofline": {"bound": "hbm", "kernel": "bikv::copy_runs_wave_kernel", "achieved": round(alg / ms / 1e6, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(alg / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                     "traffic": None, "alg_bytes_per_launch": alg, "avg_launch_ms": round(ms, 4)},
+    }
+
+
 def run_layout_change(args, bk, dev):
     """Received token-major pages -> the Worker's per-layer paged pool and back, at the reference's own
     shapes: token_shape (128, 2, 28, 2) fp16 (Model/qwen2.py:512-522), 28 layer tensors of
@@ -620,6 +701,10 @@ def main():
 
     if args.workload == "reference_200x50":
         out = run_reference_scenario(args, bk, dev)
+        print(json.dumps(out), flush=True)
+        return
+    if args.workload == "qwen2_7b_token_major":
+        out = run_token_major(args, bk, workloads, dev)
         print(json.dumps(out), flush=True)
         return
     if args.workload == "layout_change":
