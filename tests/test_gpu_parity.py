@@ -498,6 +498,64 @@ def test_copy_runs_zero_copy_from_pinned_host(bk, oracle, cuda):
     assert _to_np(dst).tobytes() == want.tobytes()
 
 
+# ---- seeded random sweep ------------------------------------------------------------------------
+def test_random_pools_batches_and_knobs_match_oracle(bk, oracle, cuda):
+    """Forty seeded cases over everything a caller can vary at once: plane count, pool size, tile size
+    (wave-mover shapes, ragged pieces, tiny and odd tiles), a page stride wider than the tile, an
+    optional scale class, staging layout, duplicate and out-of-order ids, empty requests, walk order and
+    chunk, workgroup size. Gather against the oracle, then scatter into other pages; the gaps between
+    tiles must keep their canary."""
+    rng = np.random.default_rng(2024)
+    tiles = [16, 80, 1000, 1024, 3072, 4096, 5000, 8192, 16384, 20480, 65536]
+    try:
+        for case in range(40):
+            n_planes = int(rng.integers(1, 9))
+            n_pages = int(rng.integers(6, 50))
+            tile = int(rng.choice(tiles))
+            gap = int(rng.choice([0, 0, 16, 64, 4096])) if tile % 16 == 0 else 0
+            stile = int(rng.choice([0, 0, 4, 32, 48]))
+            layout = str(rng.choice(["layer_major", "page_major"]))
+            knobs = dict(order=int(rng.integers(-1, 2)), log2_chunk=int(rng.integers(-1, 5)),
+                         wave_block=int(rng.choice([64, 128, 256])), nontemporal=int(rng.choice([-1, 0, 1, 4])))
+            _announce(f"random case {case}: planes={n_planes} pages={n_pages} tile={tile}+{gap} scale={stile} {layout} {knobs}")
+            bk.set_tuning(**knobs)
+            back_h = rng.integers(0, 256, size=(n_planes, n_pages, tile + gap), dtype=np.uint8)
+            back_d = torch.from_numpy(back_h).to(cuda)
+            pool_h = np.ascontiguousarray(back_h[:, :, :tile])
+            sc_h = rng.integers(0, 256, size=(n_planes, n_pages, max(stile, 1)), dtype=np.uint8)
+            sc_d = torch.from_numpy(sc_h).to(cuda)
+            pool = bk.PagedKVPool([back_d[q].data_ptr() for q in range(n_planes)], n_pages, tile, tile + gap, cuda,
+                                  scale_plane_ptrs=[sc_d[q].data_ptr() for q in range(n_planes)] if stile else None,
+                                  scale_tile_bytes=stile, scale_page_stride_bytes=stile, keepalive=(back_d, sc_d))
+            n_req = int(rng.integers(1, 5))
+            g_reqs = [rng.integers(0, n_pages, size=int(rng.integers(0, n_pages))) for _ in range(n_req)]   # duplicates
+            gb = pool.make_batch(g_reqs, layout)
+            st, sc = pool.gather(gb)
+            pool.check()
+            assert _to_np(st).tobytes() == oracle.gather_layered_c(pool_h, g_reqs, layout).tobytes(), case
+            if stile:
+                assert _to_np(sc).tobytes() == oracle.gather_layered_c(sc_h, g_reqs, layout).tobytes(), case
+            perm = rng.permutation(n_pages)
+            cuts = np.sort(rng.integers(0, n_pages, size=n_req - 1))
+            s_reqs = [np.ascontiguousarray(a) for a in np.split(perm[: int(rng.integers(1, n_pages + 1))], [c for c in cuts if c < n_pages])]
+            s_reqs = [r for r in s_reqs]
+            sb = pool.make_batch(s_reqs, layout)
+            src = rng.integers(0, 256, size=sb.n_slots * tile, dtype=np.uint8)
+            ssrc = rng.integers(0, 256, size=sb.n_slots * max(stile, 1), dtype=np.uint8)
+            pool.scatter(sb, torch.from_numpy(src).to(cuda), torch.from_numpy(ssrc).to(cuda) if stile else None)
+            pool.check()
+            oracle.scatter_layered_c(pool_h, s_reqs, src, layout)
+            got = _to_np(back_d).reshape(n_planes, n_pages, tile + gap)
+            assert got[:, :, :tile].tobytes() == pool_h.tobytes(), case
+            assert got[:, :, tile:].tobytes() == back_h[:, :, tile:].tobytes(), case      # gaps untouched
+            if stile:
+                oracle.scatter_layered_c(sc_h, s_reqs, ssrc[: sb.n_slots * stile], layout)
+                assert _to_np(sc_d).tobytes() == sc_h.tobytes(), case
+            pool.close()
+    finally:
+        bk.set_tuning(seg=0, wave_block=64, unroll=4, nontemporal=-1, order=-1, log2_chunk=-1)
+
+
 # ---- HIP graph capture --------------------------------------------------------------------------
 def test_gather_scatter_and_run_copy_replay_from_a_hip_graph(bk, oracle, cuda):
     """The asynchronous entry points only launch kernels (no allocation, no memset, no synchronisation),
