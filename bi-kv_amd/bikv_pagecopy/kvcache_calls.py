@@ -38,7 +38,7 @@ def _dims(n_pages: int, page_size: int, dims: Sequence[int]):
     return d
 
 
-def _tables(info: Dict, page_size: int, dims: Sequence[int], pack_partial_pages, device):
+def _tables(info: Dict, page_size: int, dims: Sequence[int], pack_partial_pages, device, index_pool=None):
     pages_list = info["cache_pages_list"]
     tokens = [int(p[1]) for p in info["id_token_pair"]]
     ept = int(dims[0]) * int(dims[1]) * int(dims[2]) * int(dims[3])
@@ -50,14 +50,17 @@ def _tables(info: Dict, page_size: int, dims: Sequence[int], pack_partial_pages,
     n = off.shape[1]
     if not pack_partial_pages and n:
         off[1] = range(0, n * page_size * ept, page_size * ept)
-    dev = torch.from_numpy(off).to(device) if n else torch.empty((off.shape[0], 0), dtype=torch.int64, device=device)
+    if index_pool is not None and n:
+        dev = index_pool.load(off)            # persistent buffers (kvcache.py:60-64), no allocation
+    else:
+        dev = torch.from_numpy(off).to(device) if n else torch.empty((off.shape[0], 0), dtype=torch.int64, device=device)
     return dev, n, total
 
 
-def _send(data, info, page_size, dims, pack_partial_pages, device, whole_pages) -> Tuple[int, int]:
+def _send(data, info, page_size, dims, pack_partial_pages, device, whole_pages, index_pool=None) -> Tuple[int, int]:
     if pack_partial_pages not in (False, True, "exact"):
         raise ValueError("pack_partial_pages must be False, True or 'exact'")
-    off, n, total = _tables(info, page_size, dims, pack_partial_pages, device)
+    off, n, total = _tables(info, page_size, dims, pack_partial_pages, device, index_pool)
     d = _dims(n, page_size, dims)
     if pack_partial_pages == "exact":
         d.total_tokens = total
@@ -69,19 +72,20 @@ def _send(data, info, page_size, dims, pack_partial_pages, device, whole_pages) 
 
 def shared_data_batch_pages(cuda_cache_data: torch.Tensor, combined_task_info: Dict, page_size: int,
                             dims: Sequence[int] = REFERENCE_DIMS,
-                            pack_partial_pages=False) -> Tuple[int, int]:
-    """Device pool -> consumer ring. Returns (pages copied, tokens published)."""
+                            pack_partial_pages=False, index_pool=None) -> Tuple[int, int]:
+    """Device pool -> consumer ring. Returns (pages copied, tokens published). `index_pool` (a
+    RunIndexPool) keeps the offset tables in persistent device buffers."""
     if not cuda_cache_data.is_cuda:
         raise RuntimeError("Cache data must be on CUDA")
     return _send(cuda_cache_data, combined_task_info, page_size, dims, pack_partial_pages,
-                 cuda_cache_data.device, ipc_service.producer_copy_pages)
+                 cuda_cache_data.device, ipc_service.producer_copy_pages, index_pool)
 
 
 def shared_data_batch_pages_cpu2gpu(cpu_cache_data: torch.Tensor, combined_task_info: Dict, page_size: int,
                                     device, dims: Sequence[int] = REFERENCE_DIMS,
-                                    pack_partial_pages=False) -> Tuple[int, int]:
+                                    pack_partial_pages=False, index_pool=None) -> Tuple[int, int]:
     """Pinned host pool -> consumer ring, the GPU reading host memory directly (kvcache.py:241-366)."""
     if cpu_cache_data.is_cuda or not cpu_cache_data.is_pinned():
         raise RuntimeError("CPU data must be pinned memory")
     return _send(cpu_cache_data, combined_task_info, page_size, dims, pack_partial_pages,
-                 torch.device(device), ipc_service.producer_zero_copy_pages)
+                 torch.device(device), ipc_service.producer_zero_copy_pages, index_pool)

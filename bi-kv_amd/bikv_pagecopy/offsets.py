@@ -18,6 +18,7 @@ this builder is vectorised numpy and produces one [2, n] array for a single uplo
 from typing import Sequence, Tuple
 
 import numpy as np
+import torch
 
 
 def build_run_offsets(cache_pages_list: Sequence[Sequence[int]], item_tokens: Sequence[int],
@@ -54,3 +55,34 @@ def build_run_offsets(cache_pages_list: Sequence[Sequence[int]], item_tokens: Se
     if with_sizes:
         out[2] = sizes
     return out, int(sizes.sum())
+
+
+class RunIndexPool:
+    """Persistent device index buffers, as KVCache keeps them (kvcache.py:60-64, `src_index_pool` /
+    `dst_index_pool` of `max_pages` int64 entries each, handed out by `get_index_tensors`, :83-86 —
+    which returns the source pool twice; here the rows are distinct). One device tensor of `rows` x
+    `max_pages` int64 and a pinned host mirror: `load()` copies a freshly built offset table into the
+    mirror and uploads it with one asynchronous copy on the current stream, so a transfer allocates
+    nothing and never uploads from pageable memory."""
+
+    def __init__(self, max_pages: int, device, rows: int = 3):
+        self.max_pages = int(max_pages)
+        self.rows = int(rows)
+        self.device = torch.device(device)
+        self.dev = torch.full((self.rows, self.max_pages), -1, dtype=torch.int64, device=self.device)
+        self.host = torch.empty((self.rows, self.max_pages), dtype=torch.int64, pin_memory=True)
+        self._busy = None
+
+    def load(self, table: np.ndarray) -> torch.Tensor:
+        """table: [r, n] int64 with r <= rows, n <= max_pages. Returns the [r, n] device rows
+        (each row contiguous), valid until the next load()."""
+        r, n = table.shape
+        if r > self.rows or n > self.max_pages:
+            raise RuntimeError(f"Requested {n} exceeds pool size {self.max_pages}")   # kvcache.py:84
+        if self._busy is not None:
+            self._busy.synchronize()          # the previous upload still reads the mirror
+        self.host[:r, :n] = torch.from_numpy(np.ascontiguousarray(table, dtype=np.int64))
+        self.dev[:r, :n].copy_(self.host[:r, :n], non_blocking=True)
+        self._busy = torch.cuda.Event()
+        self._busy.record(torch.cuda.current_stream(self.device))
+        return self.dev[:r, :n]

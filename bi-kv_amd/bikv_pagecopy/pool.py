@@ -50,10 +50,9 @@ class PageBatch:
     def desc(self, plane_begin=0, plane_count=0, slot_bias=0) -> _lib.PageBatchDesc:
         d = _lib.PageBatchDesc()
         if self.n_pages:
-            base = self.index.data_ptr()
-            d.page_ids = base
-            d.slots = base + 8 * self.n_pages
-            d.slot_strides = base + 16 * self.n_pages
+            d.page_ids = self.index[0].data_ptr()       # rows need not be adjacent (persistent buffers)
+            d.slots = self.index[1].data_ptr()
+            d.slot_strides = self.index[2].data_ptr()
         d.n_pages = self.n_pages
         d.plane_begin = plane_begin
         d.plane_count = plane_count
@@ -190,9 +189,15 @@ class PagedKVPool:
         return cls(ptrs, t0.shape[0], tile, 2 * tile, t0.device, t0.dtype, keepalive=list(layers))
 
     # ---- batches ----------------------------------------------------------------------------
-    def make_batch(self, requests: Sequence[Sequence[int]], layout: str = LAYER_MAJOR) -> PageBatch:
+    def make_batch(self, requests: Sequence[Sequence[int]], layout: str = LAYER_MAJOR, index_pool=None) -> PageBatch:
+        """Builds and uploads the index arrays of a batch. With `index_pool` (offsets.RunIndexPool, 3 rows)
+        they go into its persistent device buffers through its pinned mirror: no allocation, no upload
+        from pageable memory; the batch is then valid until the pool's next load()."""
         idx, req_pages = build_index(requests, self.n_planes, layout)
-        dev = torch.from_numpy(idx).to(self.device) if idx.size else torch.empty((3, 0), dtype=torch.int64, device=self.device)
+        if index_pool is not None and idx.size:
+            dev = index_pool.load(idx)
+        else:
+            dev = torch.from_numpy(idx).to(self.device) if idx.size else torch.empty((3, 0), dtype=torch.int64, device=self.device)
         return PageBatch(dev, req_pages, self.n_planes, layout)
 
     def empty_staging(self, batch: PageBatch):

@@ -314,3 +314,41 @@ def test_backpressure_holds_the_producer_until_release(ipc, cuda):
         ipc.consumer_release()
     with pytest.raises(RuntimeError, match="not initialised"):
         ipc.producer_set_backpressure(True)
+
+
+def test_persistent_index_buffers_for_offsets_and_batches(ipc, oracle, cuda):
+    """RunIndexPool = the reference's src_index_pool / dst_index_pool (kvcache.py:60-64): tables of
+    successive transfers reuse the same device buffers."""
+    import bikv_pagecopy as bk
+    from bikv_pagecopy import kvcache_calls
+    print("[case] persistent index buffers", flush=True)
+    name = f"/bikv_test_idxpool_{os.getpid()}"
+    dims, page_size, pool_pages = (64, 2, 3, 2), 16, 50
+    ept = dims[0] * dims[1] * dims[2] * dims[3]
+    ipc.consumer_init(0, name, 64 << 20)
+    ipc.producer_init(0, name)
+    rng = np.random.default_rng(31)
+    pool_h = rng.integers(0, 65536, size=(pool_pages * page_size, ept), dtype=np.uint16)
+    pool_t = torch.from_numpy(pool_h.view(np.int16)).view(torch.float16).to(cuda)
+    idx = bk.RunIndexPool(max_pages=pool_pages, device=cuda)
+    base = idx.dev.data_ptr()
+    for pages_list, tokens in (([[7, 2, 49], [4]], [40, 16]), ([[1], [30, 31, 0, 9], [5, 6]], [3, 64, 17])):
+        info = {"infer_worker": 0, "token_num": sum(tokens),
+                "id_token_pair": list(enumerate(tokens)), "cache_pages_list": pages_list}
+        n, total = kvcache_calls.shared_data_batch_pages(pool_t, info, page_size, dims, "exact", index_pool=idx)
+        got = ipc.consumer_receive(timeout_ms=5000)
+        want = oracle.packed_items_np(pool_h, pages_list, tokens, page_size)
+        assert total == sum(tokens) and got.cpu().contiguous().view(torch.int16).numpy().tobytes() == want.tobytes()
+        assert idx.dev.data_ptr() == base
+    with pytest.raises(RuntimeError, match="exceeds pool size"):
+        idx.load(np.zeros((2, pool_pages + 1), dtype=np.int64))
+    # the layered batch builder takes the same kind of pool
+    planes_h = rng.integers(0, 256, size=(4, 30, 4096), dtype=np.uint8)
+    kv = bk.PagedKVPool.from_stacked(torch.from_numpy(planes_h).to(cuda), plane_dims=1)
+    bidx = bk.RunIndexPool(max_pages=64, device=cuda)
+    for reqs in ([rng.permutation(30)[:11], rng.permutation(30)[:5]], [rng.permutation(30)[:20]]):
+        for layout in ("layer_major", "page_major"):
+            b = kv.make_batch(reqs, layout, index_pool=bidx)
+            st, _ = kv.gather(b)
+            kv.check()
+            assert st.cpu().numpy().tobytes() == oracle.gather_layered_c(planes_h, reqs, layout).tobytes()
