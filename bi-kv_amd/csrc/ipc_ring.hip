@@ -15,6 +15,7 @@
 #include "pagecopy_kernels.h"
 
 #include <cerrno>
+#include <cstdlib>
 #include <cstring>
 #include <ctime>
 #include <deque>
@@ -235,6 +236,16 @@ extern "C" int bikv_producer_init(int device, const char* shm_name) {
     unmap_role(r);
     return fail(BIKV_ESTATE, "Processes must run on the same host");
   }
+  const bool same_process = g_consumer.ctrl && strcmp(g_consumer.shm_name, shm_name) == 0;
+  // Mapping another process's allocation of 2 GiB or more has been seen not to return on some
+  // ROCm hosts; such a ring is refused unless the deployment opts in.
+  const char* allow = getenv("BIKV_IPC_ALLOW_LARGE");
+  if (!same_process && r.ctrl->buffer_size >= (size_t(2) << 30) && !(allow && allow[0] == '1')) {
+    const size_t bytes = r.ctrl->buffer_size;
+    unmap_role(r);
+    return fail(BIKV_ERANGE, "the consumer's ring is %zu bytes: IPC mappings of 2 GiB or more are refused "
+                             "(set BIKV_IPC_ALLOW_LARGE=1 to map it anyway)", bytes);
+  }
   {
     hipError_t e = hipSetDevice(device);
     if (e != hipSuccess) {
@@ -242,7 +253,7 @@ extern "C" int bikv_producer_init(int device, const char* shm_name) {
       return fail_hip(e, "hipSetDevice");
     }
   }
-  if (g_consumer.ctrl && strcmp(g_consumer.shm_name, shm_name) == 0) {
+  if (same_process) {
     r.mem = g_consumer.mem;  // same process: no IPC mapping needed (or possible)
     r.ipc_mapped = false;
   } else {

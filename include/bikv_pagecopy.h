@@ -337,7 +337,10 @@ typedef struct bikv_tensor_dims {
 /* consumer_init (ipc_service.cpp:20-74): unlink+create shm, init semaphores, record hostname and
  * device, allocate the device ring, publish its IPC handle. */
 int bikv_consumer_init(int device, const char* shm_name, size_t buffer_bytes);
-/* producer_init (ipc_service.cpp:77-110): open shm, same-host check, map the ring. */
+/* producer_init (ipc_service.cpp:77-110): open shm, same-host check, map the ring. A producer in
+ * ANOTHER process than the consumer refuses a ring of 2 GiB or more with BIKV_ERANGE (opening an IPC
+ * mapping that large has been seen not to return on some ROCm hosts); the environment variable
+ * BIKV_IPC_ALLOW_LARGE=1 lifts the limit. */
 int bikv_producer_init(int device, const char* shm_name);
 /* producer_cleanup / consumer_cleanup (ipc_service.cpp:171-202). Idempotent. */
 void bikv_producer_cleanup(void);

@@ -310,3 +310,25 @@ def test_plain_c_client_compiles_against_the_header_alone():
                             "-c", os.path.join(root, "tests", "c_client", "abi_client.c"), "-o", os.path.join(tmp, "c.o")],
                            capture_output=True, text=True)
         assert r.returncode == 0, r.stderr
+
+
+def test_producer_refuses_to_map_a_ring_of_2_gib_from_another_process(lib):
+    """The check happens on the control block, before any GPU call: a control block that announces a
+    2 GiB ring (written here by hand, as a consumer in another process would) is refused."""
+    import mmap
+    from bikv_pagecopy import _lib
+    name = f"/bikv_test_bigring_{os.getpid()}"
+    path = "/dev/shm" + name
+    ctrl = _lib.SharedControl()
+    host = os.uname().nodename.encode()
+    ctrl.hostname = host
+    ctrl.buffer_size = 2 << 30
+    with open(path, "wb") as f:
+        f.write(bytes(ctrl))
+    try:
+        os.environ.pop("BIKV_IPC_ALLOW_LARGE", None)
+        rc = lib.bikv_producer_init(0, name.encode())
+        assert rc == -6 and b"2 GiB" in lib.bikv_last_error()
+        assert not lib.bikv_producer_control()
+    finally:
+        os.unlink(path)
