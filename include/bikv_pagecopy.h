@@ -51,7 +51,11 @@ int bikv_abi_version(void);
 const char* bikv_last_error(void);
 
 /* Reads and clears the status word of `device` after synchronising `stream`.
- * Returns BIKV_OK, or BIKV_EBOUNDS with *bits_out (nullable) holding the BIKV_ST_* bits. */
+ * Returns BIKV_OK, or BIKV_EBOUNDS with *bits_out (nullable) holding the BIKV_ST_* bits.
+ * There is ONE status word per device, shared by every stream and host thread: a check reports (and
+ * clears) whatever any launch on that device has raised since the previous check, so callers that run
+ * several streams should treat a report as "some launch since the last check skipped work". Memory
+ * safety never depends on the check: out-of-range units are skipped by the kernels themselves. */
 int bikv_check_status(int device, void* stream, uint32_t* bits_out);
 
 /* Kernel launch knobs, for measurement. Keys: "seg" (0 = default: the wave mover, one 16-byte
