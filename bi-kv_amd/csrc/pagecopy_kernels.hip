@@ -1,16 +1,18 @@
 // gfx950 kernels of the KV page-copy path. Pure data movement: every lane moves 16-byte vectors
-// (global_load_dwordx4 / global_store_dwordx4), a wavefront moves 1 KiB per instruction, and a
-// 256-lane workgroup moves one 4 KiB "row" per vector slot. No arithmetic on the payload, so the
-// kernels are dtype-agnostic and bit-exact by construction (NaN payloads and fp8 bit patterns are
-// never routed through a floating-point type).
+// (global_load_dwordx4 / global_store_dwordx4) and a wavefront moves 1 KiB per instruction. No
+// arithmetic on the payload, so the kernels are dtype-agnostic and bit-exact by construction (NaN
+// payloads and fp8 bit patterns are never routed through a floating-point type).
 //
 // Semantics follow the reference's two kernels, block_per_page_copy_kernel and
 // zero_copy_page_kernel (Bi-KV/SharedMemory/CUDA_Shared/copy_kernel.cu:9-36, 39-66):
 //   dst[dst_off[i] + e] = src[src_off[i] + e]   for every run i and every byte e of the run.
 // The reference moves one 2-byte scalar per thread per iteration with one 1024-thread block per
-// page; here the unit of scheduling is a 16 KiB..256 KiB span so that a batch of a few hundred
-// large pages still fills 256 CUs, and page descriptors are resolved once per workgroup into LDS
-// and broadcast from there.
+// page. Here the default movers (tile_move_wave_kernel for the layered pool, copy_runs_wave_kernel
+// for the reference's runs) give every 1 KiB piece its own 64-lane workgroup, one vector per lane,
+// with the piece's descriptor fetched by scalar loads: millions of tiny independent workgroups are
+// what this GPU copies fastest with. The LDS-staged segment movers further down (a segment of pages
+// per 256-lane workgroup, descriptors resolved once into LDS and broadcast) take the shapes the
+// wave movers do not: tiles that are not 16-byte aligned, tiny tiles, misaligned pools.
 #include "pagecopy_kernels.h"
 
 namespace bikv {
@@ -350,9 +352,9 @@ __global__ __launch_bounds__(B) void tile_move_wave_kernel(const MoveArgs a) {
 //     adjacent (chunk of 1 page); with a layer-major image a scatter reads runs of 16 tiles per
 //     plane, and a gather — whose dense side is the WRITTEN one — does best writing each plane's
 //     range front to back (order 0);
-//   * the nt hint helps every case above, nt with system scope (policy 2 of move16) another 2-4 % and
-//     it takes away most of the run-to-run spread; without a layout hint hints are kept off for
-//     scatters, where nt is neutral to slightly negative in order 0.
+//   * the nt hint helps every case above, nt with system scope (policy 2 of move16) another 1-3 %;
+//     without a layout hint hints are kept off for scatters, where nt is neutral to slightly
+//     negative in order 0.
 struct WavePolicy {
   int order, log2_chunk;
   int nt;   // cache policy of move16: 0, 1 or 2
