@@ -143,6 +143,8 @@ _SIGNATURES = {
     "bikv_host_free": (C.c_int, [C.c_void_p]),
     "bikv_consumer_init": (C.c_int, [C.c_int, C.c_char_p, C.c_size_t]),
     "bikv_producer_init": (C.c_int, [C.c_int, C.c_char_p]),
+    "bikv_producer_reserve": (C.c_int, [C.c_size_t, C.POINTER(C.c_void_p)]),
+    "bikv_producer_publish": (C.c_int, [C.POINTER(C.c_int64), C.c_size_t, C.c_int32, C.c_void_p]),
     "bikv_producer_set_backpressure": (C.c_int, [C.c_int, C.c_int64]),
     "bikv_consumer_release": (C.c_int, []),
     "bikv_producer_cleanup": (None, []),

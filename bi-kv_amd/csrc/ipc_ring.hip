@@ -45,6 +45,9 @@ struct Role {
   bool backpressure = false;
   int64_t bp_timeout_ms = -1;
   std::deque<std::pair<size_t, size_t>> in_flight;
+  // producer only: window handed out by bikv_producer_reserve and not published yet
+  bool reserved = false;
+  size_t reserved_at = 0, reserved_bytes = 0;
 };
 
 Role g_producer, g_consumer;
@@ -388,6 +391,43 @@ extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64
   }
   ring_publish(c, bytes, shape, ndim, dtype_code);
   producer_published(g_producer, at, bytes);
+  return BIKV_OK;
+}
+
+// Two-step producer for callers that fill the ring themselves (a layered gather whose staging image
+// IS the consumer's ring window, the way block_per_page_copy_kernel writes straight into the mapped
+// buffer, copy_kernel.cu:92-113): reserve applies the reference's wrap rule and hands out the write
+// pointer; publish performs the reference's bookkeeping for exactly the reserved bytes.
+extern "C" int bikv_producer_reserve(size_t bytes, void** ptr) {
+  if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
+  if (!ptr) return fail(BIKV_EINVAL, "null pointer argument");
+  bikv_shared_control* c = g_producer.ctrl;
+  if (bytes > c->buffer_size)
+    return fail(BIKV_ERANGE, "reservation of %zu bytes does not fit the %zu-byte ring", bytes, c->buffer_size);
+  size_t at = 0;
+  const int rc = producer_reserve(g_producer, bytes, &at);
+  if (rc) return rc;
+  g_producer.reserved = true;
+  g_producer.reserved_at = at;
+  g_producer.reserved_bytes = bytes;
+  *ptr = static_cast<char*>(g_producer.mem) + at;
+  return BIKV_OK;
+}
+
+extern "C" int bikv_producer_publish(const int64_t* shape, size_t ndim, int32_t dtype_code, void* stream) {
+  if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
+  if (!g_producer.reserved) return fail(BIKV_ESTATE, "nothing is reserved (call bikv_producer_reserve first)");
+  if (ndim > BIKV_MAX_DIM) return fail(BIKV_EINVAL, "at most %d dimensions can be published", BIKV_MAX_DIM);
+  if (ndim > 0 && !shape) return fail(BIKV_EINVAL, "null pointer argument");
+  BIKV_DEVICE(g_producer.device);
+  // the bytes must be in the ring before the consumer is woken; a kernel that skipped work is an error
+  int rc = sync_and_check(g_producer.device, static_cast<hipStream_t>(stream));
+  if (rc) return rc;
+  rc = producer_wait_slot(g_producer);
+  if (rc) return rc;
+  g_producer.reserved = false;
+  ring_publish(g_producer.ctrl, g_producer.reserved_bytes, shape, ndim, dtype_code);
+  producer_published(g_producer, g_producer.reserved_at, g_producer.reserved_bytes);
   return BIKV_OK;
 }
 

@@ -36,6 +36,7 @@ __all__ = [
     "TensorDims", "producer_init", "producer_send", "producer_cleanup", "consumer_init",
     "consumer_receive", "consumer_cleanup", "producer_copy_pages", "cuda_producer_copy_pages",
     "producer_zero_copy_pages", "producer_copy_tokens", "producer_set_backpressure", "consumer_release",
+    "producer_reserve", "producer_publish",
 ]
 
 # dtype codes carried in the control block's first spare int (0 = float16, what a reference
@@ -87,6 +88,33 @@ def producer_cleanup():
 
 def consumer_cleanup():
     _lib.load().bikv_consumer_cleanup()
+
+
+def producer_reserve(nbytes):
+    """Not in the reference's module. Reserves `nbytes` of the consumer's ring (the reference's wrap
+    rule, copy_kernel.cu:87-89) and returns them as a uint8 device tensor that the caller fills itself,
+    e.g. as the staging image of PagedKVPool.gather; producer_publish then hands it to the consumer."""
+    ptr = C.c_void_p()
+    with torch.cuda.device(_producer_device()):
+        _lib.check(_lib.load().bikv_producer_reserve(int(nbytes), C.byref(ptr)))
+    device = torch.device("cuda", _producer_device())
+    if nbytes == 0:
+        return torch.empty(0, dtype=torch.uint8, device=device)
+    return torch.as_tensor(_RingWindow(ptr.value, int(nbytes)), device=device)
+
+
+def producer_publish(shape, dtype=torch.float16):
+    """Publishes the reserved bytes as a tensor of `shape` (at most 5 dimensions) and `dtype`; waits for
+    the current stream first and raises, publishing nothing, if a kernel writing the window skipped
+    out-of-range work."""
+    shape = tuple(int(x) for x in shape)
+    if len(shape) > _lib.MAX_DIM:
+        raise RuntimeError(f"Tensor must have at most {_lib.MAX_DIM} dimensions")
+    if dtype not in _CODE_OF:
+        raise RuntimeError(f"unsupported dtype {dtype}")
+    arr = (C.c_int64 * _lib.MAX_DIM)(*shape)
+    with torch.cuda.device(_producer_device()):
+        _lib.check(_lib.load().bikv_producer_publish(arr, len(shape), _CODE_OF[dtype], _stream()))
 
 
 def producer_set_backpressure(enabled, timeout_ms=-1):

@@ -380,6 +380,16 @@ int bikv_producer_copy_tokens(const void* src, int64_t src_bytes, const int64_t*
 int bikv_producer_send(const void* dev_src, size_t bytes, const int64_t* shape, size_t ndim,
                        int32_t dtype_code, void* stream);
 
+/* The producer's two halves on their own, for callers that fill the ring themselves — a layered
+ * gather whose staging image IS the consumer's ring window, the way block_per_page_copy_kernel
+ * writes straight into the mapped buffer (copy_kernel.cu:92-113). bikv_producer_reserve applies the
+ * reference's wrap rule (copy_kernel.cu:87-89) and returns the device pointer to write `bytes` at;
+ * bikv_producer_publish waits for `stream`, fails with BIKV_EBOUNDS (publishing nothing) if a kernel
+ * skipped work, and then does the reference's bookkeeping (copy_kernel.cu:116-128) for exactly the
+ * reserved bytes. One reservation at a time. */
+int bikv_producer_reserve(size_t bytes, void** ptr);
+int bikv_producer_publish(const int64_t* shape, size_t ndim, int32_t dtype_code, void* stream);
+
 /* consumer_receive (ipc_service.cpp:146-168): sem_wait(sem_start) (timeout_ms < 0 = wait forever,
  * as the reference does; on timeout returns BIKV_ESTATE), then hands out a NON-OWNING pointer into
  * the ring, valid until the producer wraps over it. */

@@ -352,3 +352,47 @@ def test_persistent_index_buffers_for_offsets_and_batches(ipc, oracle, cuda):
             st, _ = kv.gather(b)
             kv.check()
             assert st.cpu().numpy().tobytes() == oracle.gather_layered_c(planes_h, reqs, layout).tobytes()
+
+
+@pytest.mark.parametrize("layout", ["layer_major", "page_major"])
+def test_layered_gather_straight_into_the_ring(ipc, oracle, cuda, layout):
+    """The staging image of a layered gather IS the consumer's ring window (what a transfer between
+    two GPUs does with a peer-mapped buffer): reserve, gather into the window, publish."""
+    import bikv_pagecopy as bk
+    print(f"[case] layered gather into the ring, {layout}", flush=True)
+    name = f"/bikv_test_ringgather_{os.getpid()}"
+    rng = np.random.default_rng(37)
+    n_planes, n_pages, P, H, D = 6, 48, 16, 2, 64
+    tile = P * H * D * 2
+    pool_h = rng.integers(0, 256, size=(n_planes, n_pages, tile), dtype=np.uint8)
+    pool = bk.PagedKVPool.from_stacked(torch.from_numpy(pool_h).to(cuda), plane_dims=1)
+    ipc.consumer_init(0, name, int(2.5 * 20 * n_planes * tile))
+    ipc.producer_init(0, name)
+    ctrl = ipc._lib.load().bikv_producer_control().contents
+    offsets = []
+    for k in range(4):                                      # the fourth transfer wraps
+        reqs = [rng.permutation(n_pages)[:11], rng.permutation(n_pages)[:9]]
+        batch = pool.make_batch(reqs, layout)
+        window = ipc.producer_reserve(batch.n_slots * tile)
+        pool.gather(batch, window)
+        shape = (n_planes, 20, P, H, D) if layout == "layer_major" else (20, n_planes, P, H, D)
+        ipc.producer_publish(shape, torch.float16)
+        offsets.append(int(ctrl.last_valid_offset))
+        got = ipc.consumer_receive(timeout_ms=5000)
+        assert tuple(got.shape) == shape and got.dtype == torch.float16
+        assert got.cpu().contiguous().view(torch.uint8).numpy().tobytes() == oracle.gather_layered_c(pool_h, reqs, layout).tobytes(), k
+    per = 20 * n_planes * tile
+    assert offsets == [0, per, 0, per]
+    # a kernel that skipped work is not published
+    bad = pool.make_batch([[1, 2, 3]], layout)
+    bad.index[0, 1] = n_pages + 7
+    before = (int(ctrl.last_valid_offset), int(ctrl.current_offset))
+    window = ipc.producer_reserve(bad.n_slots * tile)
+    pool.gather(bad, window)
+    with pytest.raises(RuntimeError, match="page-id"):
+        ipc.producer_publish((3 * n_planes, P, H, D), torch.float16)
+    assert (int(ctrl.last_valid_offset), int(ctrl.current_offset)) == before
+    with pytest.raises(RuntimeError, match="timed out"):
+        ipc.consumer_receive(timeout_ms=50)
+    with pytest.raises(RuntimeError, match="does not fit"):
+        ipc.producer_reserve(1 << 40)
