@@ -126,3 +126,103 @@ def test_two_process_page_copy_over_hip_ipc(oracle, cuda, backpressure):
         want = np.zeros(N_RUNS * PAGE_ELEMS, dtype=np.uint16)
         oracle.copy_runs_c(pool, want, so, do, PAGE_ELEMS)
         assert got == want.tobytes(), f"transfer {k} differs"
+
+
+# ---- a whole transfer between two processes: layered gather -> ring -> layered scatter -------------
+L_PLANES, L_PAGES, L_TILE, L_TRANSFERS = 4, 40, 8192, 4
+
+
+def _layer_pool(seed):
+    return np.random.default_rng(seed).integers(0, 256, size=(L_PLANES, L_PAGES, L_TILE), dtype=np.uint8)
+
+
+def _layer_transfer(k):
+    rng = np.random.default_rng(2000 + k)
+    src = [rng.permutation(L_PAGES)[:7], rng.permutation(L_PAGES)[:5]]          # gathered from the sender's pool
+    perm = rng.permutation(L_PAGES)
+    dst = [perm[:7], perm[7:12]]                                                # unique pages of the receiver's pool
+    return src, dst
+
+
+def _layer_receiver(name, ready, out):
+    try:
+        _paths()
+        import torch
+        import ipc_service
+        import bikv_pagecopy as bk
+        per = 12 * L_PLANES * L_TILE
+        ipc_service.consumer_init(0, name, 5 * per // 2)
+        ready.set()
+        pool_d = torch.from_numpy(_layer_pool(7)).cuda()
+        pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+        for k in range(L_TRANSFERS):
+            _, dst = _layer_transfer(k)
+            t = ipc_service.consumer_receive(timeout_ms=60000)
+            assert tuple(t.shape) == (L_PLANES, 12, L_TILE) and t.dtype == torch.uint8
+            pool.scatter(pool.make_batch(dst, "layer_major"), t.reshape(-1))
+            pool.check()                                    # the ring window has been read
+            ipc_service.consumer_release()
+        digest = pool_d.cpu().numpy().tobytes()
+        ipc_service.consumer_cleanup()
+        out.put(("receiver", "ok", digest))
+    except Exception as e:  # noqa: BLE001
+        out.put(("receiver", f"{type(e).__name__}: {e}", None))
+
+
+def _layer_sender(name, ready, out):
+    try:
+        _paths()
+        import torch
+        import ipc_service
+        import bikv_pagecopy as bk
+        if not ready.wait(120):
+            raise RuntimeError("receiver did not come up")
+        ipc_service.producer_init(0, name)
+        ipc_service.producer_set_backpressure(True, timeout_ms=60000)
+        pool = bk.PagedKVPool.from_stacked(torch.from_numpy(_layer_pool(5)).cuda(), plane_dims=1)
+        for k in range(L_TRANSFERS):
+            src, _ = _layer_transfer(k)
+            batch = pool.make_batch(src, "layer_major")
+            window = ipc_service.producer_reserve(batch.n_slots * L_TILE)
+            pool.gather(batch, window)                      # kernels store into the receiver's memory
+            ipc_service.producer_publish((L_PLANES, 12, L_TILE), torch.uint8)
+        ipc_service.producer_cleanup()
+        out.put(("sender", "ok", None))
+    except Exception as e:  # noqa: BLE001
+        out.put(("sender", f"{type(e).__name__}: {e}", None))
+
+
+def test_two_process_layered_transfer(oracle, cuda):
+    """Sender gathers request pages of its paged pool straight into the receiver's ring (the ring is
+    the staging image, mapped through a HIP IPC handle); the receiver scatters each image into pages of
+    its own pool. Paced by sem_complete only. The receiver's final pool must equal the oracle's."""
+    print("[case] two processes: layered gather -> ring -> layered scatter", flush=True)
+    ctx = mp.get_context("spawn")
+    name = f"/bikv_test_2proc_layer_{os.getpid()}"
+    ready, out = ctx.Event(), ctx.Queue()
+    procs = [ctx.Process(target=_layer_receiver, args=(name, ready, out)),
+             ctx.Process(target=_layer_sender, args=(name, ready, out))]
+    for p in procs:
+        p.start()
+    results = {}
+    try:
+        for _ in procs:
+            who, status, payload = out.get(timeout=240)
+            results[who] = (status, payload)
+    finally:
+        for p in procs:
+            p.join(timeout=30)
+            if p.is_alive():
+                p.terminate()
+        try:
+            os.unlink("/dev/shm" + name)
+        except FileNotFoundError:
+            pass
+    assert results["sender"][0] == "ok", results
+    assert results["receiver"][0] == "ok", (results["receiver"][0], results["sender"][0])
+    src_pool, want = _layer_pool(5), _layer_pool(7)
+    for k in range(L_TRANSFERS):
+        src, dst = _layer_transfer(k)
+        image = oracle.gather_layered_c(src_pool, src, "layer_major")
+        oracle.scatter_layered_c(want, dst, image, "layer_major")
+    assert results["receiver"][1] == want.tobytes()
