@@ -69,20 +69,22 @@ class RunIndexPool:
         self.max_pages = int(max_pages)
         self.rows = int(rows)
         self.device = torch.device(device)
-        self.dev = torch.full((self.rows, self.max_pages), -1, dtype=torch.int64, device=self.device)
-        self.host = torch.empty((self.rows, self.max_pages), dtype=torch.int64, pin_memory=True)
+        self.dev = torch.full((self.rows * self.max_pages,), -1, dtype=torch.int64, device=self.device)
+        self.host = torch.empty(self.rows * self.max_pages, dtype=torch.int64, pin_memory=True)
+        self._host_np = self.host.numpy()
         self._busy = None
 
     def load(self, table: np.ndarray) -> torch.Tensor:
-        """table: [r, n] int64 with r <= rows, n <= max_pages. Returns the [r, n] device rows
-        (each row contiguous), valid until the next load()."""
+        """table: [r, n] int64 with r <= rows, n <= max_pages. Returns it as an [r, n] device tensor
+        (the leading r*n entries of the buffer), valid until the next load()."""
         r, n = table.shape
         if r > self.rows or n > self.max_pages:
             raise RuntimeError(f"Requested {n} exceeds pool size {self.max_pages}")   # kvcache.py:84
         if self._busy is not None:
             self._busy.synchronize()          # the previous upload still reads the mirror
-        self.host[:r, :n] = torch.from_numpy(np.ascontiguousarray(table, dtype=np.int64))
-        self.dev[:r, :n].copy_(self.host[:r, :n], non_blocking=True)
-        self._busy = torch.cuda.Event()
+        self._host_np[: r * n].reshape(r, n)[...] = table
+        self.dev[: r * n].copy_(self.host[: r * n], non_blocking=True)
+        if self._busy is None:
+            self._busy = torch.cuda.Event()
         self._busy.record(torch.cuda.current_stream(self.device))
-        return self.dev[:r, :n]
+        return self.dev[: r * n].view(r, n)
