@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libbikv_pagecopy.so")
 
 MAX_DIM = 5
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 OK, EINVAL, EHIP, ESYS, ESTATE, EBOUNDS, ERANGE = 0, -1, -2, -3, -4, -5, -6
 ST_SRC_RANGE, ST_DST_RANGE, ST_PAGE_ID = 1, 2, 4
@@ -33,6 +33,8 @@ class PoolDesc(C.Structure):
         ("scale_tile_bytes", C.c_int64),
         ("scale_page_stride_bytes", C.c_int64),
         ("scale_plane_base", C.POINTER(C.c_void_p)),
+        ("row_bytes", C.c_int64),
+        ("row_stride_bytes", C.c_int64),
     ]
 
 

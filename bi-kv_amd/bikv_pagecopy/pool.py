@@ -97,7 +97,8 @@ class PagedKVPool:
     def __init__(self, plane_ptrs: Sequence[int], n_pages: int, tile_bytes: int,
                  page_stride_bytes: int, device, dtype=torch.uint8,
                  scale_plane_ptrs: Optional[Sequence[int]] = None, scale_tile_bytes: int = 0,
-                 scale_page_stride_bytes: int = 0, keepalive=None):
+                 scale_page_stride_bytes: int = 0, keepalive=None, row_bytes: int = 0,
+                 row_stride_bytes: int = 0):
         self.device = torch.device(device)
         if self.device.type != "cuda":
             raise RuntimeError("PagedKVPool needs a GPU pool (device must be cuda)")
@@ -115,6 +116,8 @@ class PagedKVPool:
         d.n_pages = self.n_pages
         d.tile_bytes = self.tile_bytes
         d.page_stride_bytes = self.page_stride_bytes
+        d.row_bytes = int(row_bytes)
+        d.row_stride_bytes = int(row_stride_bytes)
         arr = (C.c_void_p * self.n_planes)(*[int(p) for p in plane_ptrs])
         d.plane_base = C.cast(arr, C.POINTER(C.c_void_p))
         if scale_plane_ptrs is not None:
@@ -171,6 +174,24 @@ class PagedKVPool:
             sp = scale.reshape((-1,) + tuple(scale.shape[plane_dims:]))
             splanes = [sp[q] for q in range(sp.shape[0])]
         return cls.from_planes([planes[q] for q in range(planes.shape[0])], splanes)
+
+    @classmethod
+    def from_token_kv_layers(cls, layers: Sequence[torch.Tensor], block_tokens: int):
+        """layers[l] is [blocks*block_tokens, 2, heads, dim] as the Worker holds its cache
+        (Bi-KV/Worker/Worker.py:74-78): K and V interleave token by token, so the tile of (page, K|V) is
+        block_tokens rows of heads*dim elements, two rows apart. Plane q = 2*l + k."""
+        for t in layers:
+            cls._check_plane(t)
+        t0 = layers[0]
+        if t0.dim() != 4 or t0.shape[1] != 2 or t0.shape[0] % block_tokens:
+            raise RuntimeError("expected [blocks*block_tokens, 2, heads, dim] per layer")
+        if any(t.shape != t0.shape or t.dtype != t0.dtype for t in layers):
+            raise RuntimeError("all layers must share shape and dtype")
+        es = t0.element_size()
+        row = t0.shape[2] * t0.shape[3] * es
+        ptrs = [t.data_ptr() + k * row for t in layers for k in (0, 1)]
+        return cls(ptrs, t0.shape[0] // block_tokens, block_tokens * row, block_tokens * 2 * row, t0.device,
+                   dtype=t0.dtype, keepalive=list(layers), row_bytes=row, row_stride_bytes=2 * row)
 
     @classmethod
     def from_layers_kv_adjacent(cls, layers: Sequence[torch.Tensor]):

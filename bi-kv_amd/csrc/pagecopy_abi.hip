@@ -108,6 +108,7 @@ struct bikv_pool {
   int n_planes;
   int64_t n_pages;
   int64_t tile_bytes, page_stride;
+  int64_t row_bytes, row_stride;    // row_bytes == tile_bytes: contiguous tiles
   int64_t scale_tile_bytes, scale_page_stride;
   const char** d_plane_base;        // device table: payload planes, then scale planes
   uint64_t align_bits;              // OR of every base, stride and tile size (payload)
@@ -188,9 +189,19 @@ extern "C" int bikv_pool_create(const bikv_pool_desc* d, bikv_pool** out) {
   if (has_scale && (!d->scale_plane_base || d->scale_page_stride_bytes < d->scale_tile_bytes))
     return fail(BIKV_EINVAL, "scale class needs scale_plane_base and scale_page_stride_bytes >= scale_tile_bytes");
   if (d->scale_tile_bytes < 0) return fail(BIKV_EINVAL, "negative scale_tile_bytes");
+  int64_t row_bytes = d->tile_bytes, row_stride = d->tile_bytes;
+  if (d->row_bytes < 0 || d->row_stride_bytes < 0) return fail(BIKV_EINVAL, "negative row_bytes or row_stride_bytes");
+  if (d->row_bytes > 0 && d->row_bytes != d->tile_bytes) {
+    row_bytes = d->row_bytes;
+    row_stride = d->row_stride_bytes;
+    if (d->tile_bytes % row_bytes != 0 || row_stride < row_bytes)
+      return fail(BIKV_EINVAL, "need tile_bytes %% row_bytes == 0 and row_stride_bytes >= row_bytes (got %lld, %lld, %lld)",
+                  (long long)d->tile_bytes, (long long)row_bytes, (long long)row_stride);
+  }
 
   std::vector<const char*> table((size_t)d->n_planes * 2, nullptr);
-  uint64_t ab = (uint64_t)d->tile_bytes | (uint64_t)d->page_stride_bytes, sab = 0;
+  uint64_t ab = (uint64_t)d->tile_bytes | (uint64_t)d->page_stride_bytes | (uint64_t)row_bytes |
+                (uint64_t)row_stride, sab = 0;
   for (int q = 0; q < d->n_planes; ++q) {
     if (!d->plane_base[q]) return fail(BIKV_EINVAL, "plane_base[%d] is null", q);
     table[q] = static_cast<const char*>(d->plane_base[q]);
@@ -221,6 +232,8 @@ extern "C" int bikv_pool_create(const bikv_pool_desc* d, bikv_pool** out) {
   p->n_pages = d->n_pages;
   p->tile_bytes = d->tile_bytes;
   p->page_stride = d->page_stride_bytes;
+  p->row_bytes = row_bytes;
+  p->row_stride = row_stride;
   p->scale_tile_bytes = has_scale ? d->scale_tile_bytes : 0;
   p->scale_page_stride = has_scale ? d->scale_page_stride_bytes : 0;
   p->d_plane_base = static_cast<const char**>(dtab);
@@ -278,6 +291,11 @@ static int build_move(const bikv_pool* pool, const bikv_page_batch* b, const voi
   m->payload.n_slots = staging_bytes / pool->tile_bytes;
   m->payload.tile_bytes = pool->tile_bytes;
   m->payload.page_stride = pool->page_stride;
+  m->payload.row_bytes = pool->row_bytes;
+  m->payload.row_stride = pool->row_stride;
+  m->payload.log2_row = -1;
+  if ((pool->row_bytes & (pool->row_bytes - 1)) == 0)
+    for (m->payload.log2_row = 0; (int64_t(1) << m->payload.log2_row) < pool->row_bytes;) ++m->payload.log2_row;
   m->payload.vec_width = lowbit_width(pool->align_bits | (uint64_t)staging);
   if (has_scale) {
     m->scale.plane_base = pool->d_plane_base + pool->n_planes;
@@ -285,6 +303,9 @@ static int build_move(const bikv_pool* pool, const bikv_page_batch* b, const voi
     m->scale.n_slots = scale_bytes / pool->scale_tile_bytes;
     m->scale.tile_bytes = pool->scale_tile_bytes;
     m->scale.page_stride = pool->scale_page_stride;
+    m->scale.row_bytes = pool->scale_tile_bytes;
+    m->scale.row_stride = pool->scale_tile_bytes;
+    m->scale.log2_row = -1;
     m->scale.vec_width = lowbit_width(pool->scale_align_bits | (uint64_t)scale_staging);
   }
   return BIKV_OK;

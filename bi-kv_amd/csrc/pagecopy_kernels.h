@@ -17,6 +17,9 @@ struct TileClass {
   int64_t n_slots;                // slots available in the staging window
   int64_t tile_bytes;
   int64_t page_stride;
+  int64_t row_bytes;              // pool side: the tile is tile_bytes/row_bytes rows of row_bytes bytes,
+  int64_t row_stride;             // row_stride apart (row_bytes == tile_bytes: one contiguous tile)
+  int32_t log2_row;               // log2(row_bytes) when that is a power of two, else -1
   int32_t vec_width;              // widest power of two (<=16) dividing every address and size
   int32_t log2_rows;              // segment mover: tile_bytes == 4096 << log2_rows; wave mover: pieces
                                   // per tile == 1 << log2_rows, or -1 when that is not a power of two

@@ -76,6 +76,16 @@ __device__ __forceinline__ void raise(uint32_t* status, int slot) {
 // Layered tile move
 // ---------------------------------------------------------------------------------------------
 
+// Pool-side offset of byte `t` of a tile. A tile is contiguous in staging; in the pool it may be cut
+// into rows that sit row_stride apart (the Worker's per-layer tensors [tokens, 2, heads, dim],
+// Bi-KV/Worker/Worker.py:74-78, interleave K and V token by token: a (page, K|V) tile is block_tokens
+// rows of heads*dim elements, two rows apart).
+__device__ __forceinline__ uint64_t pool_offset(const TileClass& c, uint64_t t) {
+  if (c.row_bytes == c.tile_bytes) return t;
+  const uint64_t r = c.log2_row >= 0 ? t >> c.log2_row : t / (uint64_t)c.row_bytes;
+  return r * (uint64_t)c.row_stride + (t - r * (uint64_t)c.row_bytes);
+}
+
 // Resolves the (pool address, staging address) pair of every page of this workgroup's segment
 // into LDS. A tile that fails a bounds check gets a null pair and is skipped by the movers.
 template <int DIR>
@@ -167,7 +177,8 @@ __device__ __forceinline__ void move_generic_vw(const TileClass& c, int nseg,
     if (pool == 0) continue;
     const uint64_t stg = s_stage[tt];
     const uint64_t off = (uint64_t)ww * VW;
-    st<false, T>((DIR == 0 ? stg : pool) + off, ld<false, T>((DIR == 0 ? pool : stg) + off));
+    const uint64_t poff = pool_offset(c, off);      // VW divides row_bytes and row_stride
+    st<false, T>(DIR == 0 ? stg + off : pool + poff, ld<false, T>(DIR == 0 ? pool + poff : stg + off));
   }
 }
 
@@ -304,8 +315,10 @@ __global__ __launch_bounds__(B) void tile_move_wave_kernel(const MoveArgs a) {
     const uint64_t pool = plane + (uint64_t)(pid * a.payload.page_stride);
     const uint64_t stg = (uint64_t)a.payload.staging + (uint64_t)(slot * a.payload.tile_bytes);
     const uint64_t off = (uint64_t)part * (B * 16u) + threadIdx.x * 16u;
-    if (off < (uint64_t)a.payload.tile_bytes)   // the last piece of a tile may be ragged
-      move16<POL>((DIR == 0 ? pool : stg) + off, (DIR == 0 ? stg : pool) + off);
+    if (off < (uint64_t)a.payload.tile_bytes) { // the last piece of a tile may be ragged
+      const uint64_t poff = pool_offset(a.payload, off);   // 16 divides row_bytes and row_stride
+      move16<POL>(DIR == 0 ? pool + poff : stg + off, DIR == 0 ? stg + off : pool + poff);
+    }
   } else {
     // scale class: one lane per vector; order 0 spreads the lanes over the pages of plane q,
     // order 1 over the planes of page i. The launcher keeps (scale workgroups * B) below 2^32.
@@ -500,7 +513,7 @@ hipError_t launch_tile_move(int dir, MoveArgs& a, hipStream_t stream) {
   // fast mover: 16-byte aligned tiles of 2^k rows of 4 KiB
   const int64_t nrows = a.payload.tile_bytes / kRowBytes;
   const bool rows = a.payload.vec_width == 16 && (a.payload.tile_bytes % kRowBytes) == 0 &&
-                    (nrows & (nrows - 1)) == 0;
+                    (nrows & (nrows - 1)) == 0 && a.payload.row_bytes == a.payload.tile_bytes;
   a.payload.log2_rows = 0;
   if (rows)
     while ((int64_t(1) << a.payload.log2_rows) < nrows) ++a.payload.log2_rows;

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define BIKV_ABI_VERSION 1
+#define BIKV_ABI_VERSION 2
 
 enum {
   BIKV_OK = 0,
@@ -134,6 +134,14 @@ typedef struct bikv_pool_desc {
   int64_t scale_tile_bytes;        /* 0 = no scale class */
   int64_t scale_page_stride_bytes;
   const void* const* scale_plane_base; /* HOST array of n_planes device pointers, or NULL */
+  /* Tiles that are not contiguous in the pool: row_bytes > 0 cuts the payload tile into
+   * tile_bytes/row_bytes rows of row_bytes bytes that sit row_stride_bytes apart (in staging the
+   * tile stays contiguous). This is the Worker's own per-layer tensor [tokens, 2, heads, dim]
+   * (Worker.py:74-78), where K and V interleave token by token: plane (l, k) has plane_base =
+   * layer l + k*heads*dim elements, row = heads*dim elements, row stride = 2 rows, page stride =
+   * block_tokens row strides. 0 = contiguous tiles. */
+  int64_t row_bytes;
+  int64_t row_stride_bytes;
 } bikv_pool_desc;
 
 int bikv_pool_create(const bikv_pool_desc* desc, bikv_pool** out);

@@ -244,6 +244,33 @@ def scatter_layered_c(pool, requests, staging, layout="layer_major"):
     assert bad == 0, f"{bad} page ids out of range"
 
 
+def planes_of_token_kv_layers(layers, block_tokens):
+    """The Worker's per-layer tensors [blocks*block_tokens, 2, heads, dim] (Worker/Worker.py:74-78)
+    restated as the planar pool [2*L, blocks, block_tokens*heads*dim] the layered functions take:
+    plane 2*l + k, page b = the block's tokens of K (k = 0) or V (k = 1), token-major. Pure numpy
+    reshapes: the statement of the layout, independent of any stride arithmetic."""
+    planes = []
+    for a in layers:
+        slots, two, h, d = a.shape
+        assert two == 2 and slots % block_tokens == 0
+        blk = a.reshape(slots // block_tokens, block_tokens, 2, h * d)
+        for k in (0, 1):
+            planes.append(np.ascontiguousarray(blk[:, :, k, :]).reshape(slots // block_tokens, block_tokens * h * d))
+    return np.stack(planes)
+
+
+def token_kv_layers_of_planes(planes, block_tokens, heads, dim):
+    """Inverse of planes_of_token_kv_layers: list of [blocks*block_tokens, 2, heads, dim] arrays."""
+    n_planes, blocks, _ = planes.shape
+    out = []
+    for l in range(n_planes // 2):
+        a = np.empty((blocks, block_tokens, 2, heads * dim), dtype=planes.dtype)
+        for k in (0, 1):
+            a[:, :, k, :] = planes[2 * l + k].reshape(blocks, block_tokens, heads * dim)
+        out.append(a.reshape(blocks * block_tokens, 2, heads, dim))
+    return out
+
+
 def gather_layered_np(pool, requests, layout="layer_major"):
     """out_r[q][j] = pool[q][ids_r[j]] (layer-major) or out_r[j][q] (page-major), requests packed."""
     parts = []

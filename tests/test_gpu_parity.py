@@ -238,6 +238,46 @@ def test_kv_adjacent_layer_layout(bk, oracle, cuda):
 
 
 # ---- edge cases ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("P,H,D,dtype", [
+    (16, 2, 128, torch.float16),      # the Worker's own shape: 512-byte rows, 8 KiB tiles
+    (16, 4, 128, torch.bfloat16),     # 1 KiB rows: one piece of the wave mover per row
+    (16, 8, 128, torch.float16),      # 2 KiB rows
+    (8, 3, 64, torch.float16),        # 384-byte rows (not a power of two)
+    (4, 1, 8, torch.float32),         # 32-byte rows, 128-byte tiles: the segment mover
+    (5, 2, 24, torch.uint8),          # 48-byte rows, 240-byte tiles
+])
+@pytest.mark.parametrize("layout", ["layer_major", "page_major"])
+def test_worker_token_interleaved_layers(bk, oracle, cuda, P, H, D, dtype, layout):
+    """The Worker's per-layer cache [blocks*block, 2, heads, dim] (Worker/Worker.py:74-78) as the pool:
+    a (page, K|V) tile is `block` rows of heads*dim elements, two rows apart."""
+    _announce(f"worker-form pool P={P} H={H} D={D} {dtype} {layout}")
+    rng = np.random.default_rng(P * 1000 + H * 10 + D)
+    es = torch.empty((), dtype=dtype).element_size()
+    np_dt = {1: np.uint8, 2: np.uint16, 4: np.uint32}[es]
+    L, blocks = 3, 37
+    layers_h = [rng.integers(0, 256, size=(blocks * P, 2, H, D, es), dtype=np.uint8).view(np_dt)[..., 0].copy() for _ in range(L)]
+    layers_d = [torch.from_numpy(a.view(np.uint8)).to(cuda).view(dtype).view(a.shape) for a in layers_h]
+    pool = bk.PagedKVPool.from_token_kv_layers(layers_d, P)
+    assert pool.n_planes == 2 * L and pool.tile_bytes == P * H * D * es
+    planes_h = oracle.planes_of_token_kv_layers(layers_h, P).view(np.uint8)
+    reqs = [rng.permutation(blocks)[:15], np.array([3, 3]), rng.permutation(blocks)[:1], np.array([], dtype=np.int64)]
+    batch = pool.make_batch(reqs, layout)
+    st, _ = pool.gather(batch)
+    pool.check()
+    assert _to_np(st).tobytes() == oracle.gather_layered_c(planes_h, reqs, layout).tobytes()
+    perm = rng.permutation(blocks)
+    sreqs = [perm[:9], perm[9:20]]
+    sb = pool.make_batch(sreqs, layout)
+    src = rng.integers(0, 256, size=sb.n_slots * pool.tile_bytes, dtype=np.uint8)
+    pool.scatter(sb, torch.from_numpy(src).to(cuda))
+    pool.check()
+    oracle.scatter_layered_c(planes_h, sreqs, src, layout)
+    want = oracle.token_kv_layers_of_planes(planes_h.view(np_dt), P, H, D)
+    for l in range(L):
+        assert _to_np(layers_d[l]).tobytes() == want[l].tobytes(), f"layer {l}"
+    pool.close()
+
+
 def test_empty_batch_and_empty_requests(bk, oracle, cuda):
     _announce("empty")
     pool_d = torch.zeros((2, 8, 4096), dtype=torch.uint8, device=cuda)

@@ -361,3 +361,21 @@ def test_packed_offsets_with_tail_lengths_deliver_exactly_each_items_tokens(orac
     # already leaves the buffer
     over = np.full((total, ept), 0xA5A5, dtype=np.uint16)
     assert oracle.copy_runs_c(pool, over, np.asarray(so) * ept, np.asarray(do) * ept, page_size * ept) >= 1
+
+
+def test_worker_form_planes_are_the_tokens_of_each_block(oracle):
+    """planes_of_token_kv_layers against explicit indexing: element (plane 2l+k, block b, token t, head h, d)
+    is layers[l][b*P + t, k, h, d]; and the inverse restores the layers."""
+    rng = np.random.default_rng(71)
+    P, H, D, L, blocks = 4, 3, 8, 2, 5
+    layers = [rng.integers(0, 65536, size=(blocks * P, 2, H, D), dtype=np.uint16) for _ in range(L)]
+    planes = oracle.planes_of_token_kv_layers(layers, P)
+    assert planes.shape == (2 * L, blocks, P * H * D)
+    for l in range(L):
+        for k in (0, 1):
+            for b in range(blocks):
+                for t in range(P):
+                    got = planes[2 * l + k, b].reshape(P, H, D)[t]
+                    assert np.array_equal(got, layers[l][b * P + t, k])
+    back = oracle.token_kv_layers_of_planes(planes, P, H, D)
+    assert all(np.array_equal(a, b) for a, b in zip(back, layers))
