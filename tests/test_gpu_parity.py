@@ -275,6 +275,26 @@ def test_worker_token_interleaved_layers(bk, oracle, cuda, P, H, D, dtype, layou
     want = oracle.token_kv_layers_of_planes(planes_h.view(np_dt), P, H, D)
     for l in range(L):
         assert _to_np(layers_d[l]).tobytes() == want[l].tobytes(), f"layer {l}"
+    # a window of planes that starts on a V plane
+    d = batch.desc(plane_begin=1, plane_count=3)
+    win = torch.full((batch.n_slots * pool.tile_bytes,), 0xA5, dtype=torch.uint8, device=cuda)
+    from bikv_pagecopy import _lib
+    import ctypes as C
+    _lib.check(_lib.load().bikv_gather_pages(pool._h, C.byref(d), win.data_ptr(), win.numel(), None, 0,
+                                             C.c_void_p(torch.cuda.current_stream(cuda).cuda_stream)))
+    pool.check()
+    full = oracle.gather_layered_c(planes_h, reqs, layout).reshape(batch.n_slots, pool.tile_bytes)
+    got = _to_np(win).reshape(batch.n_slots, pool.tile_bytes)
+    n_pl = pool.n_planes
+    for r in range(len(reqs)):
+        m = len(reqs[r])
+        if m == 0:
+            continue
+        s0 = int(batch.req_first_slot[r])
+        blk_got, blk_want = got[s0:s0 + m * n_pl], full[s0:s0 + m * n_pl]
+        view = (lambda a: a.reshape(n_pl, m, -1)) if layout == "layer_major" else (lambda a: a.reshape(m, n_pl, -1).transpose(1, 0, 2))
+        g3, w3 = view(blk_got), view(blk_want)
+        assert np.array_equal(g3[1:4], w3[1:4]) and (g3[0] == 0xA5).all() and (g3[4:] == 0xA5).all()
     pool.close()
 
 
