@@ -34,7 +34,9 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch as a multiple of the algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this file, each scaled by the same counter's reading for the plain-copy
 # calibration launch below (summaries under profiles/). None = not measured for that workload.
-MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9949, "scatter": 1.0003}}
+MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9949, "scatter": 1.0003},
+                          "qwen2_7b_token_major": {"gather": 0.9997, "scatter": 1.0002},
+                          "layout_change": {"load": 1.0035, "store": 1.0029}}
 
 
 def parse_args():
@@ -597,7 +599,9 @@ def run_token_major(args, bk, workloads, dev):
                     "scatter": {"GBps": round(alg_s / s_ms / 1e6, 1), "avg_ms": round(s_ms, 4)}},
         "roofline": {"bound": "hbm", "kernel": "bikv::copy_runs_wave_kernel", "achieved": round(alg / ms / 1e6, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(alg / ms / 1e6 / HBM_PEAK_GBPS, 4),
-                     "traffic": None, "alg_bytes_per_launch": alg, "avg_launch_ms": round(ms, 4)},
+                     "traffic": (int(alg * MEASURED_TRAFFIC_RATIO["qwen2_7b_token_major"]["gather" if slow_g else "scatter"])
+                                 if not args.pool_pages else None),
+                     "alg_bytes_per_launch": alg, "avg_launch_ms": round(ms, 4)},
     }
 
 
@@ -673,7 +677,9 @@ def run_layout_change(args, bk, dev):
         "pages_per_s": round(2 * n_pages / (wall / args.steps), 1), "bit_exact": True,
         "roofline": {"bound": "hbm", "kernel": f"bikv::transpose_pairs_kernel<{1 if slow_is_load else 0}, 512>",
                      "achieved": round(alg / (ms_dom * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(alg / (ms_dom * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(alg / (ms_dom * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "traffic": (int(alg * MEASURED_TRAFFIC_RATIO["layout_change"]["load" if slow_is_load else "store"])
+                                 if not args.pool_pages else None),
                      "alg_bytes_per_launch": alg, "avg_launch_ms": round(ms_dom, 4)},
         "kernels": {"load": {"GBps": round(alg / (np.mean(l_ms) * 1e-3) / 1e9, 1), "avg_ms": round(float(np.mean(l_ms)), 4)},
                     "store": {"GBps": round(alg / (np.mean(s_ms) * 1e-3) / 1e9, 1), "avg_ms": round(float(np.mean(s_ms)), 4)}},
