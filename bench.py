@@ -675,7 +675,7 @@ def run_layout_change(args, bk, dev):
                                f"{n_pages} pages of {P} tokens loaded then stored per step"},
         "pct_of_hbm_peak": round(100 * 2 * alg / (wall / args.steps) / 1e9 / HBM_PEAK_GBPS, 2),
         "pages_per_s": round(2 * n_pages / (wall / args.steps), 1), "bit_exact": True,
-        "roofline": {"bound": "hbm", "kernel": f"bikv::transpose_pairs_kernel<{1 if slow_is_load else 0}, 512>",
+        "roofline": {"bound": "hbm", "kernel": f"bikv::transpose_pairs_kernel<{1 if slow_is_load else 0}, 2, 512>",
                      "achieved": round(alg / (ms_dom * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(alg / (ms_dom * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                      "traffic": (int(alg * MEASURED_TRAFFIC_RATIO["layout_change"]["load" if slow_is_load else "store"])
