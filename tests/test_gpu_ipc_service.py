@@ -396,3 +396,31 @@ def test_layered_gather_straight_into_the_ring(ipc, oracle, cuda, layout):
         ipc.consumer_receive(timeout_ms=50)
     with pytest.raises(RuntimeError, match="does not fit"):
         ipc.producer_reserve(1 << 40)
+
+
+def test_packed_transfer_against_committed_digest(ipc, cuda):
+    """The token-exact packed transfer against tests/golden/packed_and_layout.json (no oracle in the loop)."""
+    import hashlib
+    import importlib.util
+    import json
+    from bikv_pagecopy import kvcache_calls
+    print("[case] packed transfer golden digest", flush=True)
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(golden, "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    with open(os.path.join(golden, "packed_and_layout.json")) as f:
+        e = json.load(f)["packed_transfer"]
+    pool, pages_list, tokens, page_size = mg.packed_case()
+    dims = (12, 1, 1, 2)                                     # 24 elements per token
+    name = f"/bikv_test_goldpack_{os.getpid()}"
+    ipc.consumer_init(0, name, 8 << 20)
+    ipc.producer_init(0, name)
+    pool_d = torch.from_numpy(pool.view(np.int16)).view(torch.float16).to(cuda)
+    info = {"infer_worker": 0, "token_num": sum(tokens), "id_token_pair": list(enumerate(tokens)),
+            "cache_pages_list": pages_list}
+    n, total = kvcache_calls.shared_data_batch_pages(pool_d, info, page_size, dims, "exact")
+    got = ipc.consumer_receive(timeout_ms=5000)
+    assert total == e["total_tokens"] and tuple(got.shape) == (total,) + dims
+    digest = hashlib.sha256(got.cpu().contiguous().view(torch.int16).numpy().tobytes()).hexdigest()
+    assert digest == e["received_sha256"]

@@ -137,3 +137,33 @@ def test_bad_ids_are_skipped_and_reported_and_shapes_are_checked(lib, cuda):
         pool.load_token_major(tm.float(), torch.tensor([1], device=cuda))
     with pytest.raises(RuntimeError, match="int64"):
         pool.load_token_major(tm, torch.tensor([1], device=cuda, dtype=torch.int32))
+
+
+@pytest.mark.parametrize("form", ["token_kv", "block_kv"])
+def test_layout_change_against_committed_digests(lib, cuda, form):
+    """The kernels against tests/golden/packed_and_layout.json directly (no oracle in the loop)."""
+    import hashlib
+    import importlib.util
+    import json
+    import os
+    import bikv_pagecopy as bk
+    print(f"[case] layout change golden digests {form}", flush=True)
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(golden, "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    with open(os.path.join(golden, "packed_and_layout.json")) as f:
+        e = json.load(f)[f"layout_change_{form}"]
+    sha = lambda a: hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+    tm, layers, load, store = mg.layout_case(form)
+    tm_d = torch.from_numpy(tm.view(np.int16)).to(cuda).view(torch.float16)
+    layers_d = [torch.from_numpy(a.view(np.int16)).to(cuda).view(torch.float16) for a in layers]
+    P = tm.shape[1]
+    pool = bk.NHDPool.from_token_kv_layers(layers_d, P) if form == "token_kv" else bk.NHDPool.from_block_kv_layers(layers_d)
+    t = lambda a: torch.from_numpy(a).to(cuda)
+    pool.load_token_major(tm_d, t(load[0]), t(load[1]))
+    pool.check()
+    assert sha(np.stack([_to_np(x).view(np.uint16).reshape(layers[0].shape) for x in layers_d])) == e["layers_after_load_sha256"]
+    pool.store_token_major(tm_d, t(store[0]), t(store[1]))
+    pool.check()
+    assert sha(_to_np(tm_d)) == e["tm_after_store_sha256"]

@@ -379,3 +379,29 @@ def test_worker_form_planes_are_the_tokens_of_each_block(oracle):
                     assert np.array_equal(got, layers[l][b * P + t, k])
     back = oracle.token_kv_layers_of_planes(planes, P, H, D)
     assert all(np.array_equal(a, b) for a, b in zip(back, layers))
+
+
+def _golden_cases():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(GOLDEN, "make_golden.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_packed_transfer_and_layout_change_golden_digests(oracle):
+    mg = _golden_cases()
+    with open(os.path.join(GOLDEN, "packed_and_layout.json")) as f:
+        g = json.load(f)
+    pool, pages_list, tokens, page_size = mg.packed_case()
+    assert _sha(pool) == g["packed_transfer"]["pool_sha256"]
+    want = oracle.packed_items_np(pool, pages_list, tokens, page_size)
+    assert want.shape[0] == g["packed_transfer"]["total_tokens"] and _sha(want) == g["packed_transfer"]["received_sha256"]
+    for form in ("token_kv", "block_kv"):
+        tm, layers, load, store = mg.layout_case(form)
+        e = g[f"layout_change_{form}"]
+        assert _sha(tm) == e["tm_sha256"] and _sha(np.stack(layers)) == e["layers_sha256"]
+        assert oracle.transpose_pages_c(layers, form, tm, load[0], load[1], "load") == 0
+        assert _sha(np.stack(layers)) == e["layers_after_load_sha256"]
+        assert oracle.transpose_pages_c(layers, form, tm, store[0], store[1], "store") == 0
+        assert _sha(tm) == e["tm_after_store_sha256"]
