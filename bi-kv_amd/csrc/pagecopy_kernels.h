@@ -101,6 +101,7 @@ struct TransposeArgs {
   int32_t n_layers, head_dim, n_cols;             // n_cols = kv_heads * n_layers * 2
   int32_t block_tokens, elem_bytes;
   int32_t chunk_cols, chunk_rows, pitch;      // filled by the launcher
+  int32_t swz_mask;                           // pair kernel: XOR mask of the 16-byte groups of an LDS row
   uint32_t n_chunks, n_dchunks, tile_words;
   uint32_t* status;
 };

@@ -166,7 +166,8 @@ __global__ __launch_bounds__(kBlock) void transpose_pages_kernel(const Transpose
 // (consecutive lanes = consecutive vectors of a token-major row) over all banks. For 2-byte elements
 // this takes 5.5 LDS and ~60 VALU instructions per 16-byte vector moved; the element-wise kernel
 // above takes 11 and ~105 (three integer divisions per vector).
-// Needs head_dim * ES % 64 == 0 (XOR closure over the 16-byte groups of a row).
+// The XOR mask is the largest 2^k - 1 <= 7 with 2^k dividing the groups of a row, so that the permuted
+// index stays inside the row for every head_dim the entry points accept.
 struct Walk {        // (outer, inner) of a linear index that advances by the block size per step
   int outer, inner;
 };
@@ -260,7 +261,8 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
   const int Cw = a.chunk_cols >> 1;        // column pairs in the tile
   const int vpr = Cw >> UPV_SHIFT;         // 16-byte vectors per token-major row piece
   const int dgs = D / DPV;                 // 16-byte vectors per compute row
-  const int gpr = (D * UB) >> 4;           // 16-byte groups per LDS row (a multiple of 8)
+  const int gpr = (D * UB) >> 4;           // 16-byte groups per LDS row (even)
+  const int sm = a.swz_mask;               // 2^k - 1 with 2^k dividing gpr, at most 7
   const int cp0 = (int)chunk * Cw;
   // The compute side is walked layer by layer (all heads of a layer, K rows then V rows, are
   // neighbours in memory), the LDS tile is indexed by column pair (head-major): entry j of the table
@@ -287,8 +289,9 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
   const uint64_t tm_row_bytes = (uint64_t)C * ES;
   const int n_tm = D * vpr;                // vectors on the token-major side
   const int n_cp = Cw * dgs;               // (pair, 16/ES values of d) items on the compute side
-  // Unit (pair cp, d) sits in group (d / (UPV)) ^ s of row cp, s = (cp / UPV) & 7 = the index of the
-  // token-major vector the pair belongs to, mod 8.
+  // Unit (pair cp, d) sits in group (d / UPV) ^ s of row cp, s = (cp / UPV) & sm = the index of the
+  // token-major vector the pair belongs to, mod 8 (mod a smaller power of two when the row has fewer
+  // aligned groups, e.g. head_dim 80 at 2 bytes: 20 groups, mod 4).
 
   if (DIR == 1) {
     // token-major rows -> LDS, the units of a vector to as many pair rows
@@ -311,7 +314,7 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
         if (w.outer < D) {
           const int cv = w.inner, d = w.outer;
           // unit index inside row (cv*UPV + j): group (d/UPV ^ s) * UPV + d % UPV
-          Unit* row = lds_unit + (cv * UPV) * D + ((((d >> UPV_SHIFT) ^ (cv & 7)) << UPV_SHIFT) | (d & (UPV - 1)));
+          Unit* row = lds_unit + (cv * UPV) * D + ((((d >> UPV_SHIFT) ^ (cv & sm)) << UPV_SHIFT) | (d & (UPV - 1)));
           Unit e[UPV];
           __builtin_memcpy(e, &x[u], 16);
 #pragma unroll
@@ -328,7 +331,7 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
       if (o.outer < Cw) {
         const uint64_t entry = row_addr[o.outer];
         const int cp = (int)(entry >> 48), dg = o.inner;
-        const int s = (cp >> UPV_SHIFT) & 7;
+        const int s = (cp >> UPV_SHIFT) & sm;
         const int flip = (dg >> 2) & 1;                        // lanes 0-3 and 4-7 start on different halves
         const u32x4 lo = lds_vec[cp * gpr + ((2 * dg + flip) ^ s)];
         const u32x4 hi = lds_vec[cp * gpr + ((2 * dg + 1 - flip) ^ s)];
@@ -362,7 +365,7 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
       for (int u = 0; u < U; ++u) {
         if (o.outer < Cw) {
           const int cp = (int)(row_addr[o.outer] >> 48), dg = o.inner;
-          const int s = (cp >> UPV_SHIFT) & 7;
+          const int s = (cp >> UPV_SHIFT) & sm;
           u32x4 g0, g1;
           join_kv<ES>(kx[u], vx[u], g0, g1);
           lds_vec[cp * gpr + ((2 * dg) ^ s)] = g0;
@@ -377,7 +380,7 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
     for (int base = 0; base < n_tm; base += B) {
       if (w.outer < D) {
         const int cv = w.inner, d = w.outer;
-        const Unit* row = lds_unit + (cv * UPV) * D + ((((d >> UPV_SHIFT) ^ (cv & 7)) << UPV_SHIFT) | (d & (UPV - 1)));
+        const Unit* row = lds_unit + (cv * UPV) * D + ((((d >> UPV_SHIFT) ^ (cv & sm)) << UPV_SHIFT) | (d & (UPV - 1)));
         Unit e[UPV];
 #pragma unroll
         for (int j = 0; j < UPV; ++j) e[j] = row[j * D];
@@ -417,7 +420,7 @@ hipError_t launch_transpose_pages(int dir, TransposeArgs& a, hipStream_t stream)
   // compute rows (Dd = head_dim) and the widest column chunk that fits LDS. Cutting head_dim to make
   // room for wider chunks lost 10-25 %, a 16 KiB tile lost 30-60 %, so the default is the full
   // head_dim with a ~60 KiB tile (two workgroups per CU).
-  if ((D * ES) % 64 == 0 && tuning().transpose_pairs != 0 && tuning().transpose_dsplit <= 1) {
+  if (tuning().transpose_pairs != 0 && tuning().transpose_dsplit <= 1) {
     // the pair kernel: unpadded tile [Cc/2 pairs][D] units, the widest column chunk that fits
     const int64_t budget = (int64_t)tuning().transpose_lds_kib * 1024;
     int best = 0;
@@ -428,6 +431,9 @@ hipError_t launch_transpose_pages(int dir, TransposeArgs& a, hipStream_t stream)
       a.n_dchunks = 1;
       a.chunk_cols = best;
       a.pitch = 0;
+      const int gpr = D * ES / 8;               // 16-byte groups per LDS row
+      int low = gpr & -gpr;
+      a.swz_mask = (low > 8 ? 8 : low) - 1;
       a.n_chunks = (uint32_t)(C / best);
       a.tile_words = (uint32_t)((int64_t)D * best * ES / 4);
       const size_t lds = (size_t)a.tile_words * 4 + (size_t)(best / 2) * 8;

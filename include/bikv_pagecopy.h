@@ -71,8 +71,7 @@ int bikv_check_status(int device, void* stream, uint32_t* bits_out);
  * many bytes use one lane per 16-byte piece instead of one wave per KiB), "run_group" (1 = several
  * short runs share a row of the launch grid, default; 0 = one row per run), "transpose_lds_kib" and
  * "transpose_dsplit" (LDS tile budget and head_dim slices of the layout-change kernel),
- * "transpose_pairs" (head_dim * elem_bytes % 64 == 0: 1 = the K/V-pair kernel, default;
- * 0 = the element-wise kernel) and "transpose_block" (its lanes per workgroup: 128, 256, 512, 1024).
+ * "transpose_pairs" (1 = the K/V-pair kernel, default; 0 = the element-wise kernel) and "transpose_block" (its lanes per workgroup: 128, 256, 512, 1024).
  * Process-wide. */
 int bikv_set_tuning(const char* key, int64_t value);
 
