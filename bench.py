@@ -12,13 +12,18 @@ shared between requests. One step = one gather launch + one scatter launch over 
 Inputs (pool, staging, index arrays) are resident in HBM before the timed region starts.
 
 Prints ONE JSON line. `value` = algorithmic bytes (payload read + payload written) per second over
-the timed steps; `roofline` prices the slower of the two kernels against 8 TB/s with the launch
-durations measured here with HIP events on the launch stream; `cpu_baseline` times the reference's
-CPU path (torch.index_select / index_copy_ on host tensors) on this box's cores on a bounded sample
-of the same request stream.
+the timed steps (400 by default: about two seconds of back-to-back launches); `roofline` prices the
+slower of the two kernels against 8 TB/s with the launch durations measured here with HIP events on
+the launch stream (min / median / p99 per launch are in `kernels`); `cpu_baseline` times the
+reference's CPU path (torch.index_select / index_copy_ on host tensors) on this box's cores on a
+bounded sample of the same request stream.
 
-`llama3_8b` additionally runs the per-request gather -> pinned-host staging pipeline and reports
-host-link GB/s next to a plain hipMemcpyAsync of one large pinned buffer measured in the same run.
+The default run then measures, one after another at full pool size, the other named configurations
+(`configs`: Qwen2-1.5B, Llama-3-8B, Llama-3-70B fp8 + scales) and, on the Llama-3-8B pool, the
+pool <-> pinned-host staging pipeline (`staging`): all 128 requests enqueued back to back, 4-32 MiB
+chunks on 2 and 4 lanes, kernel-direct and automatic modes, both directions, each next to a plain
+hipMemcpyAsync of one large pinned buffer timed immediately before it. `--no-configs` / `--no-staging`
+skip those parts.
 """
 import argparse
 import json
@@ -42,8 +47,8 @@ MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9949, "scatter": 1.0003},
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="qwen2_7b")
     ap.add_argument("--layout", default="layer_major", choices=["layer_major", "page_major"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -52,6 +57,12 @@ def parse_args():
     ap.add_argument("--pool-pages", type=int, default=0, help="override the pool size (pages per plane)")
     ap.add_argument("--pool-alloc", choices=["planes", "stacked"], default="stacked",
                     help="one device tensor per (layer, K|V) plane, or one stacked allocation")
+    ap.add_argument("--no-configs", dest="no_configs", action="store_true",
+                    help="skip the other named configurations (default workload only)")
+    ap.add_argument("--no-staging", dest="no_staging", action="store_true",
+                    help="skip the pinned-host staging record (default workload only)")
+    ap.add_argument("--staging-passes", dest="staging_passes", type=int, default=3)
+    ap.add_argument("--staging-requests", dest="staging_requests", type=int, default=128)
     ap.add_argument("--seg", type=int, default=None)
     ap.add_argument("--unroll", type=int, default=None)
     ap.add_argument("--nontemporal", type=int, default=None)
@@ -60,8 +71,9 @@ def parse_args():
     ap.add_argument("--log2-chunk", dest="log2_chunk", type=int, default=None)
     ap.add_argument("--staging-cap-gb", dest="staging_cap_gb", type=float, default=32.0,
                     help="largest staging buffer of one launch; bigger batches take several launches")
-    ap.add_argument("--chunk-mib", type=int, default=32, help="staging pipeline chunk (llama3_8b)")
-    ap.add_argument("--buffers", type=int, default=2, help="staging pipeline lanes (stream + HBM chunk each)")
+    ap.add_argument("--chunk-mib", type=int, default=0, help="staging: measure only this chunk size (0 = the sweep)")
+    ap.add_argument("--buffers", type=int, default=2, help="staging pipeline lanes with --chunk-mib")
+    ap.add_argument("--per-launch", dest="per_launch", type=int, default=4, help="host copies per kernel launch with --chunk-mib")
     return ap.parse_args()
 
 
@@ -97,22 +109,37 @@ def make_pool(shape, dev, alloc="planes"):
     return one(shape.tile_bytes), (one(shape.scale_tile_bytes) if shape.scales else None)
 
 
-def verify_on_device(pool_t, staging, batch, requests, n_check_planes=3):
-    """Independent check at full size: torch.index_select on the device, a few planes per request."""
+def verify_on_device(pool_t, staging, batch, requests, n_full=2):
+    """Independent check at full size: torch.index_select on the device. EVERY plane of the first
+    `n_full` non-empty requests and of the last one, three planes (first, middle, last) of all others.
+    Returns (ok, plane-request pairs checked, plane-request pairs in the batch)."""
     import torch
     n_planes = len(pool_t)
-    planes = sorted({0, n_planes // 2, n_planes - 1})[:n_check_planes]
-    for r, ids in enumerate(requests):
-        if len(ids) == 0:
-            continue
+    some = sorted({0, n_planes // 2, n_planes - 1})
+    nonempty = [r for r, ids in enumerate(requests) if len(ids)]
+    full = set(nonempty[:n_full] + nonempty[-1:])
+    checked = 0
+    for r in nonempty:
         view = batch.request_view(staging, r)
-        idt = torch.from_numpy(ids).to(pool_t[0].device)
-        for q in planes:
+        idt = torch.from_numpy(requests[r]).to(pool_t[0].device)
+        for q in (range(n_planes) if r in full else some):
             want = torch.index_select(pool_t[q], 0, idt)
             got = view[q] if batch.layout == "layer_major" else view[:, q]
             if not torch.equal(got, want):
-                return False
-    return True
+                return False, checked, len(nonempty) * n_planes
+            checked += 1
+    return True, checked, len(nonempty) * n_planes
+
+
+def launch_stats(ms, alg_bytes):
+    """min / median / p99 / mean of a kernel's launch durations (HIP events around each launch)."""
+    import numpy as np
+    a = np.sort(np.asarray(ms, dtype=np.float64))
+    mean = float(a.mean())
+    return {"GBps": round(alg_bytes / (mean * 1e-3) / 1e9, 1), "avg_ms": round(mean, 4),
+            "min_ms": round(float(a[0]), 4), "median_ms": round(float(np.median(a)), 4),
+            "p99_ms": round(float(a[min(len(a) - 1, int(np.ceil(0.99 * len(a))) - 1)]), 4),
+            "max_ms": round(float(a[-1]), 4), "launches_timed": int(len(a)), "alg_bytes": int(alg_bytes)}
 
 
 def time_plain_copy(bk, dev, nbytes=2 << 30, iters=5):
@@ -203,16 +230,29 @@ def cpu_baseline(shape, wl, budget_s=12.0):
     }
 
 
-def run_gather_scatter(args, bk, workloads, dev, with_copy=True):
+# Where the `traffic` figures come from: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, kept as
+# summaries under profiles/. They are NOT measured by the run that prints them (counters need the
+# profiler); a run only multiplies its own algorithmic bytes by the ratio recorded there.
+TRAFFIC_SOURCE = "profiles/*_pmc.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this command; not measured in this run)"
+
+
+def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layout=None, steps=None,
+                       warmup=None, target_s=None, keep_pool=False):
+    """One named configuration at full size: pool resident in HBM, one launch per direction (more when the
+    staging image would exceed --staging-cap-gb), `steps` timed steps (or as many as fill `target_s`
+    seconds). Returns (json fragment, shape, workload, kept) — kept = (pool_t, pool) when keep_pool."""
     import numpy as np
     import torch
 
-    name = args.workload
+    name = name or args.workload
+    layout = layout or args.layout
+    steps = steps or args.steps
+    warmup = args.warmup if warmup is None else warmup
     shape = workloads.SHAPES[name]
     if args.pool_pages:
         shape = shape.scaled(args.pool_pages)
     wl = workloads.named(name, shape)
-    log(f"{name}: pool {shape.pool_bytes / 1e9:.2f} GB, tile {shape.tile_bytes} B x {shape.n_planes} planes")
+    log(f"{name}: pool {shape.pool_bytes / 1e9:.2f} GB, tile {shape.tile_bytes} B x {shape.n_planes} planes, layout {layout}")
     pool_t, scale_t = make_pool(shape, dev, args.pool_alloc)
     pool = bk.PagedKVPool.from_planes(pool_t, scale_t)
 
@@ -221,7 +261,7 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True):
 
     # A launch covers as many whole requests as fit a staging buffer of --staging-cap-gb; the
     # Qwen2-7B-shaped batch fits in one launch per direction, the 70B-shaped one needs a few.
-    def groups_of(reqs):
+    def groups_of(reqs, unique=False):
         cap_pages = max(1, int(args.staging_cap_gb * 1e9) // shape.page_bytes)
         out, cur, used = [], [], 0
         for r in reqs:
@@ -232,9 +272,9 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True):
             used += len(r)
         if cur:
             out.append(cur)
-        return [(pool.make_batch(g, args.layout), g) for g in out]
+        return [(pool.make_batch(g, layout, check_unique=unique), g) for g in out]
 
-    g_groups, s_groups = groups_of(g_reqs), groups_of(s_reqs)
+    g_groups, s_groups = groups_of(g_reqs), groups_of(s_reqs, unique=True)
     max_slots = max(b.n_slots for b, _ in g_groups + s_groups)
     g_st = torch.empty(max_slots * shape.tile_bytes, dtype=torch.uint8, device=dev)
     g_sc = torch.empty(max_slots * shape.scale_tile_bytes, dtype=torch.uint8, device=dev) if shape.scales else None
@@ -271,93 +311,124 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True):
         if events is not None:
             events[2].record()
 
-    for _ in range(args.warmup):
-        step()
-    pool.check()
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
     torch.cuda.synchronize(dev)
     t0 = time.perf_counter()
-    for k in range(args.steps):
+    for _ in range(max(1, warmup)):
+        step()
+    pool.check()
+    warm_step_s = (time.perf_counter() - t0) / max(1, warmup)
+    if target_s:
+        steps = int(min(4000, max(5, np.ceil(target_s / max(warm_step_s, 1e-5)))))
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    for k in range(steps):
         step(evs[k])
     torch.cuda.synchronize(dev)
     wall = time.perf_counter() - t0
     pool.check()
 
-    # per-launch averages (a direction's launches are back to back between two events)
+    # per-launch durations (a direction's launches are back to back between two events)
     g_ms = [e[0].elapsed_time(e[1]) / len(g_groups) for e in evs]
     s_ms = [e[1].elapsed_time(e[2]) / max(1, len(s_groups)) for e in evs]
-    ms_per_step = wall * 1e3 / args.steps
-    value = (alg_g + alg_s) / (wall / args.steps) / 1e9
-    g_gbps = alg_g / len(g_groups) / (np.mean(g_ms) * 1e-3) / 1e9
-    s_gbps = alg_s / len(s_groups) / (np.mean(s_ms) * 1e-3) / 1e9 if s_groups else None
-    sb = s_groups or None
+    ms_per_step = wall * 1e3 / steps
+    value = (alg_g + alg_s) / (wall / steps) / 1e9
 
     # parity at full size, outside the timed region: scattered pages must equal their source, and
-    # each gather launch is repeated and checked against torch.index_select on the device
-    ok = True
-    for b, reqs in s_groups:
-        st, sc = views(b, s_st, s_sc)
-        ok = ok and verify_on_device(pool_t, st, b, reqs)
-        if scale_t is not None:
-            ok = ok and verify_on_device(scale_t, sc, b, reqs)
-    for b, reqs in g_groups:
-        st, sc = views(b, g_st, g_sc)
-        st.zero_()
-        pool.gather(b, st, sc)
-        pool.check()
-        ok = ok and verify_on_device(pool_t, st, b, reqs)
-        if scale_t is not None:
-            ok = ok and verify_on_device(scale_t, sc, b, reqs)
+    # each gather launch is repeated into a cleared buffer and checked against torch.index_select
+    ok, checked, total = True, 0, 0
+    for grp, st_all, sc_all, regather in ((s_groups, s_st, s_sc, False), (g_groups, g_st, g_sc, True)):
+        for b, reqs in grp:
+            st, sc = views(b, st_all, sc_all)
+            if regather:
+                st.zero_()
+                pool.gather(b, st, sc)
+                pool.check()
+            for tensors, image in ((pool_t, st), (scale_t, sc)):
+                if tensors is None:
+                    continue
+                o, c, t = verify_on_device(tensors, image, b, reqs)
+                ok, checked, total = ok and o, checked + c, total + t
     if not ok:
         raise SystemExit("bench: results differ from torch.index_select on the device — not reporting")
     alg_g //= len(g_groups)          # per launch, for the roofline entries below
     alg_s //= max(1, len(s_groups))
+    g_stat = launch_stats(g_ms, alg_g)
+    s_stat = launch_stats(s_ms, alg_s) if s_groups else None
 
     copy_gbps, copy_ok = time_plain_copy(bk, dev) if with_copy else (0.0, True)
     if not copy_ok:
         raise SystemExit("bench: plain copy mismatch")
 
     # the dominant kernel = the instantiation that takes more of the step
-    dominant_is_gather = (s_gbps is None) or (float(np.sum(g_ms)) >= float(np.sum(s_ms)))
+    dominant_is_gather = (s_stat is None) or (float(np.sum(g_ms)) >= float(np.sum(s_ms)))
     kname = "bikv::tile_move_wave_kernel<0=gather>" if dominant_is_gather else "bikv::tile_move_wave_kernel<1=scatter>"
-    ach = g_gbps if dominant_is_gather else s_gbps
-    alg_dom = alg_g if dominant_is_gather else alg_s
-    ms_dom = float(np.mean(g_ms if dominant_is_gather else s_ms))
+    dom = g_stat if dominant_is_gather else s_stat
     ratio = MEASURED_TRAFFIC_RATIO.get(name, {}).get("gather" if dominant_is_gather else "scatter")
-    if args.pool_pages or args.layout != "layer_major":
-        ratio = None                                   # measured on the full-size default workload only
+    if args.pool_pages or layout != "layer_major":
+        ratio = None                                   # measured on the full-size layer-major workload only
     out = {
         "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": f"{name}: {shape.layers} layers x K/V, {shape.n_pages} pages x {shape.page_tokens} tok x "
                                f"{shape.kv_heads} heads x {shape.head_dim} {shape.dtype}"
                                f"{' + fp32 scales' if shape.scales else ''}; {len(g_reqs)} gather + {len(s_reqs)} "
                                f"scatter requests, {n_pages} pages/step in {len(g_groups)}+{len(s_groups)} launches, "
-                               f"layout {args.layout}",
+                               f"layout {layout}",
                    "pool_GB": round(shape.pool_bytes / 1e9, 2), "tile_bytes": shape.tile_bytes,
                    "planes": shape.n_planes, "pool_alloc": args.pool_alloc},
+        "timed_region_s": round(wall, 3),
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
-        "pages_per_s": round(n_pages / (wall / args.steps), 1),
+        "pages_per_s": round(n_pages / (wall / steps), 1),
         "bit_exact": True,
-        "roofline": {"bound": "hbm", "kernel": kname, "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4),
-                     "traffic": (round(ratio * alg_dom) if ratio else None),
-                     "alg_bytes_per_launch": alg_dom, "avg_launch_ms": round(ms_dom, 4)},
-        "kernels": {"gather": {"GBps": round(g_gbps, 1), "avg_ms": round(float(np.mean(g_ms)), 4),
-                               "min_ms": round(float(np.min(g_ms)), 4), "alg_bytes": alg_g},
-                    "scatter": ({"GBps": round(s_gbps, 1), "avg_ms": round(float(np.mean(s_ms)), 4),
-                                 "min_ms": round(float(np.min(s_ms)), 4), "alg_bytes": alg_s} if sb else None),
+        "bit_exact_coverage": f"torch.index_select on the device over {checked} of {total} (request, plane) images: every "
+                              "plane of the first two and the last request of each launch, first/middle/last plane of the rest",
+        "roofline": {"bound": "hbm", "kernel": kname, "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
+                     "traffic": (round(ratio * dom["alg_bytes"]) if ratio else None),
+                     "traffic_source": TRAFFIC_SOURCE if ratio else None,
+                     "alg_bytes_per_launch": dom["alg_bytes"], "avg_launch_ms": dom["avg_ms"]},
+        "kernels": {"gather": g_stat, "scatter": s_stat,
                     "plain_copy_2GiB": ({"GBps": round(copy_gbps, 1)} if with_copy else None)},
     }
-    del pool_t, scale_t, g_st, s_st
+    kept = None
+    if keep_pool:
+        kept = (pool_t, pool)
+    del g_st, s_st, g_sc, s_sc
+    if not keep_pool:
+        pool.close()
+        del pool_t, scale_t
     torch.cuda.empty_cache()
-    return out, shape, wl
+    return out, shape, wl, kept
 
 
-def run_staging(args, bk, workloads, dev):
-    """llama3_8b: per-request gather followed by the device -> pinned-host copy, overlapped in chunks."""
+def config_summary(o):
+    """The part of a configuration's measurement that goes into the default line's `configs` record."""
+    k = o["kernels"]
+    frac = lambda st: round(st["GBps"] / HBM_PEAK_GBPS, 4) if st else None
+    return {"workload": o["config"]["workload"], "pool_GB": o["config"]["pool_GB"], "value": o["value"], "unit": "GB/s",
+            "pct_of_hbm_peak": o["pct_of_hbm_peak"], "pages_per_s": o["pages_per_s"], "steps": o["steps"],
+            "timed_region_s": o["timed_region_s"], "bit_exact": o["bit_exact"],
+            "gather": dict(k["gather"], frac=frac(k["gather"])),
+            "scatter": (dict(k["scatter"], frac=frac(k["scatter"])) if k["scatter"] else None),
+            "traffic": o["roofline"]["traffic"]}
+
+
+def link_yardstick(bk, dev, host, dev_buf, reps=3):
+    """Plain hipMemcpyAsync of one large pinned buffer, both directions: best of `reps`, GB/s."""
+    n = min(host.numel(), dev_buf.numel())
+    d2h = max(n / bk.measure_d2h(dev, host, dev_buf, 0) / 1e9 for _ in range(reps))
+    h2d = max(n / bk.measure_h2d(dev, dev_buf, host, 0) / 1e9 for _ in range(reps))
+    return d2h, h2d
+
+
+def run_staging(args, bk, workloads, dev, kept=None):
+    """Llama-3-8B shape: every request of the log-normal stream gathered into pinned host memory, and
+    scattered back from it, through the staging pipeline. All requests of a pass are enqueued back to back
+    (one wait at the end); a cell is min / median over the passes, next to a plain hipMemcpyAsync of one
+    1 GiB pinned buffer timed immediately before the cell (the host-link yardstick)."""
     import numpy as np
     import torch
 
@@ -365,80 +436,133 @@ def run_staging(args, bk, workloads, dev):
     if args.pool_pages:
         shape = shape.scaled(args.pool_pages)
     wl = workloads.named("llama3_8b", shape)
-    pool_t, _ = make_pool(shape, dev, args.pool_alloc)
-    pool = bk.PagedKVPool.from_planes(pool_t)
-    reqs = wl["gather"]
-    max_pages = max(len(r) for r in reqs)
-    host = bk.pinned_empty(max_pages * shape.page_bytes)
-    host.zero_()
-    # host-link yardstick: one large pinned buffer, plain hipMemcpyAsync
-    dev_buf = torch.empty(min(host.numel(), 1 << 30), dtype=torch.uint8, device=dev)
+    if kept is None:
+        pool_t, _ = make_pool(shape, dev, args.pool_alloc)
+        pool = bk.PagedKVPool.from_planes(pool_t)
+    else:
+        pool_t, pool = kept
+    reqs = wl["gather"][: max(1, args.staging_requests)]
+    layout = "layer_major"
+    sizes = np.array([len(r) * shape.page_bytes for r in reqs], dtype=np.int64)
+    region = int(max(4 << 30, 2 * sizes.max()))
+    host = bk.pinned_empty(region)
+    dev_buf = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
     dev_buf.random_(0, 256)
-    # the first DMA into a pinned page is slower than later ones: touch the whole buffer once
-    for off in range(0, host.numel(), dev_buf.numel()):
-        n = min(dev_buf.numel(), host.numel() - off)
+    # the first DMA into a pinned page is slower than later ones: touch the whole region once
+    for off in range(0, region, dev_buf.numel()):
+        n = min(dev_buf.numel(), region - off)
         host[off: off + n].copy_(dev_buf[:n])
-    link = []
-    for _ in range(4):
-        link.append(dev_buf.numel() / bk.measure_d2h(dev, host, dev_buf, 0) / 1e9)
-    link_gbps = max(link[1:])
-    up = []
-    for _ in range(4):
-        up.append(dev_buf.numel() / bk.measure_h2d(dev, dev_buf, host, 0) / 1e9)
-    up_gbps = max(up[1:])
-    results = {}
-    for mode in ("pipelined", "direct"):
-        stager = bk.HostStager(dev, chunk_bytes=args.chunk_mib << 20, n_buffers=args.buffers)
-        batches = [pool.make_batch([r], args.layout) for r in reqs]
-        torch.cuda.synchronize(dev)
-        stager.gather_to_host(pool, batches[0], host, mode)      # warm-up
-        tot_b, tot_s, chunks = 0, 0.0, 0
-        for b in batches[: max(1, args.steps)]:
-            nb, nc, sec = stager.gather_to_host(pool, b, host, mode)
-            tot_b += nb
-            tot_s += sec
-            chunks += nc
-        # parity of the last request staged
-        b = batches[max(1, args.steps) - 1 if args.steps <= len(batches) else -1]
-        stager.gather_to_host(pool, b, host, mode)
-        r = reqs[batches.index(b)]
-        idt = torch.from_numpy(r).to(dev)
-        view = host[: b.n_slots * shape.tile_bytes].view(b.n_slots, shape.tile_bytes)
-        ok = True
-        for q in (0, shape.n_planes - 1):
-            want = torch.index_select(pool_t[q], 0, idt).cpu()
-            got = view[q * len(r): (q + 1) * len(r)] if args.layout == "layer_major" else view[q::shape.n_planes]
-            ok = ok and torch.equal(got, want)
-        if not ok:
-            raise SystemExit(f"bench: staged bytes differ ({mode})")
-        results[mode] = {"host_link_GBps": round(tot_b / tot_s / 1e9, 2), "bytes": tot_b, "chunks": chunks,
-                         "frac_of_plain_d2h": round(tot_b / tot_s / 1e9 / link_gbps, 4)}
-        # the receiving side: the staged image of a request goes host -> pool, into the pages next to
-        # the ones it came from (a different, still unique id set)
-        rx_b, rx_s = 0, 0.0
-        rx = [(b_, r_) for b_, r_ in zip(batches, reqs) if len(np.unique(r_)) == len(r_)][: max(1, args.steps)]
-        for b_, r_ in rx:
-            stager.gather_to_host(pool, b_, host, mode)
-            shifted = (np.asarray(r_) + 1) % shape.n_pages
-            sb = pool.make_batch([shifted], args.layout)
-            nb, _, sec = stager.scatter_from_host(pool, sb, host, mode)
-            rx_b += nb
-            rx_s += sec
-        if rx:
-            idt = torch.from_numpy(shifted).to(dev)
-            view = host[: sb.n_slots * shape.tile_bytes].view(sb.n_slots, shape.tile_bytes)
-            for q in (0, shape.n_planes - 1):
-                got = torch.index_select(pool_t[q], 0, idt).cpu()
-                want = (view[q * len(shifted): (q + 1) * len(shifted)] if args.layout == "layer_major"
-                        else view[q::shape.n_planes])
-                if not torch.equal(got, want):
-                    raise SystemExit(f"bench: scattered bytes differ ({mode})")
-            results[mode]["scatter_from_host_GBps"] = round(rx_b / rx_s / 1e9, 2)
-            results[mode]["scatter_frac_of_plain_h2d"] = round(rx_b / rx_s / 1e9 / up_gbps, 4)
+    # every request gets a window of the pinned region; windows rotate through it, so requests in flight
+    # together (neighbours in issue order) never share host bytes
+    offs, cur = [], 0
+    for sz in sizes:
+        if cur + sz > region:
+            cur = 0
+        offs.append(cur)
+        cur += int(sz)
+    g_batches = [pool.make_batch([r], layout) for r in reqs]
+    # the way back: each image into the pages next to the ones it came from (unique within a request)
+    s_batches = [pool.make_batch([(np.asarray(r) + 1) % shape.n_pages], layout, check_unique=True) for r in reqs]
+    torch.cuda.synchronize(dev)
+    total_bytes = int(sizes.sum())
+    passes = max(1, args.staging_passes)
+    yard = {"d2h": [], "h2d": []}
+
+    def cell(stager, mode, direction, synchronous=False):
+        d2h, h2d = link_yardstick(bk, dev, host[: dev_buf.numel()], dev_buf)
+        yard["d2h"].append(d2h)
+        yard["h2d"].append(h2d)
+        link = d2h if direction == "gather" else h2d
+        batches = g_batches if direction == "gather" else s_batches
+        rates = []
+        for p in range(passes + 1):                      # the first pass is a warm-up
+            t0 = time.perf_counter()
+            for b, off, sz in zip(batches, offs, sizes):
+                win = host[off: off + int(sz)]
+                if synchronous:
+                    (stager.gather_to_host if direction == "gather" else stager.scatter_from_host)(pool, b, win, mode)
+                else:
+                    (stager.gather_to_host_async if direction == "gather" else stager.scatter_from_host_async)(pool, b, win, mode)
+            if not synchronous:
+                stager.wait()
+            if p:
+                rates.append(total_bytes / (time.perf_counter() - t0) / 1e9)
+        return {"GBps_min": round(min(rates), 2), "GBps_median": round(float(np.median(rates)), 2),
+                "plain_GBps_just_before": round(link, 2),
+                "frac_min": round(min(rates) / link, 4), "frac_median": round(float(np.median(rates)) / link, 4)}
+
+    def verify(stager, mode):
+        """Three requests (smallest, median, largest below 1 GiB) staged synchronously and compared, every
+        plane, with torch.index_select on the device; then scattered back and read from the pool."""
+        order = np.argsort(sizes)
+        small = [i for i in order if sizes[i] <= (1 << 30)]
+        for i in {int(order[0]), int(order[len(order) // 2]), int(small[-1])}:
+            r, b, sz = reqs[i], g_batches[i], int(sizes[i])
+            win = host[:sz]
+            win.zero_()
+            stager.gather_to_host(pool, b, win, mode)
+            idt = torch.from_numpy(np.asarray(r)).to(dev)
+            view = win.view(shape.n_planes, len(r), shape.tile_bytes)
+            for q in range(shape.n_planes):
+                if not torch.equal(view[q], torch.index_select(pool_t[q], 0, idt).cpu()):
+                    raise SystemExit(f"bench: staged bytes differ ({mode}, request {i}, plane {q})")
+            stager.scatter_from_host(pool, s_batches[i], win, mode)
+            idt2 = (idt + 1) % shape.n_pages
+            for q in (0, shape.n_planes // 2, shape.n_planes - 1):
+                if not torch.equal(torch.index_select(pool_t[q], 0, idt2).cpu(), view[q]):
+                    raise SystemExit(f"bench: scattered bytes differ ({mode}, request {i}, plane {q})")
+
+    if args.chunk_mib:
+        grid = [(args.chunk_mib, args.buffers, args.per_launch)]
+    else:
+        # (chunk MiB, lanes, host copies per kernel launch); the last row is the contrast case: one kernel
+        # per small copy, the shape that made small chunks slow and erratic
+        grid = [(4, 2, 4), (8, 2, 4), (16, 2, 2), (32, 2, 1), (4, 4, 4), (8, 4, 2), (16, 4, 1), (32, 4, 1), (4, 4, 1)]
+    cells = []
+    for chunk, lanes, group in grid:
+        stager = bk.HostStager(dev, chunk_bytes=chunk << 20, n_buffers=lanes, chunks_per_launch=group)
+        if (chunk, lanes, group) == grid[0]:
+            verify(stager, "pipelined")
+        row = {"mode": "pipelined", "chunk_MiB": chunk, "lanes": lanes, "copies_per_launch": group}
+        for direction in ("gather", "scatter"):
+            row[direction + "_to_host" if direction == "gather" else "scatter_from_host"] = cell(stager, "pipelined", direction)
+        log(f"staging {row}")
+        cells.append(row)
         stager.close()
-    return {"plain_d2h_GBps": round(link_gbps, 2), "plain_h2d_GBps": round(up_gbps, 2),
-            "chunk_MiB": args.chunk_mib, "buffers": args.buffers,
-            "requests": min(len(reqs), max(1, args.steps)), **results}
+    stager = bk.HostStager(dev)          # the library's defaults: 8 MiB x 4 per launch x 2 lanes
+    verify(stager, "direct")
+    for mode in ("direct", "auto"):
+        row = {"mode": mode, "chunk_MiB": stager.chunk_bytes >> 20, "lanes": stager.n_buffers,
+               "copies_per_launch": stager.chunks_per_launch}
+        row["gather_to_host"] = cell(stager, mode, "gather")
+        row["scatter_from_host"] = cell(stager, mode, "scatter")
+        log(f"staging {row}")
+        cells.append(row)
+    # what one blocking call per request (the reference's calling pattern, kvcache.py:219-225) costs
+    per_call = {"mode": "auto", "one_blocking_call_per_request": True,
+                "gather_to_host": cell(stager, "auto", "gather", synchronous=True),
+                "scatter_from_host": cell(stager, "auto", "scatter", synchronous=True)}
+    stager.close()
+    auto = cells[-1]
+    out = {"workload": f"llama3_8b: {shape.n_pages} pages x {shape.n_planes} planes x {shape.tile_bytes} B, "
+                       f"{len(reqs)} requests of {int(sizes.min() // shape.page_bytes)}..{int(sizes.max() // shape.page_bytes)} "
+                       f"pages ({total_bytes / 1e9:.2f} GB per pass), enqueued back to back, {passes} timed passes per cell",
+           "pool_GB": round(shape.pool_bytes / 1e9, 2),
+           "plain_d2h_GBps": {"min": round(min(yard["d2h"]), 2), "median": round(float(np.median(yard["d2h"])), 2),
+                              "max": round(max(yard["d2h"]), 2), "samples": len(yard["d2h"])},
+           "plain_h2d_GBps": {"min": round(min(yard["h2d"]), 2), "median": round(float(np.median(yard["h2d"])), 2),
+                              "max": round(max(yard["h2d"]), 2), "samples": len(yard["h2d"])},
+           "host_link_GBps": auto["gather_to_host"]["GBps_median"],
+           "frac_of_plain_d2h": auto["gather_to_host"]["frac_median"],
+           "frac_of_best_plain_d2h_seen": round(auto["gather_to_host"]["GBps_median"] / max(yard["d2h"]), 4),
+           "scatter_from_host_GBps": auto["scatter_from_host"]["GBps_median"],
+           "scatter_frac_of_plain_h2d": auto["scatter_from_host"]["frac_median"],
+           "cells": cells, "per_request_blocking_calls": per_call, "bit_exact": True}
+    if kept is None:
+        pool.close()
+        del pool_t
+        torch.cuda.empty_cache()
+    return out
 
 
 def run_reference_scenario(args, bk, dev):
@@ -718,20 +842,36 @@ def main():
         out = run_layout_change(args, bk, dev)
         print(json.dumps(out), flush=True)
         return
-    out, shape, wl = run_gather_scatter(args, bk, workloads, dev)
+    if args.workload == "staging":
+        print(json.dumps({"metric": "pinned-host staging GB/s", "unit": "GB/s", "n_gpus": 1,
+                          "staging": run_staging(args, bk, workloads, dev)}), flush=True)
+        return
+    out, shape, wl, _ = run_gather_scatter(args, bk, workloads, dev)
     if knobs:
         out["config"]["tuning"] = knobs
     if not args.no_other_layout:
         # the same request stream with the other staging image (reported next to the headline number)
-        import copy
-        alt = copy.copy(args)
-        alt.layout = "page_major" if args.layout == "layer_major" else "layer_major"
-        alt.steps, alt.warmup = max(3, args.steps // 2), 2
-        log(f"same workload, staging layout {alt.layout}")
-        o2, _, _ = run_gather_scatter(alt, bk, workloads, dev, with_copy=False)
-        out["other_layout"] = {"layout": alt.layout, "value": o2["value"], "pct_of_hbm_peak": o2["pct_of_hbm_peak"],
-                               "steps": alt.steps, "kernels": {k: v for k, v in o2["kernels"].items() if v}}
-    if args.workload == "llama3_8b":
+        alt_layout = "page_major" if args.layout == "layer_major" else "layer_major"
+        log(f"same workload, staging layout {alt_layout}")
+        o2, _, _, _ = run_gather_scatter(args, bk, workloads, dev, with_copy=False, layout=alt_layout, target_s=0.6, warmup=3)
+        out["other_layout"] = {"layout": alt_layout, "value": o2["value"], "pct_of_hbm_peak": o2["pct_of_hbm_peak"],
+                               "steps": o2["steps"], "kernels": {k: v for k, v in o2["kernels"].items() if v}}
+    default_run = args.workload == "qwen2_7b" and not args.pool_pages
+    if default_run and not args.no_configs:
+        # the other named configurations, each at full size: allocated, measured for about a second, freed
+        out["configs"] = {}
+        for other in ("qwen2_1p5b", "llama3_8b", "llama3_70b_fp8"):
+            keep = other == "llama3_8b" and not args.no_staging
+            o, _, _, kept = run_gather_scatter(args, bk, workloads, dev, with_copy=False, name=other, target_s=1.0,
+                                               warmup=3, keep_pool=keep)
+            out["configs"][other] = config_summary(o)
+            if keep:
+                log("pinned-host staging on the Llama-3-8B pool")
+                out["staging"] = run_staging(args, bk, workloads, dev, kept)
+                kept[1].close()
+                del kept
+                torch.cuda.empty_cache()
+    elif args.workload == "llama3_8b" and not args.no_staging:
         out["staging"] = run_staging(args, bk, workloads, dev)
     if not args.no_cpu_baseline:
         log("timing the CPU baseline")

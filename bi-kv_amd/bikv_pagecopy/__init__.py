@@ -3,7 +3,7 @@
 Thin Python over libbikv_pagecopy.so (HIP, gfx950). PyTorch supplies device memory and streams only.
 """
 from . import _lib
-from ._lib import load, set_tuning
+from ._lib import load, require_unique, reset_tuning, set_tuning
 from .nhd import NHDPool
 from .offsets import RunIndexPool, build_run_offsets
 from .pool import LAYER_MAJOR, PAGE_MAJOR, PageBatch, PagedKVPool, build_index
@@ -11,6 +11,6 @@ from .runs import copy_runs
 from .staging import HostStager, measure_d2h, measure_h2d, pinned_empty, plan_chunks
 
 __all__ = [
-    "load", "set_tuning", "build_run_offsets", "RunIndexPool", "LAYER_MAJOR", "PAGE_MAJOR", "PageBatch", "PagedKVPool",
+    "load", "set_tuning", "reset_tuning", "require_unique", "build_run_offsets", "RunIndexPool", "LAYER_MAJOR", "PAGE_MAJOR", "PageBatch", "PagedKVPool",
     "build_index", "copy_runs", "NHDPool", "HostStager", "measure_d2h", "measure_h2d", "pinned_empty", "plan_chunks",
 ]

@@ -13,13 +13,13 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libbikv_pagecopy.so")
 
 MAX_DIM = 5
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 OK, EINVAL, EHIP, ESYS, ESTATE, EBOUNDS, ERANGE = 0, -1, -2, -3, -4, -5, -6
 ST_SRC_RANGE, ST_DST_RANGE, ST_PAGE_ID = 1, 2, 4
 LAYOUT_LAYER_MAJOR, LAYOUT_PAGE_MAJOR = 0, 1
 HINT_NONE, HINT_LAYER_MAJOR, HINT_PAGE_MAJOR = 0, 1, 2
-STAGE_PIPELINED, STAGE_DIRECT = 0, 1
+STAGE_PIPELINED, STAGE_DIRECT, STAGE_AUTO = 0, 1, 2
 
 
 class PoolDesc(C.Structure):
@@ -108,6 +108,8 @@ _SIGNATURES = {
     "bikv_last_error": (C.c_char_p, []),
     "bikv_check_status": (C.c_int, [C.c_int, C.c_void_p, C.POINTER(C.c_uint32)]),
     "bikv_set_tuning": (C.c_int, [C.c_char_p, C.c_int64]),
+    "bikv_reset_tuning": (None, []),
+    "bikv_find_duplicate": (C.c_int, [C.POINTER(C.c_int64), C.c_int64, C.POINTER(C.c_int64)]),
     "bikv_copy_runs": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
                                  C.c_int64, C.c_int64, C.c_int64, C.c_void_p]),
     "bikv_copy_runs_ragged": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
@@ -121,7 +123,14 @@ _SIGNATURES = {
                                     C.c_void_p, C.c_int64, C.c_void_p]),
     "bikv_scatter_pages": (C.c_int, [C.c_void_p, C.POINTER(PageBatchDesc), C.c_void_p, C.c_int64,
                                      C.c_void_p, C.c_int64, C.c_void_p]),
-    "bikv_stager_create": (C.c_int, [C.c_int, C.c_int64, C.c_int32, C.POINTER(C.c_void_p)]),
+    "bikv_stager_create": (C.c_int, [C.c_int, C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_void_p)]),
+    "bikv_stager_wait": (C.c_int, [C.c_void_p, C.POINTER(StageStats)]),
+    "bikv_gather_to_host_async": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PageBatchDesc),
+                                            C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_void_p,
+                                            C.c_int64, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]),
+    "bikv_scatter_from_host_async": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PageBatchDesc),
+                                               C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_void_p,
+                                               C.c_int64, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]),
     "bikv_stager_destroy": (C.c_int, [C.c_void_p]),
     "bikv_gather_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PageBatchDesc),
                                       C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_void_p,
@@ -147,6 +156,7 @@ _SIGNATURES = {
     "bikv_producer_init": (C.c_int, [C.c_int, C.c_char_p]),
     "bikv_producer_reserve": (C.c_int, [C.c_size_t, C.POINTER(C.c_void_p)]),
     "bikv_producer_publish": (C.c_int, [C.POINTER(C.c_int64), C.c_size_t, C.c_int32, C.c_void_p]),
+    "bikv_producer_cancel": (C.c_int, []),
     "bikv_producer_set_backpressure": (C.c_int, [C.c_int, C.c_int64]),
     "bikv_consumer_release": (C.c_int, []),
     "bikv_producer_cleanup": (None, []),
@@ -207,3 +217,19 @@ def set_tuning(**kw):
     lib = load()
     for k, v in kw.items():
         check(lib.bikv_set_tuning(k.encode(), int(v)))
+
+
+def reset_tuning():
+    """Every launch knob back to its default."""
+    load().bikv_reset_tuning()
+
+
+def require_unique(ids, what="page id"):
+    """Raises RuntimeError naming the first repeated id of `ids` (any integer sequence or array on the
+    host). The destinations of a scatter must be unique: two runs of one launch that write the same
+    place race, as they do in the reference's kernel (copy_kernel.cu:29-35)."""
+    import numpy as np
+    arr = np.ascontiguousarray(np.asarray(ids, dtype=np.int64).reshape(-1))
+    rc = load().bikv_find_duplicate(arr.ctypes.data_as(C.POINTER(C.c_int64)), arr.size, None)
+    if rc < 0:
+        raise RuntimeError(f"{what}: {last_error()}")

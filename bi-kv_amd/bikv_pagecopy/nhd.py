@@ -81,10 +81,15 @@ class NHDPool:
                           tm_pages.data_ptr(), block_ids.numel(),
                           C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)))
 
-    def load_token_major(self, tm: torch.Tensor, block_ids: torch.Tensor, tm_pages: Optional[torch.Tensor] = None):
+    def load_token_major(self, tm: torch.Tensor, block_ids: torch.Tensor, tm_pages: Optional[torch.Tensor] = None,
+                         check_unique: bool = False):
         """Received token-major pages -> pool blocks (unique block ids). `tm` holds pages of
         block_tokens tokens, each token [dim][heads][layers][2]; page i of the call is tm page
-        tm_pages[i] (default: i). Asynchronous on the current stream."""
+        tm_pages[i] (default: i). Asynchronous on the current stream. `check_unique=True` copies the
+        block ids to the host first (a synchronising debug aid) and raises RuntimeError naming the first
+        block that is named twice."""
+        if check_unique:
+            _lib.require_unique(block_ids.cpu().numpy(), "load_token_major block ids")
         self._call(_lib.load().bikv_nhd_load_token_major, tm, block_ids, tm_pages)
 
     def store_token_major(self, tm: torch.Tensor, block_ids: torch.Tensor, tm_pages: Optional[torch.Tensor] = None):

@@ -210,11 +210,16 @@ class PagedKVPool:
         return cls(ptrs, t0.shape[0], tile, 2 * tile, t0.device, t0.dtype, keepalive=list(layers))
 
     # ---- batches ----------------------------------------------------------------------------
-    def make_batch(self, requests: Sequence[Sequence[int]], layout: str = LAYER_MAJOR, index_pool=None) -> PageBatch:
+    def make_batch(self, requests: Sequence[Sequence[int]], layout: str = LAYER_MAJOR, index_pool=None,
+                   check_unique: bool = False) -> PageBatch:
         """Builds and uploads the index arrays of a batch. With `index_pool` (offsets.RunIndexPool, 3 rows)
         they go into its persistent device buffers through its pinned mirror: no allocation, no upload
-        from pageable memory; the batch is then valid until the pool's next load()."""
+        from pageable memory; the batch is then valid until the pool's next load().
+        `check_unique=True` (for a batch that will be SCATTERED) raises RuntimeError naming the first page
+        id that appears twice: duplicate destinations are a data race on the device."""
         idx, req_pages = build_index(requests, self.n_planes, layout)
+        if check_unique:
+            _lib.require_unique(idx[0], "scatter batch")
         if index_pool is not None and idx.size:
             dev = index_pool.load(idx)
         else:

@@ -3,9 +3,10 @@
 The reference stages outgoing KV in host tensors allocated per call (Bi-KV/DistributedStorage/
 kvcache.py:105-108, Bi-KV/Worker/Worker.py:203-206) which the RDMA endpoint then sends from a
 pinned region (Bi-KV/NetworkTransport/onesided_rdma.h:301-337). HostStager fills such a pinned
-region straight from the paged pool: chunks are gathered into per-stream HBM buffers and copied out
+region straight from the paged pool: pieces are gathered into per-stream HBM buffers and copied out
 with hipMemcpyAsync, several streams in flight (mode "pipelined"), or the gather kernel stores
-directly into the mapped pinned buffer (mode "direct").
+directly into the mapped pinned buffer (mode "direct"). Each transfer also exists in an enqueue-only
+form, so that requests follow each other on the link without a drain in between.
 """
 import ctypes as C
 
@@ -15,7 +16,7 @@ import torch
 from . import _lib
 from .pool import PagedKVPool, PageBatch, _LAYOUT_CODE
 
-_MODES = {"pipelined": _lib.STAGE_PIPELINED, "direct": _lib.STAGE_DIRECT}
+_MODES = {"pipelined": _lib.STAGE_PIPELINED, "direct": _lib.STAGE_DIRECT, "auto": _lib.STAGE_AUTO}
 
 
 def pinned_empty(nbytes: int) -> torch.Tensor:
@@ -24,17 +25,25 @@ def pinned_empty(nbytes: int) -> torch.Tensor:
 
 
 class HostStager:
-    def __init__(self, device, chunk_bytes: int = 32 << 20, n_buffers: int = 2):
+    """`n_buffers` lanes (HIP stream + HBM buffer of `chunks_per_launch` x `chunk_bytes`). Mode "auto"
+    sends with the kernel storing straight into the pinned image ("direct") and receives through the
+    DMA engine ("pipelined"): on MI355X the device -> host DMA path runs at either ~30 or ~57 GB/s
+    depending on a platform state the library cannot see, kernel stores hold ~55 GB/s in both."""
+
+    def __init__(self, device, chunk_bytes: int = 8 << 20, n_buffers: int = 2, chunks_per_launch: int = 4):
         self.device = torch.device(device)
         self.chunk_bytes = int(chunk_bytes)
         self.n_buffers = int(n_buffers)
+        self.chunks_per_launch = int(chunks_per_launch)
         idx = self.device.index if self.device.index is not None else torch.cuda.current_device()
         self._device_index = idx
+        self._keep = []          # what in-flight asynchronous calls still read
         h = C.c_void_p()
-        _lib.check(_lib.load().bikv_stager_create(idx, self.chunk_bytes, self.n_buffers, C.byref(h)))
+        _lib.check(_lib.load().bikv_stager_create(idx, self.chunk_bytes, self.chunks_per_launch, self.n_buffers,
+                                                  C.byref(h)))
         self._h = h
 
-    def _stage(self, entry: str, pool: PagedKVPool, batch: PageBatch, host, mode, host_scale):
+    def _args(self, pool: PagedKVPool, batch: PageBatch, host, mode, host_scale):
         if mode not in _MODES:
             raise ValueError(f"unknown mode {mode!r}")
         for t in (host, host_scale):
@@ -46,35 +55,66 @@ class HostStager:
                 raise RuntimeError("host staging buffer must be contiguous")
         if pool.scale_tile_bytes and host_scale is None:
             raise RuntimeError("pool has scales: a pinned host_scale buffer is required")
+        d = batch.desc()
+        rp = batch.req_pages.ctypes.data_as(C.POINTER(C.c_int64))
+        return (self._h, pool._h, C.byref(d), rp, len(batch.req_pages), _LAYOUT_CODE[batch.layout],
+                host.data_ptr(), host.numel() * host.element_size(),
+                host_scale.data_ptr() if host_scale is not None else None,
+                host_scale.numel() * host_scale.element_size() if host_scale is not None else 0,
+                _MODES[mode]), d
+
+    def _stage(self, entry: str, pool, batch, host, mode, host_scale):
+        args, d = self._args(pool, batch, host, mode, host_scale)
         # work queued on the caller's stream (e.g. the upload of the index arrays) must be visible
         torch.cuda.current_stream(self.device).synchronize()
-        d = batch.desc()
         stats = _lib.StageStats()
-        rp = batch.req_pages.ctypes.data_as(C.POINTER(C.c_int64))
-        _lib.check(getattr(_lib.load(), entry)(
-            self._h, pool._h, C.byref(d), rp, len(batch.req_pages), _LAYOUT_CODE[batch.layout],
-            host.data_ptr(), host.numel() * host.element_size(),
-            host_scale.data_ptr() if host_scale is not None else None,
-            host_scale.numel() * host_scale.element_size() if host_scale is not None else 0,
-            _MODES[mode], C.byref(stats)))
+        _lib.check(getattr(_lib.load(), entry)(*args, C.byref(stats)))
+        self._keep.clear()
         return stats.bytes, stats.n_chunks, stats.wall_seconds
 
-    def gather_to_host(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "pipelined",
+    def _stage_async(self, entry: str, pool, batch, host, mode, host_scale):
+        args, d = self._args(pool, batch, host, mode, host_scale)
+        stream = C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        _lib.check(getattr(_lib.load(), entry)(*args, stream))
+        self._keep.append((pool, batch, host, host_scale))
+
+    def gather_to_host(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "auto",
                        host_scale: torch.Tensor = None):
         """Fills `host` (pinned) with the staging image of `batch` (and `host_scale` with the scale
-        image of an fp8 pool); returns (bytes, chunks, seconds)."""
+        image of an fp8 pool); returns (bytes, host copies, seconds)."""
         return self._stage("bikv_gather_to_host", pool, batch, host, mode, host_scale)
 
-    def scatter_from_host(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "pipelined",
+    def scatter_from_host(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "auto",
                           host_scale: torch.Tensor = None):
         """Writes the staging image held in `host` (pinned; `host_scale` for an fp8 pool) into the
-        pool pages `batch` names (unique ids); returns (bytes, chunks, seconds)."""
+        pool pages `batch` names (unique ids); returns (bytes, host copies, seconds)."""
         return self._stage("bikv_scatter_from_host", pool, batch, host, mode, host_scale)
+
+    def gather_to_host_async(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "auto",
+                             host_scale: torch.Tensor = None):
+        """Enqueues the transfer behind the current stream's work and returns; wait() completes it.
+        Host images of calls in flight together must not overlap."""
+        self._stage_async("bikv_gather_to_host_async", pool, batch, host, mode, host_scale)
+
+    def scatter_from_host_async(self, pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, mode: str = "auto",
+                                host_scale: torch.Tensor = None):
+        self._stage_async("bikv_scatter_from_host_async", pool, batch, host, mode, host_scale)
+
+    def wait(self):
+        """Drains the lanes; returns (bytes, host copies, seconds) of everything enqueued since the
+        previous wait and raises if a kernel skipped out-of-range work."""
+        stats = _lib.StageStats()
+        try:
+            _lib.check(_lib.load().bikv_stager_wait(self._h, C.byref(stats)))
+        finally:
+            self._keep.clear()
+        return stats.bytes, stats.n_chunks, stats.wall_seconds
 
     def close(self):
         if getattr(self, "_h", None):
             _lib.load().bikv_stager_destroy(self._h)
             self._h = None
+        self._keep = []
 
     def __del__(self):
         try:

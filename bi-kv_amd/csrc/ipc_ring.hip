@@ -52,6 +52,13 @@ struct Role {
 
 Role g_producer, g_consumer;
 
+// Rings of this many bytes or more are neither exported nor mapped across processes.
+constexpr size_t kMaxIpcBytes = size_t(2) << 30;
+
+// Between bikv_producer_reserve and bikv_producer_publish the ring's write offset belongs to the
+// reservation: any other producer call would be handed the same window.
+const char kReservedMsg[] = "a reserved ring window is waiting for bikv_producer_publish (or bikv_producer_cancel)";
+
 sem_t* sem_of(unsigned char* raw) { return reinterpret_cast<sem_t*>(raw); }
 
 void unmap_role(Role& r) {
@@ -140,11 +147,12 @@ void producer_published(Role& p, size_t at, size_t data_size) {
   if (p.backpressure) p.in_flight.emplace_back(at, data_size);
 }
 
-// The reference's publish step (copy_kernel.cu:116-128, ipc_service.cpp:130-142).
-void ring_publish(bikv_shared_control* c, size_t data_size, const int64_t* shape, size_t ndim,
+// The reference's publish step (copy_kernel.cu:116-128, ipc_service.cpp:130-142) for the transfer
+// written at offset `at` (the value ring_reserve returned for it).
+void ring_publish(bikv_shared_control* c, size_t at, size_t data_size, const int64_t* shape, size_t ndim,
                   int32_t dtype_code) {
-  c->last_valid_offset = c->current_offset;
-  c->current_offset += data_size;
+  c->last_valid_offset = at;
+  c->current_offset = at + data_size;
   c->tensor_dim = ndim;
   for (size_t i = 0; i < ndim && i < BIKV_MAX_DIM; ++i) c->tensor_shape[i] = shape[i];
   c->data_size = data_size;
@@ -196,16 +204,21 @@ extern "C" int bikv_consumer_init(int device, const char* shm_name, size_t buffe
     shm_unlink(shm_name);
     return fail(BIKV_EHIP, "consumer_init hipMalloc failed: %s", hipGetErrorString(e));
   }
-  hipIpcMemHandle_t handle;
-  memset(&handle, 0, sizeof(handle));
-  e = hipIpcGetMemHandle(&handle, r.mem);
-  if (e != hipSuccess) {
-    (void)hipFree(r.mem);
-    unmap_role(r);
-    shm_unlink(shm_name);
-    return fail(BIKV_EHIP, "consumer_init hipIpcGetMemHandle failed: %s", hipGetErrorString(e));
+  // A ring of 2 GiB or more is never exported: IPC mappings that large have been seen not to return
+  // on some ROCm hosts. Its handle stays zeroed, a producer in another process is refused
+  // (bikv_producer_init), and a producer in this process uses the pointer directly.
+  if (buffer_bytes < kMaxIpcBytes) {
+    hipIpcMemHandle_t handle;
+    memset(&handle, 0, sizeof(handle));
+    e = hipIpcGetMemHandle(&handle, r.mem);
+    if (e != hipSuccess) {
+      (void)hipFree(r.mem);
+      unmap_role(r);
+      shm_unlink(shm_name);
+      return fail(BIKV_EHIP, "consumer_init hipIpcGetMemHandle failed: %s", hipGetErrorString(e));
+    }
+    memcpy(r.ctrl->ipc_handle, &handle, sizeof(handle));
   }
-  memcpy(r.ctrl->ipc_handle, &handle, sizeof(handle));
   g_consumer = r;
   return BIKV_OK;
 }
@@ -241,13 +254,12 @@ extern "C" int bikv_producer_init(int device, const char* shm_name) {
   }
   const bool same_process = g_consumer.ctrl && strcmp(g_consumer.shm_name, shm_name) == 0;
   // Mapping another process's allocation of 2 GiB or more has been seen not to return on some
-  // ROCm hosts; such a ring is refused unless the deployment opts in.
-  const char* allow = getenv("BIKV_IPC_ALLOW_LARGE");
-  if (!same_process && r.ctrl->buffer_size >= (size_t(2) << 30) && !(allow && allow[0] == '1')) {
+  // ROCm hosts; the consumer does not export a handle for such a ring and it is refused here.
+  if (!same_process && r.ctrl->buffer_size >= kMaxIpcBytes) {
     const size_t bytes = r.ctrl->buffer_size;
     unmap_role(r);
     return fail(BIKV_ERANGE, "the consumer's ring is %zu bytes: IPC mappings of 2 GiB or more are refused "
-                             "(set BIKV_IPC_ALLOW_LARGE=1 to map it anyway)", bytes);
+                             "(use a ring below 2 GiB, or run producer and consumer in one process)", bytes);
   }
   {
     hipError_t e = hipSetDevice(device);
@@ -305,6 +317,7 @@ static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_
                          int64_t page_size, int64_t total_tokens, const bikv_tensor_dims* dims,
                          int64_t elem_bytes, int32_t dtype_code, void* stream) {
   if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
+  if (g_producer.reserved) return fail(BIKV_ESTATE, kReservedMsg);
   if (!dims) return fail(BIKV_EINVAL, "dims is null");
   if (n_runs < 0 || page_size <= 0 || elem_bytes <= 0) return fail(BIKV_EINVAL, "bad n_runs, page_size or elem_bytes");
   if (dims->head_size <= 0 || dims->num_kv_heads <= 0 || dims->num_layers <= 0 || dims->kv_pair <= 0)
@@ -328,13 +341,14 @@ static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_
     // the window handed to the kernel ends where this transfer ends: a run that would write past
     // the published bytes is skipped and reported
     char* window = static_cast<char*>(g_producer.mem) + at;
+    if (!src_off || !dst_off) return fail(BIKV_EINVAL, "null pointer argument");
     int rc = run_tokens
-        ? bikv_copy_runs_ragged(src, src_bytes, window, data_size, src_off, dst_off, run_tokens, n_runs,
-                                run_bytes, token_bytes, stream)
-        : bikv_copy_runs(src, src_bytes, window, (int64_t)(c->buffer_size - at), src_off, dst_off,
-                         n_runs, run_bytes, elem_bytes, stream);
+        ? copy_runs_banked(ST_BANK_RING, src, src_bytes, window, data_size, src_off, dst_off, run_tokens,
+                           n_runs, run_bytes, token_bytes, stream)
+        : copy_runs_banked(ST_BANK_RING, src, src_bytes, window, data_size, src_off, dst_off, nullptr,
+                           n_runs, run_bytes, elem_bytes, stream);
     if (rc) return rc;
-    rc = sync_and_check(g_producer.device, static_cast<hipStream_t>(stream));
+    rc = sync_and_check(g_producer.device, ST_BANK_RING, static_cast<hipStream_t>(stream));
     if (rc) return rc;
   }
   const int64_t shape[5] = {total_tokens, dims->head_size, dims->num_kv_heads, dims->num_layers, dims->kv_pair};
@@ -342,7 +356,7 @@ static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_
     const int rc = producer_wait_slot(g_producer);
     if (rc) return rc;
   }
-  ring_publish(c, (size_t)data_size, shape, 5, dtype_code);
+  ring_publish(c, at, (size_t)data_size, shape, 5, dtype_code);
   producer_published(g_producer, at, (size_t)data_size);
   return BIKV_OK;
 }
@@ -369,6 +383,7 @@ extern "C" int bikv_producer_copy_tokens(const void* src, int64_t src_bytes, con
 extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64_t* shape,
                                   size_t ndim, int32_t dtype_code, void* stream) {
   if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
+  if (g_producer.reserved) return fail(BIKV_ESTATE, kReservedMsg);
   if (ndim > BIKV_MAX_DIM) return fail(BIKV_EINVAL, "at most %d dimensions can be published", BIKV_MAX_DIM);
   if ((bytes > 0 && !dev_src) || (ndim > 0 && !shape)) return fail(BIKV_EINVAL, "null pointer argument");
   bikv_shared_control* c = g_producer.ctrl;
@@ -389,7 +404,7 @@ extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64
     const int rc = producer_wait_slot(g_producer);
     if (rc) return rc;
   }
-  ring_publish(c, bytes, shape, ndim, dtype_code);
+  ring_publish(c, at, bytes, shape, ndim, dtype_code);
   producer_published(g_producer, at, bytes);
   return BIKV_OK;
 }
@@ -400,6 +415,7 @@ extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64
 // pointer; publish performs the reference's bookkeeping for exactly the reserved bytes.
 extern "C" int bikv_producer_reserve(size_t bytes, void** ptr) {
   if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
+  if (g_producer.reserved) return fail(BIKV_ESTATE, kReservedMsg);
   if (!ptr) return fail(BIKV_EINVAL, "null pointer argument");
   bikv_shared_control* c = g_producer.ctrl;
   if (bytes > c->buffer_size)
@@ -421,13 +437,22 @@ extern "C" int bikv_producer_publish(const int64_t* shape, size_t ndim, int32_t 
   if (ndim > 0 && !shape) return fail(BIKV_EINVAL, "null pointer argument");
   BIKV_DEVICE(g_producer.device);
   // the bytes must be in the ring before the consumer is woken; a kernel that skipped work is an error
-  int rc = sync_and_check(g_producer.device, static_cast<hipStream_t>(stream));
+  // (the caller's own launches report into the shared status bank: a flag raised by ANY unchecked
+  // launch on this device since the last bikv_check_status fails the publication)
+  int rc = sync_and_check(g_producer.device, ST_BANK_SHARED, static_cast<hipStream_t>(stream));
+  if (rc == BIKV_EBOUNDS) g_producer.reserved = false;   // the window is incomplete: it is never published
   if (rc) return rc;
   rc = producer_wait_slot(g_producer);
   if (rc) return rc;
   g_producer.reserved = false;
-  ring_publish(g_producer.ctrl, g_producer.reserved_bytes, shape, ndim, dtype_code);
+  ring_publish(g_producer.ctrl, g_producer.reserved_at, g_producer.reserved_bytes, shape, ndim, dtype_code);
   producer_published(g_producer, g_producer.reserved_at, g_producer.reserved_bytes);
+  return BIKV_OK;
+}
+
+extern "C" int bikv_producer_cancel(void) {
+  if (!g_producer.ctrl) return fail(BIKV_ESTATE, "producer is not initialised");
+  g_producer.reserved = false;   // nothing was published: the window is handed out again next time
   return BIKV_OK;
 }
 

@@ -5,12 +5,14 @@
 #include "pagecopy_internal.h"
 #include "pagecopy_kernels.h"
 
+#include <algorithm>
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <utility>
 #include <vector>
 
 namespace bikv {
@@ -37,15 +39,16 @@ struct DevCtx {
 static std::mutex g_ctx_mu;
 static DevCtx g_ctx[64];
 
-int device_status(int device, uint32_t** dev_ptr) {
+int device_status(int device, int bank, uint32_t** dev_ptr) {
   if (device < 0 || device >= 64) return fail(BIKV_EINVAL, "device index %d out of range", device);
+  if (bank < 0 || bank >= ST_BANKS) return fail(BIKV_EINVAL, "internal: status bank %d", bank);
   std::lock_guard<std::mutex> lk(g_ctx_mu);
   DevCtx& c = g_ctx[device];
   if (!c.status_host) {
     BIKV_DEVICE(device);
     void* h = nullptr;
-    BIKV_HIP(hipHostMalloc(&h, ST_SLOTS * sizeof(uint32_t) * 8, hipHostMallocMapped | hipHostMallocPortable));
-    memset(h, 0, ST_SLOTS * sizeof(uint32_t) * 8);
+    BIKV_HIP(hipHostMalloc(&h, ST_SLOTS * sizeof(uint32_t) * ST_BANKS, hipHostMallocMapped | hipHostMallocPortable));
+    memset(h, 0, ST_SLOTS * sizeof(uint32_t) * ST_BANKS);
     void* d = nullptr;
     hipError_t e = hipHostGetDevicePointer(&d, h, 0);
     if (e != hipSuccess) {
@@ -55,15 +58,15 @@ int device_status(int device, uint32_t** dev_ptr) {
     c.status_host = static_cast<uint32_t*>(h);
     c.status_dev = static_cast<uint32_t*>(d);
   }
-  *dev_ptr = c.status_dev;
+  *dev_ptr = c.status_dev + bank * ST_SLOTS;
   return BIKV_OK;
 }
 
-static uint32_t take_status(int device) {
+static uint32_t take_status(int device, int bank) {
   std::lock_guard<std::mutex> lk(g_ctx_mu);
   DevCtx& c = g_ctx[device];
   if (!c.status_host) return 0;
-  volatile uint32_t* s = c.status_host;
+  volatile uint32_t* s = c.status_host + bank * ST_SLOTS;
   uint32_t bits = 0;
   if (s[ST_SLOT_SRC]) bits |= BIKV_ST_SRC_RANGE;
   if (s[ST_SLOT_DST]) bits |= BIKV_ST_DST_RANGE;
@@ -82,10 +85,12 @@ static int status_error(uint32_t bits) {
               (bits & BIKV_ST_PAGE_ID) ? " page-id" : "");
 }
 
-int sync_and_check(int device, hipStream_t stream) {
+int sync_and_check(int device, int bank, hipStream_t stream) {
   BIKV_HIP(hipStreamSynchronize(stream));
-  return status_error(take_status(device));
+  return status_error(take_status(device, bank));
 }
+
+int check_bank(int device, int bank) { return status_error(take_status(device, bank)); }
 
 static int current_device(int* dev) {
   BIKV_HIP(hipGetDevice(dev));
@@ -122,10 +127,12 @@ extern "C" int bikv_check_status(int device, void* stream, uint32_t* bits_out) {
   if (device < 0 || device >= 64) return fail(BIKV_EINVAL, "device index %d out of range", device);
   BIKV_DEVICE(device);
   BIKV_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
-  const uint32_t bits = take_status(device);
+  const uint32_t bits = take_status(device, ST_BANK_SHARED);
   if (bits_out) *bits_out = bits;
   return status_error(bits);
 }
+
+extern "C" void bikv_reset_tuning(void) { tuning() = Tuning(); }
 
 extern "C" int bikv_set_tuning(const char* key, int64_t value) {
   if (!key) return fail(BIKV_EINVAL, "null tuning key");
@@ -167,6 +174,8 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
     t.transpose_block = (int)value;
   } else if (!strcmp(key, "transpose_pairs")) {
     t.transpose_pairs = value ? 1 : 0;
+  } else if (!strcmp(key, "debug_unique")) {
+    t.debug_unique = value ? 1 : 0;
   } else if (!strcmp(key, "run_chunk_kib")) {
     if (value < 0 || value > 1 << 20) return fail(BIKV_EINVAL, "run_chunk_kib out of range");
     t.run_chunk_kib = (int)value;
@@ -216,7 +225,7 @@ extern "C" int bikv_pool_create(const bikv_pool_desc* d, bikv_pool** out) {
     }
   }
   uint32_t* st = nullptr;
-  int rc = device_status(d->device, &st);
+  int rc = device_status(d->device, ST_BANK_SHARED, &st);
   if (rc) return rc;
   BIKV_DEVICE(d->device);
   void* dtab = nullptr;
@@ -256,7 +265,7 @@ namespace bikv {
 
 // Fills MoveArgs for one launch; `staging`/`scale_staging` are slot 0 of the (possibly windowed)
 // staging image after slot_bias has been applied.
-static int build_move(const bikv_pool* pool, const bikv_page_batch* b, const void* staging,
+static int build_move(int bank, const bikv_pool* pool, const bikv_page_batch* b, const void* staging,
                       int64_t staging_bytes, const void* scale_staging, int64_t scale_bytes,
                       MoveArgs* m) {
   if (!pool || !b) return fail(BIKV_EINVAL, "null pool or batch");
@@ -278,7 +287,7 @@ static int build_move(const bikv_pool* pool, const bikv_page_batch* b, const voi
   if (has_scale && (!scale_staging || scale_bytes < 0))
     return fail(BIKV_EINVAL, "pool has a scale class: scale_staging must be given");
   uint32_t* st = nullptr;
-  int rc = device_status(pool->device, &st);
+  int rc = device_status(pool->device, bank, &st);
   if (rc) return rc;
   m->page_ids = b->page_ids;
   m->slots = b->slots;
@@ -311,11 +320,11 @@ static int build_move(const bikv_pool* pool, const bikv_page_batch* b, const voi
   return BIKV_OK;
 }
 
-static int move_pages(int dir, const bikv_pool* pool, const bikv_page_batch* b, const void* staging,
+static int move_pages(int bank, int dir, const bikv_pool* pool, const bikv_page_batch* b, const void* staging,
                       int64_t staging_bytes, const void* scale_staging, int64_t scale_bytes,
                       void* stream) {
   MoveArgs m;
-  int rc = build_move(pool, b, staging, staging_bytes, scale_staging, scale_bytes, &m);
+  int rc = build_move(bank, pool, b, staging, staging_bytes, scale_staging, scale_bytes, &m);
   if (rc) return rc;
   if (m.n_batch == 0) return BIKV_OK;
   BIKV_DEVICE(pool->device);
@@ -326,22 +335,89 @@ static int move_pages(int dir, const bikv_pool* pool, const bikv_page_batch* b, 
 
 }  // namespace bikv
 
+// ---- duplicate destinations ---------------------------------------------------------------------
+// Two runs of one launch that write the same destination race (the reference's kernel has the same
+// property, copy_kernel.cu:29-35: whichever block stores last wins). bikv_find_duplicate is the check
+// on a host array; with BIKV_DEBUG_UNIQUE=1 in the environment the scattering entry points run it on a
+// copy of the caller's device ids before they launch (a debugging aid: it synchronises the stream).
+extern "C" int bikv_find_duplicate(const int64_t* ids, int64_t n, int64_t* dup_out) {
+  if (n < 0 || (n > 0 && !ids)) return fail(BIKV_EINVAL, "bad find_duplicate arguments");
+  std::vector<std::pair<int64_t, int64_t>> v((size_t)n);
+  for (int64_t i = 0; i < n; ++i) v[(size_t)i] = {ids[i], i};
+  std::sort(v.begin(), v.end());
+  // report the repeated id whose second occurrence comes first in the caller's order (within a group
+  // of equal ids the positions ascend, because the pairs were sorted)
+  int64_t best = -1, best_first = 0, best_id = 0;
+  for (size_t i = 0; i + 1 < v.size();) {
+    size_t j = i + 1;
+    while (j < v.size() && v[j].first == v[i].first) ++j;
+    if (j - i >= 2 && (best < 0 || v[i + 1].second < best)) {
+      best = v[i + 1].second;
+      best_first = v[i].second;
+      best_id = v[i].first;
+    }
+    i = j;
+  }
+  if (best < 0) return BIKV_OK;
+  if (dup_out) *dup_out = best_id;
+  return fail(BIKV_EINVAL, "destination id %lld is named more than once (entries %lld and %lld): a scatter's "
+                           "destinations must be unique", (long long)best_id, (long long)best_first, (long long)best);
+}
+
+namespace bikv {
+
+static bool debug_unique() {
+  static const bool env_on = [] {
+    const char* e = getenv("BIKV_DEBUG_UNIQUE");
+    return e && e[0] && e[0] != '0';
+  }();
+  return env_on || tuning().debug_unique != 0;
+}
+
+// Debug path: fetches `n` device ids behind `stream` and fails if one repeats.
+int check_unique_on_device(int device, const int64_t* dev_ids, int64_t n, hipStream_t stream) {
+  if (!debug_unique() || n <= 1 || !dev_ids) return BIKV_OK;
+  BIKV_DEVICE(device);
+  std::vector<int64_t> host((size_t)n);
+  BIKV_HIP(hipStreamSynchronize(stream));
+  BIKV_HIP(hipMemcpy(host.data(), dev_ids, (size_t)n * sizeof(int64_t), hipMemcpyDeviceToHost));
+  return bikv_find_duplicate(host.data(), n, nullptr);
+}
+
+}  // namespace bikv
+
 extern "C" int bikv_gather_pages(const bikv_pool* pool, const bikv_page_batch* batch, void* staging,
                                  int64_t staging_bytes, void* scale_staging,
                                  int64_t scale_staging_bytes, void* stream) {
-  return move_pages(0, pool, batch, staging, staging_bytes, scale_staging, scale_staging_bytes, stream);
+  return move_pages(ST_BANK_SHARED, 0, pool, batch, staging, staging_bytes, scale_staging, scale_staging_bytes, stream);
 }
 
 extern "C" int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* batch,
                                   const void* staging, int64_t staging_bytes,
                                   const void* scale_staging, int64_t scale_staging_bytes,
                                   void* stream) {
-  return move_pages(1, pool, batch, staging, staging_bytes, scale_staging, scale_staging_bytes, stream);
+  if (pool && batch) {
+    const int rc = check_unique_on_device(pool->device, batch->page_ids, batch->n_pages, static_cast<hipStream_t>(stream));
+    if (rc) return rc;
+  }
+  return move_pages(ST_BANK_SHARED, 1, pool, batch, staging, staging_bytes, scale_staging, scale_staging_bytes, stream);
 }
 
-static int copy_runs_impl(const void* src, int64_t src_bytes, void* dst, int64_t dst_bytes,
-                          const int64_t* src_off, const int64_t* dst_off, const int64_t* run_len,
-                          int64_t n_runs, int64_t run_bytes, int64_t unit_bytes, void* stream) {
+// The device that owns the memory behind `p`, or -1 when the runtime does not know the pointer or it is
+// host memory.
+static int device_of_pointer(const void* p) {
+  hipPointerAttribute_t at;
+  memset(&at, 0, sizeof(at));
+  if (hipPointerGetAttributes(&at, p) != hipSuccess) {
+    (void)hipGetLastError();   // an unknown pointer is not an error of this call
+    return -1;
+  }
+  return at.type == hipMemoryTypeDevice ? at.device : -1;
+}
+
+int bikv::copy_runs_banked(int bank, const void* src, int64_t src_bytes, void* dst, int64_t dst_bytes,
+                           const int64_t* src_off, const int64_t* dst_off, const int64_t* run_len,
+                           int64_t n_runs, int64_t run_bytes, int64_t unit_bytes, void* stream) {
   if (n_runs < 0 || run_bytes < 0) return fail(BIKV_EINVAL, "negative n_runs or run_bytes");
   if (n_runs == 0 || run_bytes == 0) return BIKV_OK;
   if (!src || !dst || !src_off || !dst_off) return fail(BIKV_EINVAL, "null pointer argument");
@@ -350,9 +426,18 @@ static int copy_runs_impl(const void* src, int64_t src_bytes, void* dst, int64_t
   if (!run_len && (run_bytes > src_bytes || run_bytes > dst_bytes))
     return fail(BIKV_EINVAL, "run_bytes %lld exceeds a buffer (src %lld, dst %lld bytes)",
                 (long long)run_bytes, (long long)src_bytes, (long long)dst_bytes);
-  int dev = 0;
-  int rc = current_device(&dev);
-  if (rc) return rc;
+  // The launch and its status words belong to the device that holds the data: the destination's, else
+  // the source's (one of the two may be pinned host memory), else the offset tables', and the calling
+  // thread's current device only when the runtime knows none of the pointers.
+  int dev = device_of_pointer(dst);
+  if (dev < 0) dev = device_of_pointer(src);
+  if (dev < 0) dev = device_of_pointer(src_off);
+  int rc = BIKV_OK;
+  if (dev < 0) {
+    rc = current_device(&dev);
+    if (rc) return rc;
+  }
+  BIKV_DEVICE(dev);
   RunArgs a;
   a.src = static_cast<const char*>(src);
   a.dst = static_cast<char*>(dst);
@@ -364,7 +449,7 @@ static int copy_runs_impl(const void* src, int64_t src_bytes, void* dst, int64_t
   a.run_bytes = run_bytes;
   a.unit_bytes = unit_bytes;
   a.run_lens = run_len;
-  rc = device_status(dev, &a.status);
+  rc = device_status(dev, bank, &a.status);
   if (rc) return rc;
   hipError_t e = launch_copy_runs(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail_hip(e, "copy_runs launch");
@@ -374,8 +459,8 @@ static int copy_runs_impl(const void* src, int64_t src_bytes, void* dst, int64_t
 extern "C" int bikv_copy_runs(const void* src, int64_t src_bytes, void* dst, int64_t dst_bytes,
                               const int64_t* src_off, const int64_t* dst_off, int64_t n_runs,
                               int64_t run_bytes, int64_t unit_bytes, void* stream) {
-  return copy_runs_impl(src, src_bytes, dst, dst_bytes, src_off, dst_off, nullptr, n_runs, run_bytes,
-                        unit_bytes, stream);
+  return copy_runs_banked(ST_BANK_SHARED, src, src_bytes, dst, dst_bytes, src_off, dst_off, nullptr, n_runs,
+                          run_bytes, unit_bytes, stream);
 }
 
 extern "C" int bikv_copy_runs_ragged(const void* src, int64_t src_bytes, void* dst, int64_t dst_bytes,
@@ -383,8 +468,8 @@ extern "C" int bikv_copy_runs_ragged(const void* src, int64_t src_bytes, void* d
                                      const int64_t* run_len, int64_t n_runs, int64_t max_run_bytes,
                                      int64_t unit_bytes, void* stream) {
   if (n_runs > 0 && !run_len) return fail(BIKV_EINVAL, "run_len is null");
-  return copy_runs_impl(src, src_bytes, dst, dst_bytes, src_off, dst_off, run_len, n_runs,
-                        max_run_bytes, unit_bytes, stream);
+  return copy_runs_banked(ST_BANK_SHARED, src, src_bytes, dst, dst_bytes, src_off, dst_off, run_len, n_runs,
+                          max_run_bytes, unit_bytes, stream);
 }
 
 // ---- pinned host memory -------------------------------------------------------------------
@@ -432,41 +517,71 @@ extern "C" int bikv_h2d_copy(int device, void* dev_dst, const void* host_src, in
   return link_copy(device, dev_dst, host_src, bytes, chunk_bytes, hipMemcpyHostToDevice, seconds_out);
 }
 
-// ---- device -> pinned-host staging pipeline -----------------------------------------------
-// The stager owns n_buffers "lanes": a HIP stream with its own chunk buffer in HBM. Chunk c of a
-// call goes to lane c % n_buffers, which gathers it into its buffer and then copies the buffer to
-// the host, both in stream order. Lanes never wait on each other (no cross-stream events: on this
-// platform a hipMemcpyAsync that waits on another stream's event ran at ~40 % of the link for
-// chunks below 32 MiB), so while one lane's copy occupies the host link the next lane's gather
-// and copy are already queued behind it.
+// ---- device <-> pinned-host staging pipeline -----------------------------------------------
+// The stager owns n_buffers "lanes": a HIP stream with its own buffer in HBM. Launch k of the pipeline
+// runs on lane k % n_buffers: ONE gather kernel fills the lane's buffer with `group` chunks' worth of the
+// staging image, then `group` hipMemcpyAsync calls of chunk_bytes each move it to the host, all in the
+// lane's stream order (for the receiving direction: the copies first, then one scatter kernel). Lanes
+// never wait on each other: while one lane's copies occupy the host link the next lane's kernel has
+// long finished (it moves its bytes ~100x faster than the link does) and its copies are queued.
+//
+// What shaped this (measured on MI355X, 64 KiB tiles, 1 GiB per pass, copies timed by rocprofv3's
+// memory-copy trace):
+//   * the DMA engine leaves ~9.5 us between two consecutive copies whatever stream they come from, so
+//     4 MiB copies cannot exceed ~88 % of the link and 8 / 16 / 32 MiB reach 93 / 96 / 98 %;
+//   * a kernel between two copies of one stream costs one more hand-over each way: one lane alone loses
+//     another 5-10 %, two lanes hide it, more than two add nothing;
+//   * host -> device, one kernel per copy makes small chunks erratic (4 MiB x 4 lanes: 72-95 % from pass
+//     to pass) while one kernel per 4-8 copies stays at 95-98 %: hence `group`;
+//   * ordering a copy stream behind a kernel stream with events loses 10-30 % below 16 MiB;
+//   * the device -> host DMA path has two speeds on this platform, ~30 and ~57 GB/s, and a process can
+//     sit in either for minutes (the host -> device path and kernels storing into mapped pinned memory
+//     do not show it): BIKV_STAGE_DIRECT keeps 55 GB/s in both states, which is why BIKV_STAGE_AUTO
+//     sends with the kernel and receives with the DMA engine.
 struct bikv_stager {
   int device;
-  int64_t chunk_bytes;
+  int64_t chunk_bytes;       // bytes of one host copy
+  int group;                 // copies per kernel launch
+  int64_t lane_bytes;        // chunk_bytes * group: HBM buffer of one lane
   int n_buf;
   char* ring;
-  char* scale_ring;          // grown on demand: n_buf chunks of scale tiles
+  char* scale_ring;          // grown on demand: n_buf buffers of scale tiles
   int64_t scale_ring_bytes;
   std::vector<hipStream_t> lanes;
+  hipEvent_t after;          // orders the lanes behind a caller's stream
+  uint64_t next_launch;      // launches issued since creation (lane = next_launch % n_buf)
+  // since the last bikv_stager_wait
+  int64_t pending_bytes, pending_copies;
+  bool timing;
+  std::chrono::steady_clock::time_point t_first;
 };
 
-extern "C" int bikv_stager_create(int device, int64_t chunk_bytes, int32_t n_buffers,
-                                  bikv_stager** out) {
+extern "C" int bikv_stager_create(int device, int64_t chunk_bytes, int32_t chunks_per_launch,
+                                  int32_t n_buffers, bikv_stager** out) {
   if (!out) return fail(BIKV_EINVAL, "null out");
   *out = nullptr;
-  if (chunk_bytes < 4096 || n_buffers < 1 || n_buffers > 16)
-    return fail(BIKV_EINVAL, "need chunk_bytes >= 4096 and 1 <= n_buffers <= 16");
+  if (chunk_bytes < 4096 || n_buffers < 1 || n_buffers > 16 || chunks_per_launch < 1 || chunks_per_launch > 64)
+    return fail(BIKV_EINVAL, "need chunk_bytes >= 4096, 1 <= chunks_per_launch <= 64 and 1 <= n_buffers <= 16");
+  if (chunk_bytes > (int64_t(1) << 36) / chunks_per_launch) return fail(BIKV_EINVAL, "lane buffer too large");
   uint32_t* st_ptr = nullptr;
-  int rc = device_status(device, &st_ptr);
+  int rc = device_status(device, ST_BANK_STAGER, &st_ptr);
   if (rc) return rc;
   BIKV_DEVICE(device);
   bikv_stager* st = new bikv_stager();
   st->device = device;
   st->chunk_bytes = chunk_bytes;
+  st->group = chunks_per_launch;
+  st->lane_bytes = chunk_bytes * chunks_per_launch;
   st->n_buf = n_buffers;
   st->ring = nullptr;
   st->scale_ring = nullptr;
   st->scale_ring_bytes = 0;
-  hipError_t e = hipMalloc((void**)&st->ring, (size_t)chunk_bytes * n_buffers);
+  st->after = nullptr;
+  st->next_launch = 0;
+  st->pending_bytes = st->pending_copies = 0;
+  st->timing = false;
+  hipError_t e = hipMalloc((void**)&st->ring, (size_t)st->lane_bytes * n_buffers);
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&st->after, hipEventDisableTiming);
   for (int i = 0; i < n_buffers && e == hipSuccess; ++i) {
     hipStream_t s = nullptr;
     e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);  // default priority
@@ -487,6 +602,7 @@ extern "C" int bikv_stager_destroy(bikv_stager* st) {
     (void)hipStreamSynchronize(s);
     (void)hipStreamDestroy(s);
   }
+  if (st->after) (void)hipEventDestroy(st->after);
   if (st->ring) (void)hipFree(st->ring);
   if (st->scale_ring) (void)hipFree(st->scale_ring);
   delete st;
@@ -503,90 +619,87 @@ struct Chunk {
   int64_t first_slot, n_slots;  // staging slots covered
 };
 
-// Cuts the staging image of a batch into chunks of at most `max_slots` slots. Requests are packed
-// back to back in batch order.
-static void plan_chunks(const int64_t* req_pages, int64_t n_req, int n_planes, int layout,
-                        int64_t max_slots, std::vector<Chunk>* out) {
-  int64_t first_page = 0, base_slot = 0;
-  if (layout == BIKV_LAYOUT_PAGE_MAJOR) {
-    // slot = global_page * n_planes + plane: any run of whole pages is contiguous, across requests
-    int64_t total = 0;
-    for (int64_t r = 0; r < n_req; ++r) total += req_pages[r];
-    if (max_slots >= n_planes) {
-      const int64_t per = max_slots / n_planes;
-      for (int64_t p = 0; p < total; p += per) {
-        const int64_t n = total - p < per ? total - p : per;
-        out->push_back(Chunk{p, n, 0, n_planes, p * n_planes, n * n_planes});
-      }
-    } else {
-      // a chunk is smaller than one page: cut every page into runs of consecutive planes
-      for (int64_t p = 0; p < total; ++p)
-        for (int q = 0; q < n_planes; q += (int)max_slots) {
-          const int c = n_planes - q < (int)max_slots ? n_planes - q : (int)max_slots;
-          out->push_back(Chunk{p, 1, q, c, p * n_planes + q, c});
-        }
-    }
-    return;
+// Cuts the staging image of a batch into pieces of at most `max_slots` slots, one per call of next().
+// Requests are packed back to back in batch order. Holds no memory of its own.
+class ChunkPlanner {
+ public:
+  ChunkPlanner(const int64_t* req_pages, int64_t n_req, int n_planes, int layout, int64_t max_slots)
+      : req_(req_pages), n_req_(n_req), planes_(n_planes), layout_(layout), max_(max_slots) {
+    if (layout_ == BIKV_LAYOUT_PAGE_MAJOR)
+      for (int64_t r = 0; r < n_req_; ++r) total_ += req_[r];
   }
-  for (int64_t r = 0; r < n_req; ++r) {
-    const int64_t m = req_pages[r];
-    if (m > 0) {
-      if (m <= max_slots) {
-        int k = (int)(max_slots / m);  // whole plane rows per chunk
-        if (k > n_planes) k = n_planes;
-        for (int q = 0; q < n_planes; q += k) {
-          const int c = n_planes - q < k ? n_planes - q : k;
-          out->push_back(Chunk{first_page, m, q, c, base_slot + (int64_t)q * m, (int64_t)c * m});
-        }
+
+  bool next(Chunk* out) {
+    if (layout_ == BIKV_LAYOUT_PAGE_MAJOR) {
+      // slot = global_page * n_planes + plane: any run of whole pages is contiguous, across requests
+      if (p_ >= total_) return false;
+      if (max_ >= planes_) {
+        const int64_t per = max_ / planes_;
+        const int64_t n = total_ - p_ < per ? total_ - p_ : per;
+        *out = Chunk{p_, n, 0, planes_, p_ * planes_, n * planes_};
+        p_ += n;
       } else {
-        for (int q = 0; q < n_planes; ++q)
-          for (int64_t j = 0; j < m; j += max_slots) {
-            const int64_t n = m - j < max_slots ? m - j : max_slots;
-            out->push_back(Chunk{first_page + j, n, q, 1, base_slot + (int64_t)q * m + j, n});
-          }
+        // a piece is smaller than one page: cut every page into runs of consecutive planes
+        const int c = planes_ - q_ < (int)max_ ? planes_ - q_ : (int)max_;
+        *out = Chunk{p_, 1, q_, c, p_ * planes_ + q_, c};
+        q_ += c;
+        if (q_ >= planes_) { q_ = 0; ++p_; }
       }
+      return true;
     }
-    first_page += m;
-    base_slot += m * n_planes;
+    while (r_ < n_req_ && req_[r_] == 0) ++r_;
+    if (r_ >= n_req_) return false;
+    const int64_t m = req_[r_];
+    if (m <= max_) {
+      int k = (int)(max_ / m);  // whole plane rows per piece
+      if (k > planes_) k = planes_;
+      const int c = planes_ - q_ < k ? planes_ - q_ : k;
+      *out = Chunk{first_page_, m, q_, c, base_slot_ + (int64_t)q_ * m, (int64_t)c * m};
+      q_ += c;
+    } else {
+      const int64_t n = m - j_ < max_ ? m - j_ : max_;
+      *out = Chunk{first_page_ + j_, n, q_, 1, base_slot_ + (int64_t)q_ * m + j_, n};
+      j_ += n;
+      if (j_ >= m) { j_ = 0; ++q_; }
+    }
+    if (q_ >= planes_) {
+      q_ = 0;
+      first_page_ += m;
+      base_slot_ += m * planes_;
+      ++r_;
+    }
+    return true;
   }
-}
 
-}  // namespace bikv
+ private:
+  const int64_t* req_;
+  int64_t n_req_;
+  int planes_, layout_;
+  int64_t max_;
+  int64_t total_ = 0, p_ = 0;                       // page-major walk
+  int64_t r_ = 0, j_ = 0, first_page_ = 0, base_slot_ = 0;
+  int q_ = 0;
+};
 
-extern "C" int64_t bikv_plan_chunks(const int64_t* req_pages, int64_t n_requests, int32_t n_planes,
-                                    int32_t layout, int64_t max_slots, int64_t* out, int64_t cap) {
-  if (!req_pages || n_requests < 0 || n_planes <= 0 || max_slots < 1 || (cap > 0 && !out))
-    return fail(BIKV_EINVAL, "bad plan_chunks arguments");
-  if (layout != BIKV_LAYOUT_LAYER_MAJOR && layout != BIKV_LAYOUT_PAGE_MAJOR)
-    return fail(BIKV_EINVAL, "unknown layout %d", layout);
-  for (int64_t r = 0; r < n_requests; ++r)
-    if (req_pages[r] < 0) return fail(BIKV_EINVAL, "negative req_pages[%lld]", (long long)r);
-  std::vector<Chunk> chunks;
-  plan_chunks(req_pages, n_requests, n_planes, layout, max_slots, &chunks);
-  for (size_t c = 0; c < chunks.size() && (int64_t)c < cap; ++c) {
-    int64_t* o = out + 6 * c;
-    o[0] = chunks[c].first_page; o[1] = chunks[c].n_pages;
-    o[2] = chunks[c].plane_begin; o[3] = chunks[c].plane_count;
-    o[4] = chunks[c].first_slot; o[5] = chunks[c].n_slots;
-  }
-  return (int64_t)chunks.size();
-}
+// The lanes a pipeline call runs on: the stager's own, or (allocation-free entry point) the caller's
+// stream with a buffer that already exists.
+struct LaneSet {
+  int n;
+  hipStream_t* streams;
+  char* buf;               // lane l uses buf + l*lane_bytes
+  char* scale_buf;         // lane l uses scale_buf + l*scale_lane_bytes (null: pool has no scale class)
+  int64_t lane_bytes, scale_lane_bytes, chunk_bytes;
+  uint64_t* next_launch;
+  int bank;
+};
 
-// Both directions of the host staging pipeline. dir 0: pool -> device chunk -> host image;
-// dir 1: host image -> device chunk -> pool. A lane's stream orders the two steps of a chunk and
-// keeps its chunk buffer safe from the lane's next chunk.
-static int stage_between_host(int dir, bikv_stager* st, const bikv_pool* pool,
-                              const bikv_page_batch* batch, const int64_t* req_pages,
-                              int64_t n_requests, int32_t layout, void* host_dst,
-                              int64_t host_bytes, void* host_scale_dst,
-                              int64_t host_scale_bytes, int32_t mode,
-                              bikv_stage_stats* stats) {
-  if (!st || !pool || !batch || !req_pages || !host_dst)
-    return fail(BIKV_EINVAL, "null argument");
+static int validate_stage_args(const bikv_pool* pool, const bikv_page_batch* batch, const int64_t* req_pages,
+                               int64_t n_requests, int32_t layout, const void* host, int64_t host_bytes,
+                               const void* host_scale, int64_t host_scale_bytes, int64_t* total_pages_out) {
+  if (!pool || !batch || !req_pages || !host) return fail(BIKV_EINVAL, "null argument");
   const bool has_scale = pool->scale_tile_bytes > 0;
-  if (has_scale && !host_scale_dst)
+  if (has_scale && !host_scale)
     return fail(BIKV_EINVAL, "pool has a scale class: the host scale image must be given");
-  if (pool->device != st->device) return fail(BIKV_EINVAL, "pool and stager are on different devices");
   if (layout != BIKV_LAYOUT_LAYER_MAJOR && layout != BIKV_LAYOUT_PAGE_MAJOR)
     return fail(BIKV_EINVAL, "unknown layout %d", layout);
   if (batch->plane_count > 0 && (batch->plane_begin != 0 || batch->plane_count != pool->n_planes))
@@ -600,118 +713,232 @@ static int stage_between_host(int dir, bikv_stager* st, const bikv_pool* pool,
   if (total_pages != batch->n_pages)
     return fail(BIKV_EINVAL, "req_pages sums to %lld but the batch has %lld pages",
                 (long long)total_pages, (long long)batch->n_pages);
-  const int64_t T = pool->tile_bytes;
-  const int64_t S = pool->scale_tile_bytes;
-  const int64_t image_bytes = total_pages * pool->n_planes * T;
-  const int64_t scale_image_bytes = total_pages * pool->n_planes * S;
+  const int64_t image_bytes = total_pages * pool->n_planes * pool->tile_bytes;
+  const int64_t scale_image_bytes = total_pages * pool->n_planes * pool->scale_tile_bytes;
   if (host_bytes < image_bytes)
     return fail(BIKV_ERANGE, "host buffer holds %lld bytes, staging image needs %lld",
                 (long long)host_bytes, (long long)image_bytes);
   if (has_scale && host_scale_bytes < scale_image_bytes)
     return fail(BIKV_ERANGE, "host scale buffer holds %lld bytes, scale image needs %lld",
                 (long long)host_scale_bytes, (long long)scale_image_bytes);
-  if (stats) { stats->bytes = 0; stats->n_chunks = 0; stats->wall_seconds = 0.0; }
-  if (total_pages == 0) return BIKV_OK;
-  BIKV_DEVICE(st->device);
-  const auto t0 = std::chrono::steady_clock::now();
+  *total_pages_out = total_pages;
+  return BIKV_OK;
+}
 
+// Enqueues the pipelined transfer of a batch on `L` and returns without waiting. dir 0: pool -> lane
+// buffer -> host image; dir 1: host image -> lane buffer -> pool. A lane's stream orders the steps of a
+// launch and keeps its buffer safe from the lane's next launch.
+static int issue_pipelined(int dir, const bikv_pool* pool, const bikv_page_batch* batch,
+                           const int64_t* req_pages, int64_t n_requests, int32_t layout, char* host,
+                           char* host_scale, const LaneSet& L, int64_t* n_copies) {
+  const int64_t T = pool->tile_bytes, S = pool->scale_tile_bytes;
+  const bool has_scale = S > 0;
+  int64_t max_slots = L.lane_bytes / T;
+  if (max_slots < 1)
+    return fail(BIKV_ERANGE, "chunk_bytes %lld is smaller than one tile (%lld bytes)",
+                (long long)L.lane_bytes, (long long)T);
+  if (has_scale && max_slots * S > L.scale_lane_bytes) max_slots = L.scale_lane_bytes / S;
+  if (max_slots < 1) return fail(BIKV_ERANGE, "the scale buffer of a lane is smaller than one scale tile");
+  ChunkPlanner plan(req_pages, n_requests, pool->n_planes, layout, max_slots);
+  Chunk ch;
+  while (plan.next(&ch)) {
+    const int lane = (int)(*L.next_launch % (uint64_t)L.n);
+    ++*L.next_launch;
+    hipStream_t stream = L.streams[lane];
+    char* dev_chunk = L.buf + (int64_t)lane * L.lane_bytes;
+    char* dev_scale = has_scale ? L.scale_buf + (int64_t)lane * L.scale_lane_bytes : nullptr;
+    bikv_page_batch sub = *batch;
+    sub.page_ids = batch->page_ids + ch.first_page;
+    sub.slots = batch->slots + ch.first_page;
+    sub.slot_strides = batch->slot_strides + ch.first_page;
+    sub.n_pages = ch.n_pages;
+    sub.plane_begin = ch.plane_begin;
+    sub.plane_count = ch.plane_count;
+    sub.slot_bias = ch.first_slot;
+    const int64_t bytes = ch.n_slots * T;
+    char* host_chunk = host + ch.first_slot * T;
+    char* host_scale_chunk = has_scale ? host_scale + ch.first_slot * S : nullptr;
+    if (dir == 0) {
+      const int rc = move_pages(L.bank, 0, pool, &sub, dev_chunk, bytes, dev_scale, ch.n_slots * S, stream);
+      if (rc) return rc;
+    }
+    for (int64_t off = 0; off < bytes; off += L.chunk_bytes) {
+      const int64_t n = bytes - off < L.chunk_bytes ? bytes - off : L.chunk_bytes;
+      BIKV_HIP(dir == 0 ? hipMemcpyAsync(host_chunk + off, dev_chunk + off, (size_t)n, hipMemcpyDeviceToHost, stream)
+                        : hipMemcpyAsync(dev_chunk + off, host_chunk + off, (size_t)n, hipMemcpyHostToDevice, stream));
+      ++*n_copies;
+    }
+    if (has_scale)
+      BIKV_HIP(dir == 0 ? hipMemcpyAsync(host_scale_chunk, dev_scale, (size_t)(ch.n_slots * S), hipMemcpyDeviceToHost, stream)
+                        : hipMemcpyAsync(dev_scale, host_scale_chunk, (size_t)(ch.n_slots * S), hipMemcpyHostToDevice, stream));
+    if (dir == 1) {
+      const int rc = move_pages(L.bank, 1, pool, &sub, dev_chunk, bytes, dev_scale, ch.n_slots * S, stream);
+      if (rc) return rc;
+    }
+  }
+  return BIKV_OK;
+}
+
+}  // namespace bikv
+
+extern "C" int64_t bikv_plan_chunks(const int64_t* req_pages, int64_t n_requests, int32_t n_planes,
+                                    int32_t layout, int64_t max_slots, int64_t* out, int64_t cap) {
+  if (!req_pages || n_requests < 0 || n_planes <= 0 || max_slots < 1 || (cap > 0 && !out))
+    return fail(BIKV_EINVAL, "bad plan_chunks arguments");
+  if (layout != BIKV_LAYOUT_LAYER_MAJOR && layout != BIKV_LAYOUT_PAGE_MAJOR)
+    return fail(BIKV_EINVAL, "unknown layout %d", layout);
+  for (int64_t r = 0; r < n_requests; ++r)
+    if (req_pages[r] < 0) return fail(BIKV_EINVAL, "negative req_pages[%lld]", (long long)r);
+  ChunkPlanner plan(req_pages, n_requests, n_planes, layout, max_slots);
+  Chunk ch;
+  int64_t c = 0;
+  for (; plan.next(&ch); ++c) {
+    if (c >= cap) continue;
+    int64_t* o = out + 6 * c;
+    o[0] = ch.first_page; o[1] = ch.n_pages;
+    o[2] = ch.plane_begin; o[3] = ch.plane_count;
+    o[4] = ch.first_slot; o[5] = ch.n_slots;
+  }
+  return c;
+}
+
+static void drain_lanes(bikv_stager* st) {
+  for (hipStream_t s : st->lanes) (void)hipStreamSynchronize(s);
+}
+
+// Both directions of the host staging pipeline, enqueue only.
+static int stage_issue(int dir, bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
+                       const int64_t* req_pages, int64_t n_requests, int32_t layout, void* host,
+                       int64_t host_bytes, void* host_scale, int64_t host_scale_bytes, int32_t mode,
+                       void* after_stream) {
+  if (!st) return fail(BIKV_EINVAL, "null argument");
+  int64_t total_pages = 0;
+  int rc = validate_stage_args(pool, batch, req_pages, n_requests, layout, host, host_bytes, host_scale,
+                               host_scale_bytes, &total_pages);
+  if (rc) return rc;
+  if (pool->device != st->device) return fail(BIKV_EINVAL, "pool and stager are on different devices");
+  if (mode == BIKV_STAGE_AUTO) mode = dir == 0 ? BIKV_STAGE_DIRECT : BIKV_STAGE_PIPELINED;
+  if (mode != BIKV_STAGE_DIRECT && mode != BIKV_STAGE_PIPELINED)
+    return fail(BIKV_EINVAL, "unknown staging mode %d", mode);
+  if (total_pages == 0) return BIKV_OK;
+  const bool has_scale = pool->scale_tile_bytes > 0;
+  const int64_t T = pool->tile_bytes, S = pool->scale_tile_bytes;
+  const int64_t image_bytes = total_pages * pool->n_planes * T;
+  const int64_t scale_image_bytes = total_pages * pool->n_planes * S;
+  BIKV_DEVICE(st->device);
+  if (dir == 1) {
+    rc = check_unique_on_device(st->device, batch->page_ids, batch->n_pages, static_cast<hipStream_t>(after_stream));
+    if (rc) return rc;
+  }
+  if (!st->timing) {
+    st->timing = true;
+    st->t_first = std::chrono::steady_clock::now();
+  }
+  const int n_lanes_used = mode == BIKV_STAGE_DIRECT ? 1 : st->n_buf;
+  if (after_stream) {
+    // the caller's stream may still be uploading the index arrays: the lanes start behind it
+    BIKV_HIP(hipEventRecord(st->after, static_cast<hipStream_t>(after_stream)));
+    for (int l = 0; l < n_lanes_used; ++l) {
+      const int lane = (int)((st->next_launch + (uint64_t)l) % (uint64_t)st->n_buf);
+      BIKV_HIP(hipStreamWaitEvent(st->lanes[lane], st->after, 0));
+    }
+  }
+  int64_t copies = 0;
   if (mode == BIKV_STAGE_DIRECT) {
     void* dptr = nullptr;
     void* sptr = nullptr;
-    BIKV_HIP(hipHostGetDevicePointer(&dptr, host_dst, 0));
-    if (has_scale) BIKV_HIP(hipHostGetDevicePointer(&sptr, host_scale_dst, 0));
-    int rc = dir == 0
-        ? bikv_gather_pages(pool, batch, dptr, image_bytes, sptr, scale_image_bytes, st->lanes[0])
-        : bikv_scatter_pages(pool, batch, dptr, image_bytes, sptr, scale_image_bytes, st->lanes[0]);
+    BIKV_HIP(hipHostGetDevicePointer(&dptr, host, 0));
+    if (has_scale) BIKV_HIP(hipHostGetDevicePointer(&sptr, host_scale, 0));
+    const int lane = (int)(st->next_launch++ % (uint64_t)st->n_buf);
+    rc = move_pages(ST_BANK_STAGER, dir, pool, batch, dptr, image_bytes, sptr, scale_image_bytes, st->lanes[lane]);
     if (rc) return rc;
-    rc = sync_and_check(st->device, st->lanes[0]);
-    if (rc) return rc;
-    if (stats) stats->n_chunks = 1;
-  } else if (mode == BIKV_STAGE_PIPELINED) {
-    const int64_t max_slots = st->chunk_bytes / T;
-    if (max_slots < 1)
-      return fail(BIKV_ERANGE, "chunk_bytes %lld is smaller than one tile (%lld bytes)",
-                  (long long)st->chunk_bytes, (long long)T);
-    // the scale tiles of a chunk ride in a second, much smaller buffer per lane
-    const int64_t scale_chunk = has_scale ? ((max_slots * S + 255) & ~int64_t(255)) : 0;
-    if (scale_chunk * st->n_buf > st->scale_ring_bytes) {
-      for (hipStream_t s : st->lanes) BIKV_HIP(hipStreamSynchronize(s));
+  } else {
+    // the scale tiles of a launch ride in a second, much smaller buffer per lane
+    const int64_t max_slots = st->lane_bytes / T;
+    const int64_t scale_lane = has_scale ? ((max_slots * S + 255) & ~int64_t(255)) : 0;
+    if (scale_lane * st->n_buf > st->scale_ring_bytes) {
+      drain_lanes(st);
       if (st->scale_ring) BIKV_HIP(hipFree(st->scale_ring));
       st->scale_ring = nullptr;
       st->scale_ring_bytes = 0;
-      BIKV_HIP(hipMalloc((void**)&st->scale_ring, (size_t)(scale_chunk * st->n_buf)));
-      st->scale_ring_bytes = scale_chunk * st->n_buf;
+      BIKV_HIP(hipMalloc((void**)&st->scale_ring, (size_t)(scale_lane * st->n_buf)));
+      st->scale_ring_bytes = scale_lane * st->n_buf;
     }
-    std::vector<Chunk> chunks;
-    plan_chunks(req_pages, n_requests, pool->n_planes, layout, max_slots, &chunks);
-    hipError_t e = hipSuccess;
-    int rc = BIKV_OK;
-    for (size_t c = 0; c < chunks.size(); ++c) {
-      const Chunk& ch = chunks[c];
-      if (ch.n_slots * T > st->chunk_bytes) {
-        rc = fail(BIKV_ERANGE, "internal: planned chunk exceeds the device chunk buffer");
-        break;
-      }
-      const int lane = (int)(c % (size_t)st->n_buf);
-      char* dev_chunk = st->ring + (int64_t)lane * st->chunk_bytes;
-      char* dev_scale = has_scale ? st->scale_ring + (int64_t)lane * scale_chunk : nullptr;
-      bikv_page_batch sub = *batch;
-      sub.page_ids = batch->page_ids + ch.first_page;
-      sub.slots = batch->slots + ch.first_page;
-      sub.slot_strides = batch->slot_strides + ch.first_page;
-      sub.n_pages = ch.n_pages;
-      sub.plane_begin = ch.plane_begin;
-      sub.plane_count = ch.plane_count;
-      sub.slot_bias = ch.first_slot;
-      char* host_chunk = static_cast<char*>(host_dst) + ch.first_slot * T;
-      char* host_scale_chunk = has_scale ? static_cast<char*>(host_scale_dst) + ch.first_slot * S : nullptr;
-      if (dir == 0) {
-        rc = bikv_gather_pages(pool, &sub, dev_chunk, ch.n_slots * T, dev_scale, ch.n_slots * S,
-                               st->lanes[lane]);
-        if (rc) break;
-        e = hipMemcpyAsync(host_chunk, dev_chunk, (size_t)(ch.n_slots * T), hipMemcpyDeviceToHost,
-                           st->lanes[lane]);
-        if (e != hipSuccess) break;
-        if (has_scale) {
-          e = hipMemcpyAsync(host_scale_chunk, dev_scale, (size_t)(ch.n_slots * S),
-                             hipMemcpyDeviceToHost, st->lanes[lane]);
-          if (e != hipSuccess) break;
-        }
-      } else {
-        e = hipMemcpyAsync(dev_chunk, host_chunk, (size_t)(ch.n_slots * T), hipMemcpyHostToDevice,
-                           st->lanes[lane]);
-        if (e != hipSuccess) break;
-        if (has_scale) {
-          e = hipMemcpyAsync(dev_scale, host_scale_chunk, (size_t)(ch.n_slots * S),
-                             hipMemcpyHostToDevice, st->lanes[lane]);
-          if (e != hipSuccess) break;
-        }
-        rc = bikv_scatter_pages(pool, &sub, dev_chunk, ch.n_slots * T, dev_scale, ch.n_slots * S,
-                                st->lanes[lane]);
-        if (rc) break;
-      }
+    LaneSet L;
+    L.n = st->n_buf;
+    L.streams = st->lanes.data();
+    L.buf = st->ring;
+    L.scale_buf = has_scale ? st->scale_ring : nullptr;
+    L.lane_bytes = st->lane_bytes;
+    L.scale_lane_bytes = has_scale ? st->scale_ring_bytes / st->n_buf : 0;
+    L.chunk_bytes = st->chunk_bytes;
+    L.next_launch = &st->next_launch;
+    L.bank = ST_BANK_STAGER;
+    rc = issue_pipelined(dir, pool, batch, req_pages, n_requests, layout, static_cast<char*>(host),
+                         static_cast<char*>(host_scale), L, &copies);
+    if (rc) {
+      drain_lanes(st);   // nothing is left in flight on an error path
+      return rc;
     }
-    // Drain every lane whatever happened, so that no work is left in flight on an error path.
-    hipError_t es = hipSuccess;
-    for (hipStream_t s : st->lanes) {
-      const hipError_t e1 = hipStreamSynchronize(s);
-      if (e1 != hipSuccess) es = e1;
-    }
-    if (rc) return rc;
-    if (e != hipSuccess) return fail_hip(e, "staging pipeline");
-    if (es != hipSuccess) return fail_hip(es, "hipStreamSynchronize(lane)");
-    rc = sync_and_check(st->device, st->lanes[0]);
-    if (rc) return rc;
-    if (stats) stats->n_chunks = (int64_t)chunks.size();
-  } else {
-    return fail(BIKV_EINVAL, "unknown staging mode %d", mode);
+  }
+  st->pending_bytes += image_bytes + scale_image_bytes;
+  st->pending_copies += mode == BIKV_STAGE_DIRECT ? 1 : copies;
+  return BIKV_OK;
+}
+
+extern "C" int bikv_stager_wait(bikv_stager* st, bikv_stage_stats* stats) {
+  if (!st) return fail(BIKV_EINVAL, "null argument");
+  BIKV_DEVICE(st->device);
+  hipError_t es = hipSuccess;
+  for (hipStream_t s : st->lanes) {
+    const hipError_t e1 = hipStreamSynchronize(s);
+    if (e1 != hipSuccess) es = e1;
   }
   const auto t1 = std::chrono::steady_clock::now();
   if (stats) {
-    stats->bytes = image_bytes + scale_image_bytes;
-    stats->wall_seconds = std::chrono::duration<double>(t1 - t0).count();
+    stats->bytes = st->pending_bytes;
+    stats->n_chunks = st->pending_copies;
+    stats->wall_seconds = st->timing ? std::chrono::duration<double>(t1 - st->t_first).count() : 0.0;
   }
-  return BIKV_OK;
+  st->pending_bytes = st->pending_copies = 0;
+  st->timing = false;
+  if (es != hipSuccess) return fail_hip(es, "hipStreamSynchronize(lane)");
+  return check_bank(st->device, ST_BANK_STAGER);
+}
+
+extern "C" int bikv_gather_to_host_async(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
+                                         const int64_t* req_pages, int64_t n_requests, int32_t layout,
+                                         void* host_dst, int64_t host_bytes, void* host_scale_dst,
+                                         int64_t host_scale_bytes, int32_t mode, void* after_stream) {
+  return stage_issue(0, st, pool, batch, req_pages, n_requests, layout, host_dst, host_bytes, host_scale_dst,
+                     host_scale_bytes, mode, after_stream);
+}
+
+extern "C" int bikv_scatter_from_host_async(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
+                                            const int64_t* req_pages, int64_t n_requests, int32_t layout,
+                                            const void* host_src, int64_t host_bytes,
+                                            const void* host_scale_src, int64_t host_scale_bytes,
+                                            int32_t mode, void* after_stream) {
+  return stage_issue(1, st, pool, batch, req_pages, n_requests, layout, const_cast<void*>(host_src), host_bytes,
+                     const_cast<void*>(host_scale_src), host_scale_bytes, mode, after_stream);
+}
+
+// The synchronous forms: whatever earlier asynchronous calls left in flight is awaited first, so that the
+// statistics and the status cover this call alone.
+static int stage_sync(int dir, bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
+                      const int64_t* req_pages, int64_t n_requests, int32_t layout, void* host,
+                      int64_t host_bytes, void* host_scale, int64_t host_scale_bytes, int32_t mode,
+                      bikv_stage_stats* stats) {
+  if (!st) return fail(BIKV_EINVAL, "null argument");
+  if (stats) { stats->bytes = 0; stats->n_chunks = 0; stats->wall_seconds = 0.0; }
+  if (st->timing) {
+    const int rc0 = bikv_stager_wait(st, nullptr);
+    if (rc0) return rc0;
+  }
+  int rc = stage_issue(dir, st, pool, batch, req_pages, n_requests, layout, host, host_bytes, host_scale,
+                       host_scale_bytes, mode, nullptr);
+  if (rc) return rc;
+  return bikv_stager_wait(st, stats);
 }
 
 extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
@@ -720,8 +947,8 @@ extern "C" int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool,
                                    int64_t host_bytes, void* host_scale_dst,
                                    int64_t host_scale_bytes, int32_t mode,
                                    bikv_stage_stats* stats) {
-  return stage_between_host(0, st, pool, batch, req_pages, n_requests, layout, host_dst, host_bytes,
-                            host_scale_dst, host_scale_bytes, mode, stats);
+  return stage_sync(0, st, pool, batch, req_pages, n_requests, layout, host_dst, host_bytes,
+                    host_scale_dst, host_scale_bytes, mode, stats);
 }
 
 extern "C" int bikv_scatter_from_host(bikv_stager* st, const bikv_pool* pool,
@@ -730,9 +957,9 @@ extern "C" int bikv_scatter_from_host(bikv_stager* st, const bikv_pool* pool,
                                       int64_t host_bytes, const void* host_scale_src,
                                       int64_t host_scale_bytes, int32_t mode,
                                       bikv_stage_stats* stats) {
-  return stage_between_host(1, st, pool, batch, req_pages, n_requests, layout,
-                            const_cast<void*>(host_src), host_bytes,
-                            const_cast<void*>(host_scale_src), host_scale_bytes, mode, stats);
+  return stage_sync(1, st, pool, batch, req_pages, n_requests, layout,
+                    const_cast<void*>(host_src), host_bytes,
+                    const_cast<void*>(host_scale_src), host_scale_bytes, mode, stats);
 }
 
 // ---- per-layer paged NHD pool and the fused layout change ------------------------------------
@@ -772,7 +999,7 @@ extern "C" int bikv_nhd_create(const bikv_nhd_desc* d, bikv_nhd** out) {
   if (((d->block_stride_elems | d->kv_stride_elems | d->token_stride_elems) * d->elem_bytes) & 15)
     return fail(BIKV_EINVAL, "strides must be multiples of 16 bytes");
   uint32_t* st = nullptr;
-  int rc = device_status(d->device, &st);
+  int rc = device_status(d->device, ST_BANK_SHARED, &st);
   if (rc) return rc;
   BIKV_DEVICE(d->device);
   void* dtab = nullptr;
@@ -835,7 +1062,7 @@ static int transpose_pages(int dir, const bikv_nhd* nhd, void* tm, int64_t tm_by
   a.n_cols = (int32_t)cols;
   a.block_tokens = nhd->block_tokens;
   a.elem_bytes = nhd->elem_bytes;
-  int rc = device_status(nhd->device, &a.status);
+  int rc = device_status(nhd->device, ST_BANK_SHARED, &a.status);
   if (rc) return rc;
   BIKV_DEVICE(nhd->device);
   hipError_t e = launch_transpose_pages(dir, a, static_cast<hipStream_t>(stream));
@@ -852,5 +1079,9 @@ extern "C" int bikv_nhd_store_token_major(const bikv_nhd* nhd, void* tm, int64_t
 extern "C" int bikv_nhd_load_token_major(const bikv_nhd* nhd, const void* tm, int64_t tm_bytes,
                                          const int64_t* block_ids, const int64_t* tm_pages,
                                          int64_t n_pages, void* stream) {
+  if (nhd) {
+    const int rc = check_unique_on_device(nhd->device, block_ids, n_pages, static_cast<hipStream_t>(stream));
+    if (rc) return rc;
+  }
   return transpose_pages(1, nhd, const_cast<void*>(tm), tm_bytes, block_ids, tm_pages, n_pages, stream);
 }

@@ -10,11 +10,29 @@ namespace bikv {
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int fail_hip(hipError_t e, const char* what);
 
-// Device-side pointer of the host-mapped status block of `device` (created on first use).
-int device_status(int device, uint32_t** dev_ptr);
+// The host-mapped status block of a device is cut into banks, one per kind of caller, so that the
+// synchronous entry points (ring producer, host stager) judge their own launches only: a flag left
+// behind by somebody's unchecked asynchronous launch cannot fail them, and bikv_check_status() from
+// another thread cannot clear a flag they are about to read.
+enum : int {
+  ST_BANK_SHARED = 0,   // the asynchronous entry points; read and cleared by bikv_check_status()
+  ST_BANK_RING = 1,     // copies issued by the ring producer
+  ST_BANK_STAGER = 2,   // launches of the host staging pipeline
+  ST_BANKS = 8
+};
 
-// Synchronises `stream`, then converts raised status slots into BIKV_EBOUNDS.
-int sync_and_check(int device, hipStream_t stream);
+// Device-side pointer of bank `bank` of the status block of `device` (created on first use).
+int device_status(int device, int bank, uint32_t** dev_ptr);
+
+// Synchronises `stream`, then converts raised status slots of `bank` into BIKV_EBOUNDS (and clears them).
+int sync_and_check(int device, int bank, hipStream_t stream);
+// The same without the synchronisation, for callers that have drained their streams themselves.
+int check_bank(int device, int bank);
+
+// The run copy behind bikv_copy_runs[_ragged], reporting into a chosen status bank.
+int copy_runs_banked(int bank, const void* src, int64_t src_bytes, void* dst, int64_t dst_bytes,
+                     const int64_t* src_off, const int64_t* dst_off, const int64_t* run_len,
+                     int64_t n_runs, int64_t run_bytes, int64_t unit_bytes, void* stream);
 
 // Makes `device` current for the scope and puts the caller's device back afterwards, so that an
 // entry point never changes the current device of the thread that called it.

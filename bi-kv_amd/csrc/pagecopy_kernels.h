@@ -63,6 +63,7 @@ struct Tuning {
   int transpose_dsplit = 0;    // slices of head_dim per tile; 0 = default (1: whole compute rows)
   int transpose_pairs = 1;     // the K/V-pair kernel where the shape allows (0 = element-wise kernel)
   int transpose_block = 512;   // lanes per workgroup of the K/V-pair kernel: 128, 256, 512, 1024
+  int debug_unique = 0;        // 1 = scattering entry points check their destination ids on the host first
 };
 Tuning& tuning();
 

@@ -36,7 +36,7 @@ __all__ = [
     "TensorDims", "producer_init", "producer_send", "producer_cleanup", "consumer_init",
     "consumer_receive", "consumer_cleanup", "producer_copy_pages", "cuda_producer_copy_pages",
     "producer_zero_copy_pages", "producer_copy_tokens", "producer_set_backpressure", "consumer_release",
-    "producer_reserve", "producer_publish",
+    "producer_reserve", "producer_publish", "producer_cancel",
 ]
 
 # dtype codes carried in the control block's first spare int (0 = float16, what a reference
@@ -115,6 +115,12 @@ def producer_publish(shape, dtype=torch.float16):
     arr = (C.c_int64 * _lib.MAX_DIM)(*shape)
     with torch.cuda.device(_producer_device()):
         _lib.check(_lib.load().bikv_producer_publish(arr, len(shape), _CODE_OF[dtype], _stream()))
+
+
+def producer_cancel():
+    """Not in the reference's module. Gives up a reserved window without publishing it. While a window
+    is reserved every other producer call raises: it would be handed the same ring bytes."""
+    _lib.check(_lib.load().bikv_producer_cancel())
 
 
 def producer_set_backpressure(enabled, timeout_ms=-1):

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define BIKV_ABI_VERSION 2
+#define BIKV_ABI_VERSION 3
 
 enum {
   BIKV_OK = 0,
@@ -71,9 +71,21 @@ int bikv_check_status(int device, void* stream, uint32_t* bits_out);
  * many bytes use one lane per 16-byte piece instead of one wave per KiB), "run_group" (1 = several
  * short runs share a row of the launch grid, default; 0 = one row per run), "transpose_lds_kib" and
  * "transpose_dsplit" (LDS tile budget and head_dim slices of the layout-change kernel),
- * "transpose_pairs" (1 = the K/V-pair kernel, default; 0 = the element-wise kernel) and "transpose_block" (its lanes per workgroup: 128, 256, 512, 1024).
+ * "transpose_pairs" (1 = the K/V-pair kernel, default; 0 = the element-wise kernel) and "transpose_block" (its lanes per workgroup: 128, 256, 512, 1024),
+ * "debug_unique" (1 = what BIKV_DEBUG_UNIQUE=1 in the environment switches on, see bikv_find_duplicate).
  * Process-wide. */
 int bikv_set_tuning(const char* key, int64_t value);
+/* Every knob back to its default. */
+void bikv_reset_tuning(void);
+
+/* Host-side check for scatters: BIKV_OK when the n ids (HOST array) are pairwise different, else
+ * BIKV_EINVAL with a message naming the repeated id and the two entries that hold it, and *dup_out
+ * (nullable) set to that id. Two runs of one launch that write the same destination race here exactly
+ * as in the reference's kernel (copy_kernel.cu:29-35: whichever block stores last wins), so callers
+ * that cannot vouch for their page lists check them with this. With BIKV_DEBUG_UNIQUE=1 in the
+ * environment, bikv_scatter_pages, bikv_scatter_from_host and bikv_nhd_load_token_major run the same
+ * check on a copy of their device ids before launching (a debugging aid: it synchronises the stream). */
+int bikv_find_duplicate(const int64_t* ids, int64_t n, int64_t* dup_out);
 
 /* --------------------------------------------------------------------------------------------
  * 1. Run copy — the reference's generic offset->offset page copy.
@@ -182,37 +194,46 @@ int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* batch,
                        void* stream);
 
 /* --------------------------------------------------------------------------------------------
- * 3. Device -> pinned-host staging pipeline.
+ * 3. Device <-> pinned-host staging pipeline.
  *
  * The reference stages KV for the transport in host tensors (kvcache.py:105-108, Worker.py:203-206)
  * that the RDMA endpoint sends from a pinned host region (onesided_rdma.h:301-337). This pipeline
- * fills such a region chunk by chunk: chunk c is gathered into the HBM buffer of stream c % n_buffers
- * and copied from there to `host_dst` with hipMemcpyAsync on the same stream, so that the copy of one
- * chunk overlaps the gather (and queued copy) of the next ones.
+ * fills such a region straight from the paged pool. A stager owns n_buffers lanes, each a HIP stream
+ * with an HBM buffer of chunks_per_launch * chunk_bytes. Launch k runs on lane k % n_buffers: one
+ * gather kernel fills the lane's buffer with the next contiguous piece of the staging image, then one
+ * hipMemcpyAsync per chunk_bytes moves it to `host_dst`, all in the lane's stream order, so the copies
+ * of one lane overlap the kernel (and queued copies) of the others.
  *
  * `req_pages` (HOST array, n_requests entries) gives the number of pages of each request; pages of
  * request r occupy batch entries [sum(req_pages[:r]), +req_pages[r]) and, in staging, a contiguous
- * block of req_pages[r]*n_planes slots whose layout is `layout`. Chunks are cut on request, plane
- * and page boundaries so that each chunk is one contiguous byte range of the staging image.
+ * block of req_pages[r]*n_planes slots whose layout is `layout`. Pieces are cut on request, plane
+ * and page boundaries so that each is one contiguous byte range of the staging image.
  * `host_dst` must be pinned (hipHostMalloc / torch pin_memory) and hold the whole staging image; the
  * scale tiles of a pool with a scale class go, slot for slot, into a second pinned image.
- * Synchronous: returns when all bytes are in host memory.
+ *
+ * Modes: BIKV_STAGE_PIPELINED as above; BIKV_STAGE_DIRECT lets the kernel store into (read from) the
+ * mapped pinned image itself, no HBM hop and no DMA engine; BIKV_STAGE_AUTO picks DIRECT for
+ * pool -> host and PIPELINED for host -> pool, the faster and steadier choice per direction on MI355X
+ * (the device -> host DMA path runs at either ~30 or ~57 GB/s there, whichever state the platform is
+ * in, while kernel stores to pinned memory hold ~55 GB/s).
  * ------------------------------------------------------------------------------------------ */
-typedef struct bikv_stager bikv_stager; /* opaque; owns n_buffers HIP streams, each with a chunk buffer */
+typedef struct bikv_stager bikv_stager; /* opaque; owns n_buffers HIP streams, each with an HBM buffer */
 
 enum { BIKV_LAYOUT_LAYER_MAJOR = 0, BIKV_LAYOUT_PAGE_MAJOR = 1 };
-enum { BIKV_STAGE_PIPELINED = 0, /* gather to HBM chunk, then hipMemcpyAsync D2H */
-       BIKV_STAGE_DIRECT = 1 };  /* kernel stores straight into the mapped pinned buffer */
+enum { BIKV_STAGE_PIPELINED = 0, BIKV_STAGE_DIRECT = 1, BIKV_STAGE_AUTO = 2 };
 
-int bikv_stager_create(int device, int64_t chunk_bytes, int32_t n_buffers, bikv_stager** out);
+int bikv_stager_create(int device, int64_t chunk_bytes, int32_t chunks_per_launch, int32_t n_buffers,
+                       bikv_stager** out);
 int bikv_stager_destroy(bikv_stager* st);
 
 typedef struct bikv_stage_stats {
-  int64_t bytes;        /* payload bytes delivered to host memory */
-  int64_t n_chunks;
-  double wall_seconds;  /* host wall time of the call */
+  int64_t bytes;        /* payload bytes delivered */
+  int64_t n_chunks;     /* host copies issued (1 per direct launch) */
+  double wall_seconds;  /* host wall time from the first enqueue to the end of the wait */
 } bikv_stage_stats;
 
+/* Synchronous: returns when all bytes are in host memory; BIKV_EBOUNDS if a page id or slot was
+ * rejected by a kernel of THIS call (the stager's launches have a status word of their own). */
 int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
                         const int64_t* req_pages, int64_t n_requests, int32_t layout,
                         void* host_dst, int64_t host_bytes,
@@ -222,9 +243,8 @@ int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool, const bikv_page_
 
 /* The receiving side: the transport has landed a staging image (same layout as above) in pinned
  * host memory (the reference holds received KV in host tensors, Worker.py:166-169, and reads a
- * pinned host pool from the GPU in kvcache.py:241-366); chunk c is copied host -> HBM chunk buffer
- * and scattered from there into the pool on lane c % n_buffers. BIKV_STAGE_DIRECT lets the scatter
- * kernel read the mapped pinned image itself. Page ids must be unique (a scatter). Synchronous. */
+ * pinned host pool from the GPU in kvcache.py:241-366); each piece is copied host -> lane buffer and
+ * scattered from there into the pool. Page ids must be unique (a scatter). Synchronous. */
 int bikv_scatter_from_host(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
                            const int64_t* req_pages, int64_t n_requests, int32_t layout,
                            const void* host_src, int64_t host_bytes,
@@ -232,7 +252,26 @@ int bikv_scatter_from_host(bikv_stager* st, const bikv_pool* pool, const bikv_pa
                            int64_t host_scale_bytes, int32_t mode,
                            bikv_stage_stats* stats /* nullable */);
 
-/* The chunk plan bikv_gather_to_host and bikv_scatter_from_host would use, without touching a GPU: writes up to `cap` chunks
+/* The same two transfers, enqueued only: the call returns as soon as kernels and copies are queued on
+ * the stager's lanes, so the calling thread can build the next request while the link is busy, and
+ * consecutive calls follow each other on the lanes without a drain in between (each request of the
+ * reference is one blocking call, kvcache.py:219-225). `after_stream` (nullable hipStream_t): work
+ * already queued there — typically the upload of the index arrays — is awaited by the lanes first.
+ * The batch's device arrays, the pool and both host images must stay valid until bikv_stager_wait
+ * returns; host images of calls in flight together must not overlap. bikv_stager_wait drains the
+ * lanes, reports everything enqueued since the previous wait in `stats` (nullable) and returns
+ * BIKV_EBOUNDS if any of those launches skipped out-of-range work. */
+int bikv_gather_to_host_async(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
+                              const int64_t* req_pages, int64_t n_requests, int32_t layout,
+                              void* host_dst, int64_t host_bytes, void* host_scale_dst,
+                              int64_t host_scale_bytes, int32_t mode, void* after_stream);
+int bikv_scatter_from_host_async(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
+                                 const int64_t* req_pages, int64_t n_requests, int32_t layout,
+                                 const void* host_src, int64_t host_bytes, const void* host_scale_src,
+                                 int64_t host_scale_bytes, int32_t mode, void* after_stream);
+int bikv_stager_wait(bikv_stager* st, bikv_stage_stats* stats);
+
+/* The pieces a stager whose lane buffer holds `max_slots_per_chunk` tiles cuts a batch into, without touching a GPU: writes up to `cap` pieces
  * as 6 int64 each (first_page, n_pages, plane_begin, plane_count, first_slot, n_slots) into `out`
  * and returns the total number of chunks (which may exceed cap), or a negative code. */
 int64_t bikv_plan_chunks(const int64_t* req_pages, int64_t n_requests, int32_t n_planes,
@@ -346,12 +385,12 @@ typedef struct bikv_tensor_dims {
 } bikv_tensor_dims;
 
 /* consumer_init (ipc_service.cpp:20-74): unlink+create shm, init semaphores, record hostname and
- * device, allocate the device ring, publish its IPC handle. */
+ * device, allocate the device ring, publish its IPC handle. A ring of 2 GiB or more is not exported
+ * (its handle stays zeroed): only a producer in the consumer's own process can use it. */
 int bikv_consumer_init(int device, const char* shm_name, size_t buffer_bytes);
 /* producer_init (ipc_service.cpp:77-110): open shm, same-host check, map the ring. A producer in
  * ANOTHER process than the consumer refuses a ring of 2 GiB or more with BIKV_ERANGE (opening an IPC
- * mapping that large has been seen not to return on some ROCm hosts); the environment variable
- * BIKV_IPC_ALLOW_LARGE=1 lifts the limit. */
+ * mapping that large has been seen not to return on some ROCm hosts). */
 int bikv_producer_init(int device, const char* shm_name);
 /* producer_cleanup / consumer_cleanup (ipc_service.cpp:171-202). Idempotent. */
 void bikv_producer_cleanup(void);
@@ -392,10 +431,15 @@ int bikv_producer_send(const void* dev_src, size_t bytes, const int64_t* shape, 
  * writes straight into the mapped buffer (copy_kernel.cu:92-113). bikv_producer_reserve applies the
  * reference's wrap rule (copy_kernel.cu:87-89) and returns the device pointer to write `bytes` at;
  * bikv_producer_publish waits for `stream`, fails with BIKV_EBOUNDS (publishing nothing) if a kernel
- * skipped work, and then does the reference's bookkeeping (copy_kernel.cu:116-128) for exactly the
- * reserved bytes. One reservation at a time. */
+ * skipped work (the reservation is then dropped), and then does the reference's bookkeeping
+ * (copy_kernel.cu:116-128) for exactly the reserved bytes. One reservation at a time: until it is
+ * published or given up with bikv_producer_cancel, every other producer call (send, copy_pages,
+ * copy_tokens, a second reserve) fails with BIKV_ESTATE, because it would be handed the same window.
+ * The caller's launches report into the status word bikv_check_status reads, so a flag left by any
+ * unchecked launch on the device since the last check also fails the publication. */
 int bikv_producer_reserve(size_t bytes, void** ptr);
 int bikv_producer_publish(const int64_t* shape, size_t ndim, int32_t dtype_code, void* stream);
+int bikv_producer_cancel(void);
 
 /* consumer_receive (ipc_service.cpp:146-168): sem_wait(sem_start) (timeout_ms < 0 = wait forever,
  * as the reference does; on timeout returns BIKV_ESTATE), then hands out a NON-OWNING pointer into

@@ -138,6 +138,70 @@ int main(void) {
     fprintf(stderr, "abi_client: bad page id not reported (bits 0x%x)\n", bits);
     return 1;
   }
+
+  /* 5. staging pipeline: two requests enqueued back to back into two pinned images, one wait; then the
+   *    first image travels back into other pages through the synchronous call */
+  {
+    enum { R0 = 3, R1 = 4 };
+    const int64_t r0_ids[R0] = {9, 3, 27};
+    const int64_t r1_ids[R1] = {14, 9, 0, 38};
+    const int64_t back_ids[R0] = {20, 21, 4};
+    void *img0_v, *img1_v;
+    CHECK(bikv_host_alloc((int64_t)N_PLANES * R0 * TILE, &img0_v));
+    CHECK(bikv_host_alloc((int64_t)N_PLANES * R1 * TILE, &img1_v));
+    uint8_t* img[2];
+    img[0] = (uint8_t*)img0_v;
+    img[1] = (uint8_t*)img1_v;
+    bikv_stager* stager = NULL;
+    CHECK(bikv_stager_create(0, 2 * TILE, 2, 2, &stager));
+    /* index arrays of both requests live side by side in the pinned index block */
+    for (int i = 0; i < R0; ++i) { ids[i] = r0_ids[i]; slots[i] = i; strides[i] = R0; }
+    for (int i = 0; i < R1; ++i) { ids[8 + i] = r1_ids[i]; slots[8 + i] = i; strides[8 + i] = R1; }
+    bikv_page_batch b0, b1;
+    memset(&b0, 0, sizeof(b0));
+    b0.page_ids = ids; b0.slots = slots; b0.slot_strides = strides; b0.n_pages = R0;
+    b0.layout_hint = BIKV_HINT_LAYER_MAJOR;
+    b1 = b0;
+    b1.page_ids = ids + 8; b1.slots = slots + 8; b1.slot_strides = strides + 8; b1.n_pages = R1;
+    const int64_t n0 = R0, n1 = R1;
+    memset(img[0], 0xA5, (size_t)N_PLANES * R0 * TILE);
+    memset(img[1], 0xA5, (size_t)N_PLANES * R1 * TILE);
+    CHECK(bikv_gather_to_host_async(stager, handle, &b0, &n0, 1, BIKV_LAYOUT_LAYER_MAJOR, img[0],
+                                    (int64_t)N_PLANES * R0 * TILE, NULL, 0, BIKV_STAGE_PIPELINED, NULL));
+    CHECK(bikv_gather_to_host_async(stager, handle, &b1, &n1, 1, BIKV_LAYOUT_LAYER_MAJOR, img[1],
+                                    (int64_t)N_PLANES * R1 * TILE, NULL, 0, BIKV_STAGE_AUTO, NULL));
+    bikv_stage_stats stats;
+    CHECK(bikv_stager_wait(stager, &stats));
+    if (stats.bytes != (int64_t)N_PLANES * (R0 + R1) * TILE) {
+      fprintf(stderr, "abi_client: stager reports %lld bytes\n", (long long)stats.bytes);
+      return 1;
+    }
+    for (int q = 0; q < N_PLANES; ++q) {
+      for (int i = 0; i < R0; ++i)
+        if (memcmp(img[0] + ((int64_t)q * R0 + i) * TILE, pool + ((int64_t)q * N_PAGES + r0_ids[i]) * TILE, TILE) != 0) {
+          fprintf(stderr, "abi_client: staged tile (request 0, plane %d, entry %d) differs\n", q, i);
+          return 1;
+        }
+      for (int i = 0; i < R1; ++i)
+        if (memcmp(img[1] + ((int64_t)q * R1 + i) * TILE, pool + ((int64_t)q * N_PAGES + r1_ids[i]) * TILE, TILE) != 0) {
+          fprintf(stderr, "abi_client: staged tile (request 1, plane %d, entry %d) differs\n", q, i);
+          return 1;
+        }
+    }
+    for (int i = 0; i < R0; ++i) ids[i] = back_ids[i];
+    CHECK(bikv_find_duplicate(ids, R0, NULL));
+    CHECK(bikv_scatter_from_host(stager, handle, &b0, &n0, 1, BIKV_LAYOUT_LAYER_MAJOR, img[0],
+                                 (int64_t)N_PLANES * R0 * TILE, NULL, 0, BIKV_STAGE_AUTO, &stats));
+    for (int q = 0; q < N_PLANES; ++q)
+      for (int i = 0; i < R0; ++i)
+        if (memcmp(pool + ((int64_t)q * N_PAGES + back_ids[i]) * TILE, img[0] + ((int64_t)q * R0 + i) * TILE, TILE) != 0) {
+          fprintf(stderr, "abi_client: tile scattered from the host (plane %d, entry %d) differs\n", q, i);
+          return 1;
+        }
+    CHECK(bikv_stager_destroy(stager));
+    CHECK(bikv_host_free(img0_v));
+    CHECK(bikv_host_free(img1_v));
+  }
   CHECK(bikv_pool_destroy(handle));
   CHECK(bikv_host_free(pool_v));
   CHECK(bikv_host_free(stg_v));

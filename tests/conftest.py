@@ -35,3 +35,13 @@ def cuda():
     if not torch.cuda.is_available():
         pytest.skip("no GPU in this process")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(autouse=True)
+def _default_tuning_after_each_test():
+    """Launch knobs are process-wide: a test that changes them (and then fails before putting them
+    back) must not leak its settings into the tests that follow."""
+    yield
+    from bikv_pagecopy import _lib
+    if _lib._lib is not None:
+        _lib.reset_tuning()

@@ -32,8 +32,13 @@ def _dims(ipc, s, total_tokens):
 
 
 def _scenario(name):
+    """The reference's scripted scenario. Its ring is 2 GiB; a ring that size is never exported over HIP
+    IPC here, so the scenario runs on a ring 4 KiB short of it, which holds the same 7 transfers and
+    wraps at the same points."""
     with open(os.path.join(GOLDEN, "reference_scenarios.json")) as f:
-        return json.load(f)[name]
+        s = json.load(f)[name]
+    s["buffer_size"] = min(s["buffer_size"], (2 << 30) - 4096)
+    return s
 
 
 def test_reference_page_ipc_scenario(ipc, cuda):
@@ -211,6 +216,12 @@ def test_cache_side_callers_from_task_info(ipc, oracle, cuda, pinned_host_pool):
     else:
         n, tokens = kvcache_calls.shared_data_batch_pages(pool_t, info, page_size, dims)
     assert (n, tokens) == (7, 7 * page_size)
+    # the per-stage timers the reference prints under SM_DEBUG (kvcache.py:155-238)
+    t = kvcache_calls.last_stage_times()
+    assert (t.pages, t.tokens, t.data_bytes) == (7, 7 * page_size, 7 * page_elems * 2)
+    assert t.index_ms > 0 and t.upload_ms > 0 and t.copy_ms > 0 and t.total_ms >= t.copy_ms
+    assert t.copy_MBps == pytest.approx(t.data_bytes / (t.copy_ms * 1e-3) / 2 ** 20)
+    assert "IPC page copy" in t.report() and "MB/s" in t.report()
     got = ipc.consumer_receive(timeout_ms=5000)
     assert tuple(got.shape) == (7 * page_size,) + dims
     pages = np.array([7, 2, 49, 4, 30, 31, 0])
@@ -396,6 +407,89 @@ def test_layered_gather_straight_into_the_ring(ipc, oracle, cuda, layout):
         ipc.consumer_receive(timeout_ms=50)
     with pytest.raises(RuntimeError, match="does not fit"):
         ipc.producer_reserve(1 << 40)
+
+
+def test_nothing_else_may_use_the_ring_while_a_window_is_reserved(ipc, cuda):
+    """Between reserve and publish the write offset belongs to the reservation: send, copy_pages,
+    copy_tokens and a second reserve would be handed the same bytes, so they are refused; the
+    reservation is published at the offset it was given, or given up with producer_cancel."""
+    print("[case] reserve / publish misuse", flush=True)
+    name = f"/bikv_test_reserve_misuse_{os.getpid()}"
+    ipc.consumer_init(0, name, 1 << 20)
+    ipc.producer_init(0, name)
+    ctrl = ipc._lib.load().bikv_producer_control().contents
+    first = torch.arange(4096, dtype=torch.float16, device=cuda)
+    ipc.producer_send(first)                                   # ring offset 0..8192
+    assert ipc.consumer_receive(timeout_ms=5000).data_ptr() == ipc._lib.load().bikv_consumer_buffer()
+    window = ipc.producer_reserve(2048)
+    window.copy_(torch.arange(2048, device=cuda).to(torch.uint8))
+    d = ipc.TensorDims()
+    d.head_size, d.num_kv_heads, d.num_layers, d.kv_pair = 8, 1, 1, 2
+    offs = torch.zeros(1, dtype=torch.int64, device=cuda)
+    for misuse in (lambda: ipc.producer_send(first),
+                   lambda: ipc.producer_copy_pages(first, offs, offs, 16, d),
+                   lambda: ipc.producer_copy_tokens(first, offs, offs, torch.ones(1, dtype=torch.int64, device=cuda), 16, d),
+                   lambda: ipc.producer_reserve(64)):
+        with pytest.raises(RuntimeError, match="reserved ring window"):
+            misuse()
+    assert int(ctrl.current_offset) == 8192                    # untouched by the refused calls
+    ipc.producer_publish((2048,), torch.uint8)
+    assert (int(ctrl.last_valid_offset), int(ctrl.current_offset), int(ctrl.data_size)) == (8192, 8192 + 2048, 2048)
+    got = ipc.consumer_receive(timeout_ms=5000)
+    assert torch.equal(got, torch.arange(2048, device=cuda).to(torch.uint8))
+    # a reservation that is given up leaves the ring where it was
+    ipc.producer_reserve(512)
+    ipc.producer_cancel()
+    ipc.producer_send(first)
+    assert int(ctrl.last_valid_offset) == 8192 + 2048
+    with pytest.raises(RuntimeError, match="nothing is reserved"):
+        ipc.producer_publish((1,), torch.uint8)
+
+
+def test_whole_page_copy_cannot_write_past_the_published_tensor(ipc, cuda):
+    """A destination offset beyond the transfer's own bytes is skipped and reported even though the ring
+    has room behind it: those bytes may belong to a tensor the consumer still holds."""
+    print("[case] copy_pages destination extent", flush=True)
+    name = f"/bikv_test_dst_extent_{os.getpid()}"
+    ipc.consumer_init(0, name, 1 << 20)
+    ipc.producer_init(0, name)
+    d = ipc.TensorDims()
+    d.head_size, d.num_kv_heads, d.num_layers, d.kv_pair = 8, 1, 1, 2
+    page_size, page_elems = 4, 4 * 16
+    pool = torch.arange(8 * page_elems, dtype=torch.float16, device=cuda)
+    so = torch.tensor([0, page_elems], dtype=torch.int64, device=cuda)
+    do = torch.tensor([0, 2 * page_elems], dtype=torch.int64, device=cuda)   # second run lands one page too far
+    with pytest.raises(RuntimeError, match="destination-range"):
+        ipc.producer_copy_pages(pool, so, do, page_size, d)
+    with pytest.raises(RuntimeError, match="timed out"):
+        ipc.consumer_receive(timeout_ms=50)
+    # a flag raised by somebody else's unchecked launch does not fail the producer's next transfer
+    import bikv_pagecopy as bk
+    bk.copy_runs(pool, torch.empty_like(pool), torch.tensor([1 << 40], dtype=torch.int64, device=cuda),
+                 torch.zeros(1, dtype=torch.int64, device=cuda), page_elems)
+    ipc.producer_copy_pages(pool, so, torch.tensor([0, page_elems], dtype=torch.int64, device=cuda), page_size, d)
+    assert tuple(ipc.consumer_receive(timeout_ms=5000).shape) == (8, 8, 1, 1, 2)
+    from bikv_pagecopy import runs
+    with pytest.raises(RuntimeError, match="source-range"):
+        runs.check(cuda)                                       # ... and is still there for its owner
+
+
+def test_a_ring_of_2_gib_is_not_exported_over_ipc(ipc, cuda):
+    """The consumer leaves the IPC handle of a ring of 2 GiB or more zeroed; a producer in the same
+    process still works on it."""
+    print("[case] 2 GiB ring stays in-process", flush=True)
+    name = f"/bikv_test_bigring_local_{os.getpid()}"
+    ipc.consumer_init(0, name, 2 << 30)
+    ctrl = ipc._lib.load().bikv_consumer_control().contents
+    assert bytes(ctrl.ipc_handle) == bytes(64)
+    ipc.producer_init(0, name)
+    t = torch.arange(1000, dtype=torch.float16, device=cuda)
+    ipc.producer_send(t)
+    assert torch.equal(ipc.consumer_receive(timeout_ms=5000), t)
+    ipc.producer_cleanup()
+    ipc.consumer_cleanup()
+    ipc.consumer_init(0, name, 1 << 20)
+    assert bytes(ipc._lib.load().bikv_consumer_control().contents.ipc_handle) != bytes(64)
 
 
 def test_packed_transfer_against_committed_digest(ipc, cuda):

@@ -680,3 +680,36 @@ def test_plain_c_program_drives_the_library(bk, cuda):
         subprocess.run(["make", "-C", here], check=True, capture_output=True, timeout=100)
     r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     assert r.returncode == 0 and "abi_client: ok" in r.stdout, (r.returncode, r.stdout, r.stderr)
+
+
+def test_duplicate_scatter_destinations_are_refused_in_debug_mode(bk, cuda):
+    """With the debug check on (BIKV_DEBUG_UNIQUE=1 or the tuning knob), a scatter whose page ids repeat
+    is refused before it launches; a gather with the same ids is legal."""
+    print("[case] duplicate destinations, debug check", flush=True)
+    pool_d = torch.zeros((2, 32, 4096), dtype=torch.uint8, device=cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    with pytest.raises(RuntimeError, match="scatter batch: destination id 5"):
+        pool.make_batch([[1, 5, 2], [5]], check_unique=True)
+    batch = pool.make_batch([[1, 5, 2], [5]])
+    staging, _ = pool.gather(batch)
+    pool.check()
+    bk.set_tuning(debug_unique=1)
+    pool.gather(batch, staging)                      # duplicates are fine in a gather
+    with pytest.raises(RuntimeError, match=r"destination id 5 is named more than once \(entries 1 and 3\)"):
+        pool.scatter(batch, staging)
+    ok = pool.make_batch([[1, 5, 2], [7]], check_unique=True)
+    pool.scatter(ok, staging)
+    pool.check()
+    bk.set_tuning(debug_unique=0)
+    # the layout change's load has the same rule for its block ids
+    layers = [torch.zeros((8 * 16, 2, 2, 64), dtype=torch.float16, device=cuda) for _ in range(2)]
+    nhd = bk.NHDPool.from_token_kv_layers(layers, 16)
+    tm = torch.zeros((2, 16, 64, 2, 2, 2), dtype=torch.float16, device=cuda)
+    ids = torch.tensor([3, 3], dtype=torch.int64, device=cuda)
+    with pytest.raises(RuntimeError, match="block ids: destination id 3"):
+        nhd.load_token_major(tm, ids, check_unique=True)
+    bk.set_tuning(debug_unique=1)
+    with pytest.raises(RuntimeError, match="destination id 3"):
+        nhd.load_token_major(tm, ids)
+    nhd.store_token_major(tm, torch.tensor([3, 4], dtype=torch.int64, device=cuda))
+    nhd.check()

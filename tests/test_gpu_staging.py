@@ -20,16 +20,19 @@ def test_gather_to_host_matches_oracle(lib, oracle, cuda, layout, mode):
     reqs = [rng.permutation(n_pages)[:m] for m in (3, 40, 1, 0, 17)]
     batch = pool.make_batch(reqs, layout)
     want = oracle.gather_layered_c(pool_h, reqs, layout).tobytes()
-    for chunk_tiles, n_buf in ((8, 2), (1, 3), (64, 1)):
-        stager = bk.HostStager(cuda, chunk_bytes=chunk_tiles * tile, n_buffers=n_buf)
+    for chunk_tiles, n_buf, group in ((8, 2, 1), (1, 3, 1), (64, 1, 1), (2, 2, 4), (1, 2, 8), (3, 3, 2)):
+        stager = bk.HostStager(cuda, chunk_bytes=chunk_tiles * tile, n_buffers=n_buf, chunks_per_launch=group)
         host = bk.pinned_empty(batch.n_slots * tile)
         host.fill_(0xA5)
         nbytes, n_chunks, sec = stager.gather_to_host(pool, batch, host, mode)
         assert nbytes == batch.n_slots * tile and sec > 0
-        assert host.numpy().tobytes() == want, (chunk_tiles, n_buf)
+        assert host.numpy().tobytes() == want, (chunk_tiles, n_buf, group)
         if mode == "pipelined":
-            plan = bk.plan_chunks(batch.req_pages, n_planes, layout, chunk_tiles)
-            assert n_chunks == len(plan)
+            # one launch per piece of the plan, one host copy per chunk_bytes of a piece
+            plan = bk.plan_chunks(batch.req_pages, n_planes, layout, chunk_tiles * group)
+            assert n_chunks == sum(-(-int(p[5]) // chunk_tiles) for p in plan)
+        else:
+            assert n_chunks == 1
         stager.close()
 
 
@@ -49,8 +52,8 @@ def test_gather_to_host_moves_scales_with_the_payload(lib, oracle, cuda, layout,
     batch = pool.make_batch(reqs, layout)
     want = oracle.gather_layered_c(pool_h, reqs, layout).tobytes()
     swant = oracle.gather_layered_c(scale_h, reqs, layout).tobytes()
-    for chunk_tiles in (4, 1, 64):
-        stager = bk.HostStager(cuda, chunk_bytes=chunk_tiles * tile, n_buffers=2)
+    for chunk_tiles, group in ((4, 1), (1, 1), (64, 1), (2, 4)):
+        stager = bk.HostStager(cuda, chunk_bytes=chunk_tiles * tile, n_buffers=2, chunks_per_launch=group)
         host = bk.pinned_empty(batch.n_slots * tile).fill_(0xA5)
         shost = bk.pinned_empty(batch.n_slots * stile).fill_(0xA5)
         nbytes, _, _ = stager.gather_to_host(pool, batch, host, mode, host_scale=shost)
@@ -72,11 +75,11 @@ def test_gather_to_host_argument_checks(lib, cuda):
         stager.gather_to_host(pool, batch, torch.empty(batch.n_slots * 4096, dtype=torch.uint8))
     with pytest.raises(RuntimeError, match="staging image needs"):
         stager.gather_to_host(pool, batch, bk.pinned_empty(4096))
-    tiny = bk.HostStager(cuda, chunk_bytes=4096, n_buffers=1)
+    tiny = bk.HostStager(cuda, chunk_bytes=4096, n_buffers=1, chunks_per_launch=1)
     big_d = torch.zeros((1, 4, 8192), dtype=torch.uint8, device=cuda)
     big = bk.PagedKVPool.from_stacked(big_d, plane_dims=1)
     with pytest.raises(RuntimeError, match="smaller than one tile"):
-        tiny.gather_to_host(big, big.make_batch([[0]]), bk.pinned_empty(8192))
+        tiny.gather_to_host(big, big.make_batch([[0]]), bk.pinned_empty(8192), "pipelined")
     with pytest.raises(RuntimeError):
         bk.HostStager(cuda, chunk_bytes=16, n_buffers=2)
 
@@ -112,20 +115,20 @@ def test_scatter_from_host_matches_oracle(lib, oracle, cuda, layout, mode):
     oracle.scatter_layered_c(want, reqs, image, layout)
     swant = scale_h.copy()
     oracle.scatter_layered_c(swant, reqs, simage, layout)
-    for chunk_tiles, n_buf in ((8, 2), (1, 3), (64, 1)):
+    for chunk_tiles, n_buf, group in ((8, 2, 1), (1, 3, 1), (64, 1, 1), (2, 2, 4)):
         pool_d = torch.from_numpy(pool_h).to(cuda)
         scale_d = torch.from_numpy(scale_h).to(cuda)
         pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1, scale=scale_d)
         batch = pool.make_batch(reqs, layout)
-        stager = bk.HostStager(cuda, chunk_bytes=chunk_tiles * tile, n_buffers=n_buf)
+        stager = bk.HostStager(cuda, chunk_bytes=chunk_tiles * tile, n_buffers=n_buf, chunks_per_launch=group)
         host = bk.pinned_empty(n_slots * tile)
         host.copy_(torch.from_numpy(image))
         shost = bk.pinned_empty(n_slots * stile)
         shost.copy_(torch.from_numpy(simage))
         nbytes, n_chunks, sec = stager.scatter_from_host(pool, batch, host, mode, host_scale=shost)
         assert nbytes == n_slots * (tile + stile) and sec > 0
-        assert np.array_equal(pool_d.cpu().numpy(), want), (chunk_tiles, n_buf)
-        assert np.array_equal(scale_d.cpu().numpy(), swant), (chunk_tiles, n_buf)
+        assert np.array_equal(pool_d.cpu().numpy(), want), (chunk_tiles, n_buf, group)
+        assert np.array_equal(scale_d.cpu().numpy(), swant), (chunk_tiles, n_buf, group)
         # and back: the gather of the same pages returns the image
         back = bk.pinned_empty(n_slots * tile).fill_(0xA5)
         sback = bk.pinned_empty(n_slots * stile).fill_(0xA5)
@@ -151,7 +154,7 @@ def test_scatter_from_host_argument_checks(lib, cuda):
     bad.index[0, 1] = 99
     host = bk.pinned_empty(batch.n_slots * 4096).fill_(7)
     with pytest.raises(RuntimeError, match="page-id"):
-        stager.scatter_from_host(pool, bad, host)
+        stager.scatter_from_host(pool, bad, host, "pipelined")
     got = pool_d.cpu()
     assert bool((got[:, 1] == 7).all()) and bool((got[:, 3] == 7).all()) and bool((got[:, 2] == 0).all())
 
@@ -166,3 +169,87 @@ def test_measure_h2d_runs(lib, cuda):
         dev.zero_()
         sec = bk.measure_h2d(cuda, dev, host, chunk)
         assert sec > 0 and torch.equal(dev.cpu(), host)
+
+
+@pytest.mark.parametrize("mode", ["pipelined", "direct", "auto"])
+def test_requests_enqueued_back_to_back_share_the_lanes(lib, oracle, cuda, mode):
+    """Enqueue-only form: several requests go onto the lanes without a drain in between, each into its
+    own part of the pinned region; one wait() completes them all. Then the same images travel back into
+    other pages, also enqueued back to back."""
+    import bikv_pagecopy as bk
+    print(f"[case] asynchronous staging {mode}", flush=True)
+    rng = np.random.default_rng(53)
+    n_planes, n_pages, tile = 8, 120, 16384
+    pool_h = rng.integers(0, 256, size=(n_planes, n_pages, tile), dtype=np.uint8)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    perm = rng.permutation(n_pages)
+    sizes = [7, 1, 19, 4, 11]
+    cuts = np.cumsum(sizes)
+    reqs = [np.ascontiguousarray(a) for a in np.split(perm[:cuts[-1]], cuts[:-1])]
+    stager = bk.HostStager(cuda, chunk_bytes=2 * tile, n_buffers=2, chunks_per_launch=2)
+    images = [bk.pinned_empty(len(r) * n_planes * tile).fill_(0xA5) for r in reqs]
+    batches = [pool.make_batch([r], "layer_major") for r in reqs]       # uploads queue on the current stream
+    for b, img in zip(batches, images):
+        stager.gather_to_host_async(pool, b, img, mode)
+    nbytes, copies, sec = stager.wait()
+    assert nbytes == sum(img.numel() for img in images) and copies >= len(reqs) and sec > 0
+    for r, img in zip(reqs, images):
+        assert img.numpy().tobytes() == oracle.gather_layered_c(pool_h, [r]).tobytes()
+    # back into fresh pages
+    fresh = perm[cuts[-1]: 2 * cuts[-1]]
+    dst = [np.ascontiguousarray(a) for a in np.split(fresh, cuts[:-1])]
+    want = pool_h.copy()
+    for d, img in zip(dst, images):
+        oracle.scatter_layered_c(want, [d], img.numpy())
+    sbatches = [pool.make_batch([d], "layer_major") for d in dst]
+    for b, img in zip(sbatches, images):
+        stager.scatter_from_host_async(pool, b, img, mode)
+    stager.wait()
+    assert np.array_equal(pool_d.cpu().numpy(), want)
+    # a rejected id in one of several enqueued requests is reported by the wait, the others land
+    bad = pool.make_batch([dst[0]], "layer_major")
+    bad.index[0, 0] = n_pages + 5
+    stager.gather_to_host_async(pool, batches[1], images[1].fill_(0), mode)
+    stager.gather_to_host_async(pool, bad, images[0], mode)
+    with pytest.raises(RuntimeError, match="page-id"):
+        stager.wait()
+    assert images[1].numpy().tobytes() == oracle.gather_layered_c(pool_h, [reqs[1]]).tobytes()
+    assert stager.wait()[0] == 0            # nothing pending, status cleared
+    stager.close()
+
+
+@pytest.mark.parametrize("chunk_mib,lanes,group", [(4, 2, 4), (8, 2, 4), (16, 2, 2), (4, 4, 1), (16, 4, 1)])
+def test_llama3_8b_requests_staged_in_4_to_16_mib_chunks(lib, oracle, cuda, chunk_mib, lanes, group):
+    """The Llama-3-8B-shaped workload itself: 64 KiB tiles x 64 planes (4 MiB per logical page), the
+    leading requests of its log-normal stream, device -> pinned host in 4-16 MiB chunks and back, both
+    modes, against the oracle's staging image."""
+    import bikv_pagecopy as bk
+    from bikv_pagecopy import workloads as w
+    shape = w.SHAPES["llama3_8b"].scaled(160)                 # 160 pages x 4 MiB = 640 MiB pool
+    print(f"[case] llama3_8b staging {chunk_mib} MiB x {lanes} lanes x {group} per launch", flush=True)
+    assert shape.tile_bytes == 65536 and shape.n_planes == 64
+    # the leading requests of the real stream (its length distribution, ids of this pool), each cut to at
+    # most 30 pages = 120 MiB of staging image
+    reqs = [r[:30] for r in w.named("llama3_8b", shape)["gather"][:5]]
+    assert len(reqs) == 5 and len({len(r) for r in reqs}) > 1
+    rng = np.random.default_rng(59)
+    pool_h = rng.integers(0, 256, size=(shape.n_planes, shape.n_pages, shape.tile_bytes), dtype=np.uint8)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    stager = bk.HostStager(cuda, chunk_bytes=chunk_mib << 20, n_buffers=lanes, chunks_per_launch=group)
+    for mode in ("pipelined", "direct"):
+        for r in reqs:
+            b = pool.make_batch([r], "layer_major")
+            host = bk.pinned_empty(b.n_slots * shape.tile_bytes).fill_(0xA5)
+            stager.gather_to_host(pool, b, host, mode)
+            want = oracle.gather_layered_c(pool_h, [r])
+            assert host.numpy().tobytes() == want.tobytes(), (mode, len(r))
+    # and the way back: the last image into the pages next to the ones it came from
+    shifted = (np.asarray(reqs[-1]) + 1) % shape.n_pages
+    sb = pool.make_batch([shifted], "layer_major", check_unique=True)
+    stager.scatter_from_host(pool, sb, host, "pipelined")
+    oracle.scatter_layered_c(pool_h, [shifted], host.numpy())
+    assert np.array_equal(pool_d.cpu().numpy(), pool_h)
+    stager.close()
+    pool.close()

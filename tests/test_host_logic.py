@@ -326,9 +326,59 @@ def test_producer_refuses_to_map_a_ring_of_2_gib_from_another_process(lib):
     with open(path, "wb") as f:
         f.write(bytes(ctrl))
     try:
-        os.environ.pop("BIKV_IPC_ALLOW_LARGE", None)
         rc = lib.bikv_producer_init(0, name.encode())
         assert rc == -6 and b"2 GiB" in lib.bikv_last_error()
         assert not lib.bikv_producer_control()
     finally:
         os.unlink(path)
+
+
+def test_find_duplicate_names_the_first_repeated_destination(lib):
+    """Host-side check for scatters (duplicate destinations race on the device, as they do in the
+    reference's kernel, copy_kernel.cu:29-35), against a brute-force statement."""
+    import numpy as np
+    import bikv_pagecopy as bk
+    from bikv_pagecopy import _lib
+    bk.require_unique([])
+    bk.require_unique([5])
+    bk.require_unique(np.random.default_rng(0).permutation(1000))
+    with pytest.raises(RuntimeError, match=r"id 7 is named more than once \(entries 1 and 4\)"):
+        bk.require_unique([3, 7, 9, 2, 7, 3])
+    with pytest.raises(RuntimeError, match=r"id -2 is named more than once \(entries 0 and 1\)"):
+        bk.require_unique([-2, -2])
+    rng = np.random.default_rng(1)
+    for _ in range(200):
+        ids = rng.integers(0, 40, size=rng.integers(0, 30)).astype(np.int64)
+        seen, want = {}, None
+        for i, v in enumerate(ids.tolist()):
+            if v in seen:
+                want = (v, seen[v], i)
+                break
+            seen.setdefault(v, i)
+        dup = C.c_int64(-1)
+        rc = lib.bikv_find_duplicate(ids.ctypes.data_as(C.POINTER(C.c_int64)), len(ids), C.byref(dup))
+        if want is None:
+            assert rc == _lib.OK
+        else:
+            assert rc == _lib.EINVAL and dup.value == want[0]
+            assert f"(entries {want[1]} and {want[2]})".encode() in lib.bikv_last_error()
+    assert lib.bikv_find_duplicate(None, 3, None) == _lib.EINVAL
+
+
+def test_make_batch_can_refuse_duplicate_scatter_destinations():
+    """build_index is pure host logic; the check sits in front of it in PagedKVPool.make_batch."""
+    import numpy as np
+    import bikv_pagecopy as bk
+    from bikv_pagecopy.pool import build_index
+    idx, _ = build_index([np.array([4, 9]), np.array([1, 9, 3])], 2, "layer_major")
+    with pytest.raises(RuntimeError, match="scatter batch: destination id 9"):
+        bk.require_unique(idx[0], "scatter batch")
+
+
+def test_stage_times_report_has_the_reference_stages():
+    from bikv_pagecopy import kvcache_calls as k
+    t = k.StageTimes(pages=3, tokens=40, data_bytes=1 << 20, index_ms=0.1, upload_ms=0.2, copy_ms=0.5, total_ms=1.0)
+    assert t.copy_MBps == pytest.approx(2000.0)
+    text = t.report()
+    for word in ("offset tables", "upload", "IPC page copy", "2000.00 MB/s", "total: 1.00 ms", "0.0250 ms per token"):
+        assert word in text
