@@ -8,9 +8,9 @@ from .nhd import NHDPool
 from .offsets import RunIndexPool, build_run_offsets
 from .pool import LAYER_MAJOR, PAGE_MAJOR, PageBatch, PagedKVPool, build_index
 from .runs import copy_runs
-from .staging import HostStager, measure_d2h, measure_h2d, pinned_empty, plan_chunks
+from .staging import HostStager, gather_to_host_noalloc, measure_d2h, measure_h2d, pinned_empty, plan_chunks
 
 __all__ = [
     "load", "set_tuning", "reset_tuning", "require_unique", "build_run_offsets", "RunIndexPool", "LAYER_MAJOR", "PAGE_MAJOR", "PageBatch", "PagedKVPool",
-    "build_index", "copy_runs", "NHDPool", "HostStager", "measure_d2h", "measure_h2d", "pinned_empty", "plan_chunks",
+    "build_index", "copy_runs", "NHDPool", "HostStager", "gather_to_host_noalloc", "measure_d2h", "measure_h2d", "pinned_empty", "plan_chunks",
 ]

@@ -106,6 +106,7 @@ class SharedControl(C.Structure):
 _SIGNATURES = {
     "bikv_abi_version": (C.c_int, []),
     "bikv_last_error": (C.c_char_p, []),
+    "bikv_init": (C.c_int, [C.c_int]),
     "bikv_check_status": (C.c_int, [C.c_int, C.c_void_p, C.POINTER(C.c_uint32)]),
     "bikv_set_tuning": (C.c_int, [C.c_char_p, C.c_int64]),
     "bikv_reset_tuning": (None, []),
@@ -138,6 +139,8 @@ _SIGNATURES = {
     "bikv_scatter_from_host": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PageBatchDesc),
                                          C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_void_p,
                                          C.c_int64, C.c_void_p, C.c_int64, C.c_int32, C.POINTER(StageStats)]),
+    "bikv_gather_to_host_noalloc": (C.c_int, [C.c_void_p, C.POINTER(PageBatchDesc), C.POINTER(C.c_int64), C.c_int64,
+                                              C.c_int32, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]),
     "bikv_nhd_create": (C.c_int, [C.POINTER(NHDDesc), C.POINTER(C.c_void_p)]),
     "bikv_nhd_destroy": (C.c_int, [C.c_void_p]),
     "bikv_nhd_load_token_major": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,

@@ -123,6 +123,31 @@ class HostStager:
             pass
 
 
+def gather_to_host_noalloc(pool: PagedKVPool, batch: PageBatch, host: torch.Tensor, host_scale: torch.Tensor = None):
+    """bikv_gather_to_host_noalloc: the pipelined pool -> pinned host transfer for callers that cannot
+    allocate. One lane, the current stream, staged through a static scratch array inside the library
+    (tiles of at most 16 MiB, scale tiles of at most 64 KiB). Enqueue only: synchronise the stream (or
+    call pool.check()) before reading `host`. Calls that overlap in time on one GPU race on the scratch."""
+    for t in (host, host_scale):
+        if t is None:
+            continue
+        if t.is_cuda or not t.is_pinned():
+            raise RuntimeError("CPU data must be pinned memory")
+        if not t.is_contiguous():
+            raise RuntimeError("host staging buffer must be contiguous")
+    if pool.scale_tile_bytes and host_scale is None:
+        raise RuntimeError("pool has scales: a pinned host_scale buffer is required")
+    d = batch.desc()
+    rp = batch.req_pages.ctypes.data_as(C.POINTER(C.c_int64))
+    with torch.cuda.device(pool.device):
+        _lib.check(_lib.load().bikv_gather_to_host_noalloc(
+            pool._h, C.byref(d), rp, len(batch.req_pages), _LAYOUT_CODE[batch.layout],
+            host.data_ptr(), host.numel() * host.element_size(),
+            host_scale.data_ptr() if host_scale is not None else None,
+            host_scale.numel() * host_scale.element_size() if host_scale is not None else 0,
+            C.c_void_p(torch.cuda.current_stream(pool.device).cuda_stream)))
+
+
 def plan_chunks(req_pages, n_planes: int, layout: str, max_slots: int) -> np.ndarray:
     """The chunk plan of the pipelined mode as an [n_chunks, 6] int64 array:
     (first_page, n_pages, plane_begin, plane_count, first_slot, n_slots). Pure host logic."""

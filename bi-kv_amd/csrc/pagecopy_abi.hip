@@ -31,10 +31,22 @@ int fail_hip(hipError_t e, const char* what) {
   return fail(BIKV_EHIP, "%s failed: %s", what, hipGetErrorString(e));
 }
 
-// ---- per-device context: the host-mapped status block -------------------------------------
+// ---- scratch of the allocation-free entry point ---------------------------------------------
+// bikv_gather_to_host_noalloc stages through this array instead of a stager's hipMalloc'd buffers:
+// kScratchPayload bytes for payload tiles followed by kScratchScale bytes for scale tiles. Every GPU the
+// library runs on holds its own copy (16 MiB + 64 KiB) until the process ends. In host code the name is
+// only a handle: the device address is taken once per device with hipGetSymbolAddress (device_status
+// below) and that pointer is what kernels and copies are given.
+constexpr int64_t kScratchPayload = int64_t(16) << 20;
+constexpr int64_t kScratchScale = int64_t(64) << 10;
+constexpr int64_t kScratchCopy = int64_t(8) << 20;     // bytes per hipMemcpyAsync out of the scratch
+static __device__ __align__(256) unsigned char scratch[kScratchPayload + kScratchScale];
+
+// ---- per-device context: the host-mapped status block and the scratch address ---------------
 struct DevCtx {
   uint32_t* status_host = nullptr;  // pinned, mapped
   uint32_t* status_dev = nullptr;   // the same memory as the device sees it
+  char* scratch_dev = nullptr;      // this device's copy of `scratch`
 };
 static std::mutex g_ctx_mu;
 static DevCtx g_ctx[64];
@@ -55,11 +67,27 @@ int device_status(int device, int bank, uint32_t** dev_ptr) {
       (void)hipHostFree(h);
       return fail_hip(e, "hipHostGetDevicePointer");
     }
+    // this device's address of the scratch array (the device is current here)
+    void* sp = nullptr;
+    e = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !sp) {
+      (void)hipHostFree(h);
+      return fail_hip(e != hipSuccess ? e : hipErrorInvalidSymbol, "hipGetSymbolAddress(scratch)");
+    }
     c.status_host = static_cast<uint32_t*>(h);
     c.status_dev = static_cast<uint32_t*>(d);
+    c.scratch_dev = static_cast<char*>(sp);
   }
   *dev_ptr = c.status_dev + bank * ST_SLOTS;
   return BIKV_OK;
+}
+
+// The scratch address of a device whose context already exists; never creates one (the allocation-free
+// entry point must not allocate, and creating a context allocates the status block).
+static char* scratch_of(int device) {
+  if (device < 0 || device >= 64) return nullptr;
+  std::lock_guard<std::mutex> lk(g_ctx_mu);
+  return g_ctx[device].status_host ? g_ctx[device].scratch_dev : nullptr;
 }
 
 static uint32_t take_status(int device, int bank) {
@@ -121,6 +149,11 @@ struct bikv_pool {
 };
 
 extern "C" int bikv_abi_version(void) { return BIKV_ABI_VERSION; }
+
+extern "C" int bikv_init(int device) {
+  uint32_t* st = nullptr;
+  return device_status(device, ST_BANK_SHARED, &st);
+}
 extern "C" const char* bikv_last_error(void) { return g_err; }
 
 extern "C" int bikv_check_status(int device, void* stream, uint32_t* bits_out) {
@@ -960,6 +993,45 @@ extern "C" int bikv_scatter_from_host(bikv_stager* st, const bikv_pool* pool,
   return stage_sync(1, st, pool, batch, req_pages, n_requests, layout,
                     const_cast<void*>(host_src), host_bytes,
                     const_cast<void*>(host_scale_src), host_scale_bytes, mode, stats);
+}
+
+// The allocation-free form of bikv_gather_to_host: the same pipeline on ONE lane — the caller's stream —
+// whose buffer is this device's `scratch` array. Enqueue only. Nothing here allocates or frees: the
+// device context (status block, scratch address) was set up by bikv_init / bikv_pool_create, the planner
+// is an iterator, errors go to a thread-local buffer.
+extern "C" int bikv_gather_to_host_noalloc(const bikv_pool* pool, const bikv_page_batch* batch,
+                                           const int64_t* req_pages, int64_t n_requests, int32_t layout,
+                                           void* host_dst, int64_t host_bytes, void* host_scale_dst,
+                                           int64_t host_scale_bytes, void* stream) {
+  int64_t total_pages = 0;
+  int rc = validate_stage_args(pool, batch, req_pages, n_requests, layout, host_dst, host_bytes,
+                               host_scale_dst, host_scale_bytes, &total_pages);
+  if (rc) return rc;
+  if (pool->tile_bytes > kScratchPayload)
+    return fail(BIKV_ERANGE, "tile of %lld bytes exceeds the %lld-byte scratch of the allocation-free entry point",
+                (long long)pool->tile_bytes, (long long)kScratchPayload);
+  if (pool->scale_tile_bytes > kScratchScale)
+    return fail(BIKV_ERANGE, "scale tile of %lld bytes exceeds the %lld-byte scale scratch of the allocation-free entry point",
+                (long long)pool->scale_tile_bytes, (long long)kScratchScale);
+  char* base = scratch_of(pool->device);
+  if (!base) return fail(BIKV_ESTATE, "device %d is not set up (bikv_init)", pool->device);
+  if (total_pages == 0) return BIKV_OK;
+  BIKV_DEVICE(pool->device);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint64_t launches = 0;
+  int64_t copies = 0;
+  LaneSet L;
+  L.n = 1;
+  L.streams = &s;
+  L.buf = base;
+  L.scale_buf = pool->scale_tile_bytes > 0 ? base + kScratchPayload : nullptr;
+  L.lane_bytes = kScratchPayload;
+  L.scale_lane_bytes = pool->scale_tile_bytes > 0 ? kScratchScale : 0;
+  L.chunk_bytes = kScratchCopy;
+  L.next_launch = &launches;
+  L.bank = ST_BANK_SHARED;
+  return issue_pipelined(0, pool, batch, req_pages, n_requests, layout, static_cast<char*>(host_dst),
+                         static_cast<char*>(host_scale_dst), L, &copies);
 }
 
 // ---- per-layer paged NHD pool and the fused layout change ------------------------------------

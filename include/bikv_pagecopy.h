@@ -50,6 +50,11 @@ enum {
 int bikv_abi_version(void);
 const char* bikv_last_error(void);
 
+/* Sets up the library's per-device state on `device` (a small host-mapped status block, and the device
+ * address of the library's static scratch array). Idempotent. Every handle-creating call does the same
+ * on first use of a device; callers that must not allocate later call this up front. */
+int bikv_init(int device);
+
 /* Reads and clears the status word of `device` after synchronising `stream`.
  * Returns BIKV_OK, or BIKV_EBOUNDS with *bits_out (nullable) holding the BIKV_ST_* bits.
  * There is ONE status word per device, shared by every stream and host thread: a check reports (and
@@ -270,6 +275,25 @@ int bikv_scatter_from_host_async(bikv_stager* st, const bikv_pool* pool, const b
                                  const void* host_src, int64_t host_bytes, const void* host_scale_src,
                                  int64_t host_scale_bytes, int32_t mode, void* after_stream);
 int bikv_stager_wait(bikv_stager* st, bikv_stage_stats* stats);
+
+/* bikv_gather_to_host for callers that cannot allocate: code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc. It has no counterpart in the reference. The pipeline is the
+ * pipelined mode of bikv_gather_to_host on ONE lane, the caller's `stream`: gather kernel into a buffer,
+ * hipMemcpyAsync of at most 8 MiB each to `host_dst`, piece after piece in stream order. The buffer is
+ * not a stager's: it is a static array inside the library's device code, 16 MiB for payload tiles plus
+ * 64 KiB for scale tiles, which every GPU the library runs on holds until the process ends. The call
+ * allocates and frees nothing (no hipMalloc, no stream or event creation) and only enqueues: it returns
+ * when kernels and copies are queued on `stream`; rejected page ids / slots are reported by
+ * bikv_check_status like those of bikv_gather_pages.
+ * Limits: tile_bytes <= 16 MiB and scale_tile_bytes <= 64 KiB (BIKV_ERANGE otherwise); the device must
+ * have been set up by bikv_init or any bikv_pool_create (BIKV_ESTATE otherwise — a valid pool implies it).
+ * All calls on one GPU share that GPU's array: calls whose work overlaps in time (two streams, or two
+ * threads) race on it and deliver wrong bytes; issue them on one stream, or wait between them. */
+int bikv_gather_to_host_noalloc(const bikv_pool* pool, const bikv_page_batch* batch,
+                                const int64_t* req_pages, int64_t n_requests, int32_t layout,
+                                void* host_dst, int64_t host_bytes,
+                                void* host_scale_dst /* pinned; NULL iff the pool has no scale class */,
+                                int64_t host_scale_bytes, void* stream);
 
 /* The pieces a stager whose lane buffer holds `max_slots_per_chunk` tiles cuts a batch into, without touching a GPU: writes up to `cap` pieces
  * as 6 int64 each (first_page, n_pages, plane_begin, plane_count, first_slot, n_slots) into `out`
