@@ -40,8 +40,11 @@ HBM_PEAK_GBPS = 8000.0
 # WRITE_SIZE runs of this file, each scaled by the same counter's reading for the plain-copy
 # calibration launch below (summaries under profiles/). None = not measured for that workload.
 MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9949, "scatter": 1.0003},
+                          "qwen2_1p5b": {"gather": 1.0009},
+                          "llama3_8b": {"gather": 0.9966},
+                          "llama3_70b_fp8": {"gather": 1.0142, "scatter": 1.0001},
                           "qwen2_7b_token_major": {"gather": 0.9997, "scatter": 1.0002},
-                          "layout_change": {"load": 1.0035, "store": 1.0029}}
+                          "layout_change": {"load": 1.0034, "store": 1.0025}}
 
 
 def parse_args():
@@ -729,18 +732,20 @@ def run_token_major(args, bk, workloads, dev):
     }
 
 
-def run_layout_change(args, bk, dev):
+def run_layout_change(args, bk, dev, blocks=None, sort=True):
     """Received token-major pages -> the Worker's per-layer paged pool and back, at the reference's own
     shapes: token_shape (128, 2, 28, 2) fp16 (Model/qwen2.py:512-522), 28 layer tensors of
-    [10240*16, 2, 2, 128] (Worker.py:69-78), 4096 pages of 16 tokens per step and direction."""
+    [blocks*16, 2, 2, 128] (Worker.py:69-78: 10240 blocks), 4096 pages of 16 tokens per step and
+    direction, random blocks. The page lists are built on the host and handed over through
+    NHDPool.page_list: the load walks its list in ascending block order (`sort`), the store in the order
+    given (sorting helps the direction whose scattered side is written and hurts the other)."""
     import numpy as np
     import torch
     from oracle import pagecopy_oracle as oracle
 
-    P, D, H, L, blocks, n_pages = 16, 128, 2, 28, 10240, 4096
-    if args.pool_pages:
-        blocks = args.pool_pages
-        n_pages = min(n_pages, blocks)
+    P, D, H, L, n_pages = 16, 128, 2, 28, 4096
+    blocks = blocks or args.pool_pages or 10240
+    n_pages = min(n_pages, blocks)
     layers = [torch.empty((blocks * P, 2, H, D), dtype=torch.float16, device=dev) for _ in range(L)]
     for t in layers:
         fill_random_bytes(t)
@@ -749,17 +754,18 @@ def run_layout_change(args, bk, dev):
     fill_random_bytes(tm)
     tm_out = torch.empty_like(tm)
     rng = np.random.default_rng(6)
-    ids_h = rng.permutation(blocks)[:n_pages].astype(np.int64)
-    ids = torch.from_numpy(ids_h).to(dev)
+    ids_h = rng.permutation(blocks)[:n_pages].astype(np.int64)       # page i of tm <-> block ids_h[i]
+    ids, pages = pool.page_list(ids_h, sort=sort, check_unique=True)
+    ids_s, pages_s = pool.page_list(ids_h, sort=False)
     alg = 2 * tm.numel() * 2                       # bytes read + written per launch
 
     def step(ev=None):
         if ev:
             ev[0].record()
-        pool.load_token_major(tm, ids)             # received pages -> pool blocks
+        pool.load_token_major(tm, ids, pages)      # received pages -> pool blocks
         if ev:
             ev[1].record()
-        pool.store_token_major(tm_out, ids)        # the same blocks -> pages to send
+        pool.store_token_major(tm_out, ids_s, pages_s)  # the same blocks -> pages to send
         if ev:
             ev[2].record()
 
@@ -776,7 +782,7 @@ def run_layout_change(args, bk, dev):
     pool.check()
     if not torch.equal(tm_out.view(torch.int16), tm.view(torch.int16)):
         raise SystemExit("bench: store(load(x)) != x")
-    # a sample of pages against the CPU oracle
+    # a sample of pages against the CPU oracle (np.zeros is lazily backed: only the sampled blocks are touched)
     sample = np.arange(0, n_pages, max(1, n_pages // 8))[:8]
     lay_h = [np.zeros((blocks * P, 2, H, D), dtype=np.uint16) for _ in range(L)]
     tm_h = tm[torch.from_numpy(sample).to(dev)].cpu().view(torch.int16).numpy().view(np.uint16)
@@ -786,28 +792,36 @@ def run_layout_change(args, bk, dev):
             got = layers[l][b * P:(b + 1) * P].cpu().view(torch.int16).numpy().view(np.uint16)
             if got.tobytes() != lay_h[l][b * P:(b + 1) * P].tobytes():
                 raise SystemExit("bench: layout change differs from the oracle")
-    l_ms = [e[0].elapsed_time(e[1]) for e in evs]
-    s_ms = [e[1].elapsed_time(e[2]) for e in evs]
-    slow_is_load = np.mean(l_ms) >= np.mean(s_ms)
-    ms_dom = float(np.mean(l_ms if slow_is_load else s_ms))
-    return {
+    l_stat = launch_stats([e[0].elapsed_time(e[1]) for e in evs], alg)
+    s_stat = launch_stats([e[1].elapsed_time(e[2]) for e in evs], alg)
+    slow_is_load = l_stat["avg_ms"] >= s_stat["avg_ms"]
+    dom = l_stat if slow_is_load else s_stat
+    at_reference_shape = blocks == 10240 and sort
+    out = {
         "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
         "value": round(2 * alg / (wall / args.steps) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "u16", "data": "synthetic",
         "config": {"workload": f"layout_change: token-major pages <-> {L} layer tensors [{blocks}*{P}, 2, {H}, {D}] fp16, "
-                               f"{n_pages} pages of {P} tokens loaded then stored per step"},
+                               f"{n_pages} pages of {P} tokens loaded then stored per step, random blocks; the load walks "
+                               f"them in {'ascending block order' if sort else 'the order given'}, the store in the order given",
+                   "pool_GB": round(L * blocks * P * 2 * H * D * 2 / 1e9, 2)},
+        "timed_region_s": round(wall, 3),
         "pct_of_hbm_peak": round(100 * 2 * alg / (wall / args.steps) / 1e9 / HBM_PEAK_GBPS, 2),
         "pages_per_s": round(2 * n_pages / (wall / args.steps), 1), "bit_exact": True,
         "roofline": {"bound": "hbm", "kernel": f"bikv::transpose_pairs_kernel<{1 if slow_is_load else 0}, 2, 512>",
-                     "achieved": round(alg / (ms_dom * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(alg / (ms_dom * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
                      "traffic": (int(alg * MEASURED_TRAFFIC_RATIO["layout_change"]["load" if slow_is_load else "store"])
-                                 if not args.pool_pages else None),
-                     "alg_bytes_per_launch": alg, "avg_launch_ms": round(ms_dom, 4)},
-        "kernels": {"load": {"GBps": round(alg / (np.mean(l_ms) * 1e-3) / 1e9, 1), "avg_ms": round(float(np.mean(l_ms)), 4)},
-                    "store": {"GBps": round(alg / (np.mean(s_ms) * 1e-3) / 1e9, 1), "avg_ms": round(float(np.mean(s_ms)), 4)}},
+                                 if at_reference_shape else None),
+                     "traffic_source": TRAFFIC_SOURCE if at_reference_shape else None,
+                     "alg_bytes_per_launch": alg, "avg_launch_ms": dom["avg_ms"]},
+        "kernels": {"load": l_stat, "store": s_stat},
     }
+    pool.close()
+    del layers, tm, tm_out
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -839,7 +853,14 @@ def main():
         print(json.dumps(out), flush=True)
         return
     if args.workload == "layout_change":
+        # the reference's pool (10240 blocks per layer, 4.7 GB), then the same step with the page list walked
+        # in the order given, then on a pool that fills a production share of HBM (163840 blocks, 75 GB)
         out = run_layout_change(args, bk, dev)
+        if not args.pool_pages:
+            for key, kw in (("unsorted_walk", dict(sort=False)), ("pool_163840_blocks", dict(blocks=163840))):
+                o = run_layout_change(args, bk, dev, **kw)
+                out[key] = {"workload": o["config"]["workload"], "pool_GB": o["config"]["pool_GB"], "value": o["value"],
+                            "pct_of_hbm_peak": o["pct_of_hbm_peak"], "kernels": o["kernels"]}
         print(json.dumps(out), flush=True)
         return
     if args.workload == "staging":

@@ -146,6 +146,7 @@ struct bikv_pool {
   const char** d_plane_base;        // device table: payload planes, then scale planes
   uint64_t align_bits;              // OR of every base, stride and tile size (payload)
   uint64_t scale_align_bits;
+  bool kv_rows;                     // planes 2l and 2l+1 interleave in 512-byte rows (the pair mover's shape)
 };
 
 extern "C" int bikv_abi_version(void) { return BIKV_ABI_VERSION; }
@@ -207,6 +208,8 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
     t.transpose_block = (int)value;
   } else if (!strcmp(key, "transpose_pairs")) {
     t.transpose_pairs = value ? 1 : 0;
+  } else if (!strcmp(key, "pair_rows")) {
+    t.pair_rows = value ? 1 : 0;
   } else if (!strcmp(key, "debug_unique")) {
     t.debug_unique = value ? 1 : 0;
   } else if (!strcmp(key, "run_chunk_kib")) {
@@ -281,6 +284,12 @@ extern "C" int bikv_pool_create(const bikv_pool_desc* d, bikv_pool** out) {
   p->d_plane_base = static_cast<const char**>(dtab);
   p->align_bits = ab;
   p->scale_align_bits = sab;
+  // The Worker's [tokens, 2, heads, dim] tensors at 512 bytes per row: K and V rows of a token are the two
+  // halves of one KiB, plane 2l+1 starts one row after plane 2l.
+  p->kv_rows = !has_scale && row_bytes == 512 && row_stride == 1024 && d->tile_bytes % 1024 == 0 &&
+               d->n_planes % 2 == 0 && (ab & 15) == 0;
+  for (int q = 0; q + 1 < d->n_planes && p->kv_rows; q += 2)
+    if (table[q + 1] != table[q] + 512) p->kv_rows = false;
   *out = p;
   return BIKV_OK;
 }
@@ -339,6 +348,7 @@ static int build_move(int bank, const bikv_pool* pool, const bikv_page_batch* b,
   if ((pool->row_bytes & (pool->row_bytes - 1)) == 0)
     for (m->payload.log2_row = 0; (int64_t(1) << m->payload.log2_row) < pool->row_bytes;) ++m->payload.log2_row;
   m->payload.vec_width = lowbit_width(pool->align_bits | (uint64_t)staging);
+  m->kv_rows = pool->kv_rows && m->payload.vec_width == 16 && (pb & 1) == 0 && (pc & 1) == 0;
   if (has_scale) {
     m->scale.plane_base = pool->d_plane_base + pool->n_planes;
     m->scale.staging = static_cast<char*>(const_cast<void*>(scale_staging));

@@ -43,6 +43,8 @@ struct MoveArgs {
   int32_t order;                  // wave mover: 0 = plane by plane, 1 = page chunk by page chunk
   int32_t log2_chunk;             // order 1: pages per chunk = 2^log2_chunk
   int32_t layout_hint;            // host side only: 0 none, 1 layer-major, 2 page-major staging
+  int32_t kv_rows;                // 1 = K and V rows of a token are adjacent 512-byte halves of one KiB of the
+                                  // pool (planes 2l and 2l+1 interleave row by row): the pair mover may be used
   uint32_t* status;
 };
 
@@ -64,6 +66,8 @@ struct Tuning {
   int transpose_pairs = 1;     // the K/V-pair kernel where the shape allows (0 = element-wise kernel)
   int transpose_block = 512;   // lanes per workgroup of the K/V-pair kernel: 128, 256, 512, 1024
   int debug_unique = 0;        // 1 = scattering entry points check their destination ids on the host first
+  int pair_rows = 0;           // 1 = pools whose K and V rows interleave in 512-byte halves use the pair mover
+                               // (measured 4-6 % SLOWER than the general wave mover: off by default)
 };
 Tuning& tuning();
 

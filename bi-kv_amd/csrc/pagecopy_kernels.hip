@@ -356,6 +356,94 @@ __global__ __launch_bounds__(B) void tile_move_wave_kernel(const MoveArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Pair mover: the Worker's per-layer tensors [tokens, 2, heads, dim] (Bi-KV/Worker/Worker.py:74-78) at
+// the reference's own shape (2 KV heads x 128 x fp16) have rows of 512 bytes, K and V of a token adjacent:
+// one KiB of the pool is {K row, V row} of one token, and the K tile and the V tile of a page are two
+// different tiles of the staging image. A wave that moves 1 KiB of ONE tile therefore touches two
+// half-KiB pieces of the pool, which costs the scatter 10-15 %. Here a wave takes the two KiB of two
+// consecutive tokens instead — {K0 V0}, {K1 V1}: two 1 KiB accesses on the pool side — and exchanges the
+// upper half of the first vector with the lower half of the second between lanes i and i+32
+// (v_permlane32_swap), which turns them into {K0 K1} and {V0 V1}: two 1 KiB accesses on the staging side,
+// one in the K tile and one in the V tile. The exchange is its own inverse, so the scatter is the same
+// sequence backwards. Grid and walks are those of the wave mover with "plane" meaning layer.
+// MEASURED (MI355X, Qwen2-1.5B-shaped pool in the Worker's form, 30 GB): gather 5.85 / scatter 5.20 TB/s
+// against 6.07 / 5.51 for the general wave mover with its two half-KiB pool pieces per wave: two vectors in
+// flight per lane cost more than the contiguity gains, as they do in a plain copy. Kept selectable
+// ("pair_rows" = 1) and tested; not the default.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void load2(uint64_t a, uint64_t b, u32x4& x, u32x4& y) {
+  asm volatile("global_load_dwordx4 %0, %2, off sc1 nt\n\t"
+               "global_load_dwordx4 %1, %3, off sc1 nt\n\t"
+               "s_waitcnt vmcnt(0)"
+               : "=&v"(x), "=&v"(y) : "v"(a), "v"(b) : "memory");
+}
+__device__ __forceinline__ void store2(uint64_t a, uint64_t b, const u32x4& x, const u32x4& y) {
+  asm volatile("global_store_dwordx4 %0, %2, off sc1 nt\n\t"
+               "global_store_dwordx4 %1, %3, off sc1 nt"
+               : : "v"(a), "v"(b), "v"(x), "v"(y) : "memory");
+}
+// lanes 32-63 of x <-> lanes 0-31 of y, all four dwords
+__device__ __forceinline__ void swap_halves(u32x4& x, u32x4& y) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const auto r = __builtin_amdgcn_permlane32_swap(x[i], y[i], false, false);
+    x[i] = r[0];
+    y[i] = r[1];
+  }
+}
+
+template <int DIR>
+__global__ __launch_bounds__(64) void tile_move_pair_kernel(const MoveArgs a) {
+  const uint32_t bx = blockIdx.x;
+  const int32_t lp = a.payload.log2_rows;       // pieces (token pairs) per tile: 2^lp or n_parts
+  const uint32_t np = a.payload.n_parts;
+  const uint32_t bt = lp >= 0 ? bx >> lp : bx / np;
+  const uint32_t part = lp >= 0 ? (bx & ((1u << lp) - 1u)) : bx - bt * np;
+  const uint32_t lc = (uint32_t)a.log2_chunk;
+  int64_t layer;
+  uint32_t i;
+  if (a.order == 0) {
+    layer = blockIdx.y;
+    i = bt;
+  } else {
+    const uint64_t chunk = (uint64_t)blockIdx.y + (uint64_t)blockIdx.z * gridDim.y;
+    const uint64_t page = (chunk << lc) + (bt & ((1u << lc) - 1u));
+    if (page >= (uint64_t)a.n_batch) return;
+    i = (uint32_t)page;
+    layer = (int64_t)(bt >> lc);
+  }
+  const int64_t qk = a.plane_begin + 2 * layer;                      // the K plane; V is qk + 1
+  const int64_t pid = cload(a.page_ids + i);
+  const int64_t s0 = cload(a.slots + i) - a.slot_bias;
+  const int64_t ss = cload(a.slot_strides + i);
+  const uint64_t plane = (uint64_t)cload(a.payload.plane_base + qk);
+  const int64_t slot_k = s0 + qk * ss, slot_v = slot_k + ss;
+  const bool bad_page = (uint64_t)pid >= (uint64_t)a.n_pool_pages;
+  const bool bad_slot = (uint64_t)slot_k >= (uint64_t)a.payload.n_slots || (uint64_t)slot_v >= (uint64_t)a.payload.n_slots;
+  if (bad_page || bad_slot) {
+    if (threadIdx.x == 0 && part == 0) {
+      if (bad_page) raise(a.status, ST_SLOT_PAGE);
+      if (bad_slot) raise(a.status, DIR == 0 ? ST_SLOT_DST : ST_SLOT_SRC);
+    }
+    return;
+  }
+  const uint64_t lane = threadIdx.x * 16u;
+  const uint64_t pool = plane + (uint64_t)(pid * a.payload.page_stride) + (uint64_t)part * 2048u + lane;
+  const uint64_t sk = (uint64_t)a.payload.staging + (uint64_t)(slot_k * a.payload.tile_bytes) + (uint64_t)part * 1024u + lane;
+  const uint64_t sv = (uint64_t)a.payload.staging + (uint64_t)(slot_v * a.payload.tile_bytes) + (uint64_t)part * 1024u + lane;
+  u32x4 x, y;
+  if (DIR == 0) {
+    load2(pool, pool + 1024u, x, y);      // {K0 V0}, {K1 V1}
+    swap_halves(x, y);                    // {K0 K1}, {V0 V1}
+    store2(sk, sv, x, y);
+  } else {
+    load2(sk, sv, x, y);
+    swap_halves(x, y);
+    store2(pool, pool + 1024u, x, y);
+  }
+}
+
 // How the wave mover walks a batch, and whether it marks its accesses non-temporal. Measured on
 // MI355X with 8-64 KiB tiles and 56-160 planes of 2 GiB each:
 //   * random accesses confined to ONE plane's few GiB run ~10 % slower than the same accesses spread
@@ -492,6 +580,20 @@ static bool finish_class(TileClass& c, int forced_seg, int64_t n_batch, int plan
 
 hipError_t launch_tile_move(int dir, MoveArgs& a, hipStream_t stream) {
   if (a.n_batch <= 0 || a.plane_count <= 0) return hipSuccess;
+  if (tuning().seg == 0 && tuning().pair_rows != 0 && a.kv_rows != 0 && tuning().wave_block == 64) {
+    // K and V rows interleave in half-KiB pieces: the pair mover, planned as a wave mover over layers
+    // whose pieces are token pairs (1 KiB of each of the two staging tiles, 2 KiB of the pool)
+    dim3 grid;
+    const WavePolicy pol = choose_wave_policy(dir, a.layout_hint);
+    MoveArgs b = a;
+    b.plane_count = a.plane_count / 2;
+    if (plan_wave(b, 64, pol.order, pol.log2_chunk, &grid)) {
+      b.plane_count = a.plane_count;
+      if (dir == 0) hipLaunchKernelGGL(tile_move_pair_kernel<0>, grid, dim3(64), 0, stream, b);
+      else hipLaunchKernelGGL(tile_move_pair_kernel<1>, grid, dim3(64), 0, stream, b);
+      return hipGetLastError();
+    }
+  }
   if (tuning().seg == 0) {
     // default: the wave mover, whenever the payload shape qualifies
     dim3 grid;

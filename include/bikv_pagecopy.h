@@ -77,7 +77,10 @@ int bikv_check_status(int device, void* stream, uint32_t* bits_out);
  * short runs share a row of the launch grid, default; 0 = one row per run), "transpose_lds_kib" and
  * "transpose_dsplit" (LDS tile budget and head_dim slices of the layout-change kernel),
  * "transpose_pairs" (1 = the K/V-pair kernel, default; 0 = the element-wise kernel) and "transpose_block" (its lanes per workgroup: 128, 256, 512, 1024),
- * "debug_unique" (1 = what BIKV_DEBUG_UNIQUE=1 in the environment switches on, see bikv_find_duplicate).
+ * "debug_unique" (1 = what BIKV_DEBUG_UNIQUE=1 in the environment switches on, see bikv_find_duplicate),
+ * "pair_rows" (1 = pools whose K and V rows interleave in 512-byte halves, the Worker's own tensors at
+ * 2 KV heads x 128 x fp16, are moved two tokens at a time with the halves exchanged between lanes, so
+ * that both sides see 1 KiB accesses; 0 = default: the general wave mover, which measures 4-6 % faster).
  * Process-wide. */
 int bikv_set_tuning(const char* key, int64_t value);
 /* Every knob back to its default. */

@@ -298,6 +298,55 @@ def test_worker_token_interleaved_layers(bk, oracle, cuda, P, H, D, dtype, layou
     pool.close()
 
 
+@pytest.mark.parametrize("layout", ["layer_major", "page_major"])
+def test_pair_mover_for_half_kib_rows_matches_the_general_mover_and_the_oracle(bk, oracle, cuda, layout):
+    """The Worker's own shape (2 KV heads x 128 x fp16: 512-byte rows, K and V of a token adjacent) takes the
+    pair mover, which exchanges half-waves between lanes; every walk of it against the oracle and against
+    the general wave mover on the same pool, and a rejected page id."""
+    _announce(f"pair mover {layout}")
+    rng = np.random.default_rng(311)
+    P, H, D, L, blocks = 16, 2, 128, 5, 70
+    layers_h = [rng.integers(0, 65536, size=(blocks * P, 2, H, D), dtype=np.uint16) for _ in range(L)]
+    planes_h = oracle.planes_of_token_kv_layers(layers_h, P).view(np.uint8)
+    reqs = [rng.permutation(blocks)[:33], np.array([5, 5, 9]), rng.permutation(blocks)[:1]]
+    want = oracle.gather_layered_c(planes_h, reqs, layout).tobytes()
+    perm = rng.permutation(blocks)
+    sreqs = [perm[:21], perm[21:40]]
+    for pair_rows, order, lc in ((1, -1, -1), (1, 0, 0), (1, 1, 0), (1, 1, 2), (1, 1, 5), (0, -1, -1)):
+        bk.set_tuning(pair_rows=pair_rows, order=order, log2_chunk=lc)
+        layers_d = [torch.from_numpy(a.view(np.int16)).to(cuda).view(torch.float16) for a in layers_h]
+        pool = bk.PagedKVPool.from_token_kv_layers(layers_d, P)
+        batch = pool.make_batch(reqs, layout)
+        st, _ = pool.gather(batch)
+        pool.check()
+        assert _to_np(st).tobytes() == want, (pair_rows, order, lc)
+        sb = pool.make_batch(sreqs, layout, check_unique=True)
+        src = rng.integers(0, 256, size=sb.n_slots * pool.tile_bytes, dtype=np.uint8)
+        pool.scatter(sb, torch.from_numpy(src).to(cuda))
+        pool.check()
+        ph = planes_h.copy()
+        oracle.scatter_layered_c(ph, sreqs, src, layout)
+        back = oracle.token_kv_layers_of_planes(ph.view(np.uint16), P, H, D)
+        for l in range(L):
+            assert _to_np(layers_d[l]).tobytes() == back[l].tobytes(), (pair_rows, order, lc, l)
+        # a page id outside the pool: that page is skipped and reported, its neighbours still move
+        bad = pool.make_batch([[2, blocks + 3, 7]], layout)
+        st2 = torch.full((bad.n_slots * pool.tile_bytes,), 0xA5, dtype=torch.uint8, device=cuda)
+        pool.gather(bad, st2)
+        with pytest.raises(RuntimeError, match="page-id"):
+            pool.check()
+        v = bad.request_view(st2, 0)
+        good = oracle.gather_layered_c(ph, [np.array([2, 7])], layout)
+        gv = good.reshape(2 * L, 2, -1) if layout == "layer_major" else good.reshape(2, 2 * L, -1)
+        if layout == "layer_major":
+            assert np.array_equal(_to_np(v[:, 0]), gv[:, 0]) and np.array_equal(_to_np(v[:, 2]), gv[:, 1])
+            assert bool((v[:, 1] == 0xA5).all())
+        else:
+            assert np.array_equal(_to_np(v[0]), gv[0]) and np.array_equal(_to_np(v[2]), gv[1])
+            assert bool((v[1] == 0xA5).all())
+        pool.close()
+
+
 def test_empty_batch_and_empty_requests(bk, oracle, cuda):
     _announce("empty")
     pool_d = torch.zeros((2, 8, 4096), dtype=torch.uint8, device=cuda)

@@ -116,6 +116,36 @@ def test_default_tm_pages_is_a_dense_received_buffer(lib, oracle, cuda):
     assert layers_d[l][ids[2] * P + t, k, h, d].item() == recv[2 * P + t, d, h, l, k].item()
 
 
+def test_page_list_walks_in_block_order_with_the_same_result(lib, oracle, cuda):
+    """NHDPool.page_list sorts a host-built page list by block id and keeps each page with its block: the
+    pool and the stored pages are byte for byte what the unsorted list gives."""
+    import bikv_pagecopy as bk
+    print("[case] layout change, sorted page list", flush=True)
+    rng = np.random.default_rng(9)
+    P, D, H, L, blocks, n = 16, 128, 2, 6, 40, 17
+    tm_h, layers_h, tm_d, layers_d = _make(rng, "token_kv", 2, P, D, H, L, blocks, n, cuda)
+    pool = bk.NHDPool.from_token_kv_layers(layers_d, P)
+    ids = rng.permutation(blocks)[:n].astype(np.int64)
+    tm_pages = rng.permutation(n).astype(np.int64)           # page i of the call is tm page tm_pages[i]
+    b, p = pool.page_list(ids, tm_pages, sort=True, check_unique=True)
+    assert bool((b[1:] > b[:-1]).all()) and sorted(b.tolist()) == sorted(ids.tolist())
+    assert dict(zip(b.tolist(), p.tolist())) == dict(zip(ids.tolist(), tm_pages.tolist()))
+    pool.load_token_major(tm_d, b, p)
+    pool.check()
+    oracle.transpose_pages_c(layers_h, "token_kv", tm_h, ids, tm_pages, "load")
+    for l in range(L):
+        assert _to_np(layers_d[l]).tobytes() == layers_h[l].tobytes()
+    out = torch.zeros_like(tm_d)
+    pool.store_token_major(out, b, p)
+    pool.check()
+    assert torch.equal(out.view(torch.int16), tm_d.view(torch.int16))
+    # unsorted, default pages, and the duplicate check
+    b2, p2 = pool.page_list(ids)
+    assert b2.tolist() == ids.tolist() and p2.tolist() == list(range(n))
+    with pytest.raises(RuntimeError, match="block ids: destination id"):
+        pool.page_list([3, 5, 3], check_unique=True)
+
+
 def test_bad_ids_are_skipped_and_reported_and_shapes_are_checked(lib, cuda):
     import bikv_pagecopy as bk
     print("[case] layout change error paths", flush=True)
