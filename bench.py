@@ -24,6 +24,12 @@ pool <-> pinned-host staging pipeline (`staging`): all 128 requests enqueued bac
 chunks on 2 and 4 lanes, kernel-direct and automatic modes, both directions, each next to a plain
 hipMemcpyAsync of one large pinned buffer timed immediately before it. `--no-configs` / `--no-staging`
 skip those parts.
+
+Pools and gather destinations are allocated through the library's bikv_device_alloc, which lays their
+physical chunks alternately in the two halves of HBM (`--pool-alloc torch` / `--staging-alloc torch`
+take torch's allocator instead; the default run times the headline workload once more that way and
+reports it as `torch_alloc`). If the library's allocator cannot serve a request the run falls back to
+torch for that buffer and says so in `device_alloc`.
 """
 import argparse
 import json
@@ -39,12 +45,12 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch as a multiple of the algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this file, each scaled by the same counter's reading for the plain-copy
 # calibration launch below (summaries under profiles/). None = not measured for that workload.
-MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9949, "scatter": 1.0003},
+MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9948, "scatter": 1.0002},
                           "qwen2_1p5b": {"gather": 1.0009},
-                          "llama3_8b": {"gather": 0.9966},
+                          "llama3_8b": {"gather": 0.9967},
                           "llama3_70b_fp8": {"gather": 1.0142, "scatter": 1.0001},
                           "qwen2_7b_token_major": {"gather": 0.9997, "scatter": 1.0002},
-                          "layout_change": {"load": 1.0034, "store": 1.0025}}
+                          "layout_change": {"load": 1.0029, "store": 1.0035}}
 
 
 def parse_args():
@@ -58,8 +64,12 @@ def parse_args():
     ap.add_argument("--no-other-layout", dest="no_other_layout", action="store_true",
                     help="skip the second measurement with the other staging layout")
     ap.add_argument("--pool-pages", type=int, default=0, help="override the pool size (pages per plane)")
-    ap.add_argument("--pool-alloc", choices=["planes", "stacked"], default="stacked",
-                    help="one device tensor per (layer, K|V) plane, or one stacked allocation")
+    ap.add_argument("--pool-alloc", choices=["planes", "stacked", "spread"], default="spread",
+                    help="one torch tensor per (layer, K|V) plane, one stacked torch allocation, or one allocation "
+                         "from bikv_device_alloc (physical chunks alternating between the two halves of HBM)")
+    ap.add_argument("--staging-alloc", dest="staging_alloc", choices=["torch", "spread", "auto"], default="auto",
+                    help="where the dense staging buffers come from: torch, bikv_device_alloc, or auto = the buffer a "
+                         "gather WRITES from bikv_device_alloc, the buffer a scatter only reads from torch")
     ap.add_argument("--no-configs", dest="no_configs", action="store_true",
                     help="skip the other named configurations (default workload only)")
     ap.add_argument("--no-staging", dest="no_staging", action="store_true",
@@ -84,6 +94,25 @@ def log(msg):
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
+ALLOC_NOTES = []   # what happened when memory was asked from bikv_device_alloc (reported in the JSON line)
+
+
+def spread_empty(bk, nbytes, dev, what):
+    """A uint8 device tensor from bikv_device_alloc. If the allocator cannot serve the request (no
+    virtual-memory API on this driver, device too full) the measurement still runs, on torch memory, and the
+    JSON line says so."""
+    import torch
+    try:
+        buf = bk.DeviceBuffer(nbytes, dev)
+        log(f"bikv_device_alloc ({what}): {buf.info}")
+        ALLOC_NOTES.append({"what": what, **buf.info})
+        return buf.tensor
+    except RuntimeError as e:
+        log(f"bikv_device_alloc failed for {what}: {e}; using torch memory")
+        ALLOC_NOTES.append({"what": what, "failed": str(e)})
+        return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+
 def fill_random_bytes(t):
     """Random bytes in place, one plane at a time (bit patterns are what matters for a byte mover)."""
     import torch
@@ -100,6 +129,12 @@ def make_pool(shape, dev, alloc="planes"):
     import torch
 
     def one(tile_bytes):
+        if alloc == "spread":
+            import bikv_pagecopy as bk
+            n = shape.n_planes * shape.n_pages * tile_bytes
+            t = spread_empty(bk, n, dev, f"{shape.name} pool").view(shape.n_planes, shape.n_pages, tile_bytes)
+            fill_random_bytes(t)
+            return [t[q] for q in range(shape.n_planes)]
         if alloc == "stacked":
             t = torch.empty((shape.n_planes, shape.n_pages, tile_bytes), dtype=torch.uint8, device=dev)
             fill_random_bytes(t)
@@ -279,11 +314,15 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layo
 
     g_groups, s_groups = groups_of(g_reqs), groups_of(s_reqs, unique=True)
     max_slots = max(b.n_slots for b, _ in g_groups + s_groups)
-    g_st = torch.empty(max_slots * shape.tile_bytes, dtype=torch.uint8, device=dev)
+    if args.staging_alloc in ("spread", "auto"):
+        g_st = spread_empty(bk, max_slots * shape.tile_bytes, dev, f"{name} gather destination")
+    else:
+        g_st = torch.empty(max_slots * shape.tile_bytes, dtype=torch.uint8, device=dev)
     g_sc = torch.empty(max_slots * shape.scale_tile_bytes, dtype=torch.uint8, device=dev) if shape.scales else None
     s_st = s_sc = None
     if s_groups:
-        s_st = torch.empty_like(g_st)
+        s_st = (spread_empty(bk, g_st.numel(), dev, f"{name} scatter source") if args.staging_alloc == "spread"
+                else torch.empty_like(g_st))
         fill_random_bytes(s_st)
         if shape.scales:
             s_sc = torch.empty_like(g_sc)
@@ -381,7 +420,11 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layo
                                f"scatter requests, {n_pages} pages/step in {len(g_groups)}+{len(s_groups)} launches, "
                                f"layout {layout}",
                    "pool_GB": round(shape.pool_bytes / 1e9, 2), "tile_bytes": shape.tile_bytes,
-                   "planes": shape.n_planes, "pool_alloc": args.pool_alloc},
+                   "planes": shape.n_planes,
+                   "pool_alloc": ("bikv_device_alloc (physical chunks alternating between the halves of HBM)"
+                                  if args.pool_alloc == "spread" else f"torch ({args.pool_alloc})"),
+                   "staging_alloc": {"auto": "gather destination from bikv_device_alloc, scatter source from torch",
+                                     "spread": "bikv_device_alloc", "torch": "torch"}[args.staging_alloc]},
         "timed_region_s": round(wall, 3),
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "pages_per_s": round(n_pages / (wall / steps), 1),
@@ -732,13 +775,14 @@ def run_token_major(args, bk, workloads, dev):
     }
 
 
-def run_layout_change(args, bk, dev, blocks=None, sort=True):
+def run_layout_change(args, bk, dev, blocks=None, sort=False, pool_alloc=None):
     """Received token-major pages -> the Worker's per-layer paged pool and back, at the reference's own
     shapes: token_shape (128, 2, 28, 2) fp16 (Model/qwen2.py:512-522), 28 layer tensors of
     [blocks*16, 2, 2, 128] (Worker.py:69-78: 10240 blocks), 4096 pages of 16 tokens per step and
-    direction, random blocks. The page lists are built on the host and handed over through
-    NHDPool.page_list: the load walks its list in ascending block order (`sort`), the store in the order
-    given (sorting helps the direction whose scattered side is written and hurts the other)."""
+    direction, random blocks. The pool's memory comes from bikv_device_alloc (`--pool-alloc spread`, the
+    default) or from torch. The page lists are built on the host and handed over through NHDPool.page_list;
+    with `sort` the load walks its list in ascending block order (worth ~4 % on a torch-allocated pool that
+    sits in one half of HBM, nothing on a spread pool)."""
     import numpy as np
     import torch
     from oracle import pagecopy_oracle as oracle
@@ -746,7 +790,12 @@ def run_layout_change(args, bk, dev, blocks=None, sort=True):
     P, D, H, L, n_pages = 16, 128, 2, 28, 4096
     blocks = blocks or args.pool_pages or 10240
     n_pages = min(n_pages, blocks)
-    layers = [torch.empty((blocks * P, 2, H, D), dtype=torch.float16, device=dev) for _ in range(L)]
+    pool_alloc = pool_alloc or args.pool_alloc
+    if pool_alloc == "spread":
+        arena = spread_empty(bk, L * blocks * P * 2 * H * D * 2, dev, "layer tensors")
+        layers = list(arena.view(torch.float16).view(L, blocks * P, 2, H, D).unbind(0))
+    else:
+        layers = [torch.empty((blocks * P, 2, H, D), dtype=torch.float16, device=dev) for _ in range(L)]
     for t in layers:
         fill_random_bytes(t)
     pool = bk.NHDPool.from_token_kv_layers(layers, P)
@@ -796,16 +845,17 @@ def run_layout_change(args, bk, dev, blocks=None, sort=True):
     s_stat = launch_stats([e[1].elapsed_time(e[2]) for e in evs], alg)
     slow_is_load = l_stat["avg_ms"] >= s_stat["avg_ms"]
     dom = l_stat if slow_is_load else s_stat
-    at_reference_shape = blocks == 10240 and sort
+    at_reference_shape = blocks == 10240 and pool_alloc == "spread"
     out = {
         "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
         "value": round(2 * alg / (wall / args.steps) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "u16", "data": "synthetic",
         "config": {"workload": f"layout_change: token-major pages <-> {L} layer tensors [{blocks}*{P}, 2, {H}, {D}] fp16, "
-                               f"{n_pages} pages of {P} tokens loaded then stored per step, random blocks; the load walks "
-                               f"them in {'ascending block order' if sort else 'the order given'}, the store in the order given",
-                   "pool_GB": round(L * blocks * P * 2 * H * D * 2 / 1e9, 2)},
+                               f"{n_pages} pages of {P} tokens loaded then stored per step, random blocks"
+                               f"{'; the load walks them in ascending block order' if sort else ''}",
+                   "pool_GB": round(L * blocks * P * 2 * H * D * 2 / 1e9, 2),
+                   "pool_alloc": "bikv_device_alloc (chunks alternating between the halves of HBM)" if pool_alloc == "spread" else "torch"},
         "timed_region_s": round(wall, 3),
         "pct_of_hbm_peak": round(100 * 2 * alg / (wall / args.steps) / 1e9 / HBM_PEAK_GBPS, 2),
         "pages_per_s": round(2 * n_pages / (wall / args.steps), 1), "bit_exact": True,
@@ -822,6 +872,12 @@ def run_layout_change(args, bk, dev, blocks=None, sort=True):
     del layers, tm, tm_out
     torch.cuda.empty_cache()
     return out
+
+
+def emit(out):
+    if ALLOC_NOTES:
+        out["device_alloc"] = ALLOC_NOTES
+    print(json.dumps(out), flush=True)
 
 
 def main():
@@ -846,22 +902,24 @@ def main():
 
     if args.workload == "reference_200x50":
         out = run_reference_scenario(args, bk, dev)
-        print(json.dumps(out), flush=True)
+        emit(out)
         return
     if args.workload == "qwen2_7b_token_major":
         out = run_token_major(args, bk, workloads, dev)
-        print(json.dumps(out), flush=True)
+        emit(out)
         return
     if args.workload == "layout_change":
-        # the reference's pool (10240 blocks per layer, 4.7 GB), then the same step with the page list walked
-        # in the order given, then on a pool that fills a production share of HBM (163840 blocks, 75 GB)
+        # the reference's pool (10240 blocks per layer, 4.7 GB); then the same step on a torch-allocated pool
+        # (wherever the driver puts it), that pool with the load's page list sorted by block, and a pool that
+        # fills a production share of HBM (163840 blocks, 75 GB)
         out = run_layout_change(args, bk, dev)
         if not args.pool_pages:
-            for key, kw in (("unsorted_walk", dict(sort=False)), ("pool_163840_blocks", dict(blocks=163840))):
+            for key, kw in (("torch_alloc", dict(pool_alloc="stacked")), ("torch_alloc_sorted_load", dict(pool_alloc="stacked", sort=True)),
+                            ("pool_163840_blocks", dict(blocks=163840))):
                 o = run_layout_change(args, bk, dev, **kw)
                 out[key] = {"workload": o["config"]["workload"], "pool_GB": o["config"]["pool_GB"], "value": o["value"],
                             "pct_of_hbm_peak": o["pct_of_hbm_peak"], "kernels": o["kernels"]}
-        print(json.dumps(out), flush=True)
+        emit(out)
         return
     if args.workload == "staging":
         print(json.dumps({"metric": "pinned-host staging GB/s", "unit": "GB/s", "n_gpus": 1,
@@ -878,6 +936,15 @@ def main():
         out["other_layout"] = {"layout": alt_layout, "value": o2["value"], "pct_of_hbm_peak": o2["pct_of_hbm_peak"],
                                "steps": o2["steps"], "kernels": {k: v for k, v in o2["kernels"].items() if v}}
     default_run = args.workload == "qwen2_7b" and not args.pool_pages
+    if default_run and args.pool_alloc == "spread" and not args.no_other_layout:
+        # the same workload with pool and staging from torch.empty (hipMalloc), wherever the driver places them
+        import copy
+        alt = copy.copy(args)
+        alt.pool_alloc, alt.staging_alloc = "stacked", "torch"
+        log("same workload, pool and staging allocated by torch")
+        o3, _, _, _ = run_gather_scatter(alt, bk, workloads, dev, with_copy=False, target_s=0.6, warmup=3)
+        out["torch_alloc"] = {"value": o3["value"], "pct_of_hbm_peak": o3["pct_of_hbm_peak"], "steps": o3["steps"],
+                              "kernels": {k: v for k, v in o3["kernels"].items() if v}}
     if default_run and not args.no_configs:
         # the other named configurations, each at full size: allocated, measured for about a second, freed
         out["configs"] = {}
@@ -897,7 +964,7 @@ def main():
     if not args.no_cpu_baseline:
         log("timing the CPU baseline")
         out["cpu_baseline"] = cpu_baseline(shape, wl)
-    print(json.dumps(out), flush=True)
+    emit(out)
 
 
 if __name__ == "__main__":

@@ -20,6 +20,7 @@ ST_SRC_RANGE, ST_DST_RANGE, ST_PAGE_ID = 1, 2, 4
 LAYOUT_LAYER_MAJOR, LAYOUT_PAGE_MAJOR = 0, 1
 HINT_NONE, HINT_LAYER_MAJOR, HINT_PAGE_MAJOR = 0, 1, 2
 STAGE_PIPELINED, STAGE_DIRECT, STAGE_AUTO = 0, 1, 2
+PLACE_SPREAD, PLACE_SEQUENTIAL = 0, 1
 
 
 class PoolDesc(C.Structure):
@@ -66,6 +67,11 @@ class NHDDesc(C.Structure):
         ("token_stride_elems", C.c_int64),
         ("layer_base", C.POINTER(C.c_void_p)),
     ]
+
+
+class AllocInfo(C.Structure):
+    _fields_ = [("bytes", C.c_int64), ("chunk_bytes", C.c_int64), ("n_chunks", C.c_int32),
+                ("n_other_half", C.c_int32), ("n_fillers", C.c_int32), ("reserved", C.c_int32)]
 
 
 class StageStats(C.Structure):
@@ -153,6 +159,9 @@ _SIGNATURES = {
                                 C.POINTER(C.c_double)]),
     "bikv_h2d_copy": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
                                 C.POINTER(C.c_double)]),
+    "bikv_device_alloc": (C.c_int, [C.c_int, C.c_int64, C.c_int32, C.POINTER(C.c_void_p)]),
+    "bikv_device_free": (C.c_int, [C.c_void_p]),
+    "bikv_device_alloc_info": (C.c_int, [C.c_void_p, C.POINTER(AllocInfo)]),
     "bikv_host_alloc": (C.c_int, [C.c_int64, C.POINTER(C.c_void_p)]),
     "bikv_host_free": (C.c_int, [C.c_void_p]),
     "bikv_consumer_init": (C.c_int, [C.c_int, C.c_char_p, C.c_size_t]),

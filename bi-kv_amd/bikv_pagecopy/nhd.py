@@ -70,9 +70,10 @@ class NHDPool:
         upload. With `sort` the pages are reordered by ascending block id — the result is the same, the
         order in which the kernel walks the pool is not: neighbouring workgroups then touch neighbouring
         blocks of every layer tensor while the token-major pages are visited in a scattered order.
-        Measured on MI355X at the reference's shape (4096 of 10240 blocks): a LOAD gains ~4 % (its
-        scattered side is the written one), a STORE loses ~7 % (its dense writes become scattered), so
-        sort the list of a load and leave the list of a store as it is. `tm_pages` defaults to 0..n-1
+        Measured on MI355X at the reference's shape (4096 of 10240 blocks) with a torch-allocated pool
+        that sits in one half of HBM: a LOAD gains ~4 % (its scattered side is the written one), a STORE
+        loses ~7 % (its dense writes become scattered). On a pool from bikv_device_alloc, whose chunks
+        alternate between the halves, the order makes no difference. `tm_pages` defaults to 0..n-1
         BEFORE sorting, i.e. page i of the token-major buffer belongs to block_ids[i]."""
         import numpy as np
         ids = np.ascontiguousarray(np.asarray(block_ids, dtype=np.int64).reshape(-1))

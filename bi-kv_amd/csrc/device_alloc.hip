@@ -1,0 +1,295 @@
+// Pool memory placed for the MI355X memory system.
+//
+// Measured on MI355X (random 16 KiB tiles, one 64-lane workgroup per KiB, 4 GiB moved per launch): the
+// physical address space behaves as two halves. A copy whose RANDOM WRITES all land in one half runs at
+// 5.6-5.7 TB/s wherever its reads come from; the same writes spread over both halves run at 6.6-6.7 TB/s
+// (+18 %). Reads do not care (6.25-6.45 TB/s either way), sequential writes hardly do. Which half a piece
+// of memory lies in is a property of its PHYSICAL address: inside one hipMalloc of 112 GiB the boundary
+// sat at an offset of 64 GiB; 1 GiB physical chunks created one after the other were 95 in one half, then
+// 17 in the other. A KV pool that fits one half (every pool below ~100 GB on an otherwise empty GPU, and a
+// big pool whenever the driver happens to place it so) therefore scatters 15-18 % slower than it could,
+// and how a big pool straddles the boundary is what moved whole-process results by several percent from
+// one allocation to the next.
+//
+// Nothing in HIP names the half, but it is easy to observe: a short scatter into two chunks is ~19 %
+// faster when they lie in different halves. bikv_device_alloc builds an allocation out of physical chunks
+// (hipMemCreate), classifies every chunk against the first one with that probe, keeps equal numbers of
+// both kinds (creating — and afterwards releasing — as many filler chunks as it takes to reach the other
+// half) and maps them alternately into one virtual range (hipMemAddressReserve / hipMemMap). Every
+// window of such a pool, however small, then spreads its writes over both halves.
+#include "../../include/bikv_pagecopy.h"
+#include "pagecopy_internal.h"
+
+#include <algorithm>
+#include <map>
+#include <mutex>
+#include <vector>
+
+using namespace bikv;
+
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// The probe: every workgroup copies one KiB from a small source window into a pseudo-random 16 KiB tile of
+// target a or target b (the same shape of traffic as a page scatter). Contents are garbage: the targets are
+// fresh chunks that hold no data yet.
+__global__ __launch_bounds__(64) void probe_kernel(const char* src, uint64_t src_mask, char* a, char* b,
+                                                   uint32_t tiles_each) {
+  const uint32_t w = blockIdx.x;
+  uint32_t x = (w >> 4) * 2654435761u;          // one hash per 16 KiB tile; its 16 pieces are neighbours
+  x ^= x >> 15;
+  x *= 2246822519u;
+  x ^= x >> 13;
+  const uint32_t t = x % (2 * tiles_each);
+  char* base = t < tiles_each ? a : b;
+  const uint64_t off = (uint64_t)(t < tiles_each ? t : t - tiles_each) * 16384u + (w & 15u) * 1024u + threadIdx.x * 16u;
+  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + (((uint64_t)w * 1024u + threadIdx.x * 16u) & src_mask)));
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(base + off));
+}
+
+struct Allocation {
+  int device = 0;
+  void* va = nullptr;
+  size_t bytes = 0, chunk = 0;
+  std::vector<hipMemGenericAllocationHandle_t> handles;   // in mapping order
+  int n_other = 0;                                         // chunks classified "other half"
+  int n_fillers = 0;                                       // chunks created and released again
+};
+
+std::mutex g_mu;
+std::map<void*, Allocation> g_allocs;
+
+size_t pow2_floor(size_t x) {
+  size_t p = 1;
+  while (p * 2 <= x) p *= 2;
+  return p;
+}
+
+struct Prober {
+  hipStream_t stream = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  char* src = nullptr;
+  size_t src_bytes = size_t(1) << 30;   // far beyond the caches: the probe's reads come from HBM like a scatter's
+  void* window = nullptr;      // two chunks of virtual space: [0] the reference chunk, [1] the candidate
+  size_t chunk = 0;
+  hipMemAccessDesc acc;
+
+  int init(int device, size_t chunk_bytes) {
+    chunk = chunk_bytes;
+    acc = hipMemAccessDesc();
+    acc.location.type = hipMemLocationTypeDevice;
+    acc.location.id = device;
+    acc.flags = hipMemAccessFlagsProtReadWrite;
+    BIKV_HIP(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+    BIKV_HIP(hipEventCreate(&e0));
+    BIKV_HIP(hipEventCreate(&e1));
+    BIKV_HIP(hipMalloc((void**)&src, src_bytes));
+    BIKV_HIP(hipMemAddressReserve(&window, 2 * chunk, 0, nullptr, 0));
+    return BIKV_OK;
+  }
+  void destroy() {
+    if (window) (void)hipMemAddressFree(window, 2 * chunk);
+    if (src) (void)hipFree(src);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (stream) (void)hipStreamDestroy(stream);
+  }
+  int map(int slot, hipMemGenericAllocationHandle_t h) {
+    char* at = static_cast<char*>(window) + (size_t)slot * chunk;
+    BIKV_HIP(hipMemMap(at, chunk, 0, h, 0));
+    BIKV_HIP(hipMemSetAccess(at, chunk, &acc, 1));
+    return BIKV_OK;
+  }
+  int unmap(int slot) {
+    BIKV_HIP(hipStreamSynchronize(stream));
+    BIKV_HIP(hipMemUnmap(static_cast<char*>(window) + (size_t)slot * chunk, chunk));
+    return BIKV_OK;
+  }
+  // milliseconds of one probe launch writing ~1 GiB into slot 0 and slot `other` (0 = the reference alone)
+  int time(int other, float* ms) {
+    char* a = static_cast<char*>(window);
+    char* b = a + (size_t)other * chunk;
+    const uint32_t tiles = (uint32_t)(chunk / 16384);
+    const uint32_t grid = 1u << 20;                       // 1 Mi workgroups x 1 KiB
+    for (int i = 0; i < 2; ++i)
+      hipLaunchKernelGGL(probe_kernel, dim3(grid), dim3(64), 0, stream, src, (uint64_t)src_bytes - 1, a, b, tiles);
+    BIKV_HIP(hipEventRecord(e0, stream));
+    for (int i = 0; i < 3; ++i)
+      hipLaunchKernelGGL(probe_kernel, dim3(grid), dim3(64), 0, stream, src, (uint64_t)src_bytes - 1, a, b, tiles);
+    BIKV_HIP(hipEventRecord(e1, stream));
+    BIKV_HIP(hipEventSynchronize(e1));
+    BIKV_HIP(hipGetLastError());
+    BIKV_HIP(hipEventElapsedTime(ms, e0, e1));
+    *ms /= 3;
+    return BIKV_OK;
+  }
+};
+
+void release_all(std::vector<hipMemGenericAllocationHandle_t>& v) {
+  for (auto h : v) (void)hipMemRelease(h);
+  v.clear();
+}
+
+}  // namespace
+
+extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, void** out) {
+  if (!out) return fail(BIKV_EINVAL, "null out");
+  *out = nullptr;
+  if (bytes <= 0) return fail(BIKV_EINVAL, "bytes must be positive");
+  if (placement != BIKV_PLACE_SPREAD && placement != BIKV_PLACE_SEQUENTIAL)
+    return fail(BIKV_EINVAL, "unknown placement %d", placement);
+  BIKV_DEVICE(device);
+  hipMemAllocationProp prop = hipMemAllocationProp();
+  prop.type = hipMemAllocationTypePinned;
+  prop.location.type = hipMemLocationTypeDevice;
+  prop.location.id = device;
+  size_t gran = 0;
+  BIKV_HIP(hipMemGetAllocationGranularity(&gran, &prop, hipMemAllocationGranularityRecommended));
+  // chunks of 256 MiB .. 1 GiB, about 32 per allocation: small enough to interleave a 5 GB pool 20 ways,
+  // large enough that the probe's footprint is far beyond any cache
+  size_t chunk = std::min<size_t>(size_t(1) << 30, std::max<size_t>(size_t(256) << 20, pow2_floor((size_t)bytes / 32)));
+  if (gran > 0 && chunk % gran) chunk = (chunk + gran - 1) / gran * gran;
+  const size_t n = ((size_t)bytes + chunk - 1) / chunk;
+  const size_t want_other = placement == BIKV_PLACE_SPREAD ? n / 2 : 0;
+  const size_t want_same = n - want_other;
+
+  std::vector<hipMemGenericAllocationHandle_t> same, other, fillers;
+  Prober pr;
+  int rc = BIKV_OK;
+  auto cleanup = [&]() {
+    pr.destroy();
+    release_all(same);
+    release_all(other);
+    release_all(fillers);
+  };
+  float t_ref = 0;
+  if (placement == BIKV_PLACE_SPREAD && n >= 2) {
+    rc = pr.init(device, chunk);
+    if (rc) { cleanup(); return rc; }
+  }
+  // Create chunks until both kinds are complete. Chunks beyond the wanted number of a kind are fillers:
+  // they only push the driver's allocator on towards the other half and are released at the end. A
+  // failed creation (memory exhausted) ends the search with whatever balance was reached.
+  size_t free_b = 0, total_b = 0;
+  BIKV_HIP(hipMemGetInfo(&free_b, &total_b));
+  const size_t reserve = size_t(2) << 30;     // never take the last 2 GiB of the device
+  while (same.size() < want_same || other.size() < want_other) {
+    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess || free_b < chunk + reserve) break;
+    hipMemGenericAllocationHandle_t h;
+    if (hipMemCreate(&h, chunk, &prop, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      break;
+    }
+    bool is_other = false;
+    if (pr.window) {
+      if (same.empty()) {
+        // the first chunk is the reference: time it alone
+        rc = pr.map(0, h);
+        if (!rc) rc = pr.time(0, &t_ref);
+      } else {
+        float t = 0;
+        rc = pr.map(1, h);
+        if (!rc) rc = pr.time(1, &t);
+        if (!rc) rc = pr.unmap(1);
+        is_other = !rc && t < 0.92f * t_ref;
+      }
+      if (rc) {
+        (void)hipMemRelease(h);
+        break;
+      }
+    }
+    if (is_other) {
+      if (other.size() < want_other) other.push_back(h); else fillers.push_back(h);
+    } else {
+      if (same.size() < want_same) same.push_back(h); else fillers.push_back(h);
+    }
+  }
+  if (pr.window && !same.empty()) (void)pr.unmap(0);
+  if (rc) { cleanup(); return rc; }
+  // what one kind lacks the other makes up (from the fillers), so that the allocation is complete
+  while (same.size() + other.size() < n && !fillers.empty()) {
+    same.push_back(fillers.back());
+    fillers.pop_back();
+  }
+  if (same.size() + other.size() < n) {
+    cleanup();
+    return fail(BIKV_EHIP, "out of device memory: %zu of %zu chunks of %zu bytes could be created", same.size() + other.size(), n, chunk);
+  }
+  const int n_fillers = (int)fillers.size();
+  release_all(fillers);
+  pr.destroy();
+  pr = Prober();
+
+  // map alternately: position k takes an "other" chunk whenever that keeps the two kinds evenly mixed
+  Allocation al;
+  al.device = device;
+  al.bytes = n * chunk;
+  al.chunk = chunk;
+  al.n_other = (int)other.size();
+  al.n_fillers = n_fillers;
+  hipError_t e = hipMemAddressReserve(&al.va, al.bytes, 0, nullptr, 0);
+  if (e != hipSuccess) { cleanup(); return fail_hip(e, "hipMemAddressReserve"); }
+  size_t is = 0, io = 0;
+  for (size_t k = 0; k < n && e == hipSuccess; ++k) {
+    const bool take_other = io < other.size() && (is >= same.size() || (io + 1) * n <= (k + 1) * other.size() + n / 2);
+    hipMemGenericAllocationHandle_t h = take_other ? other[io++] : same[is++];
+    e = hipMemMap(static_cast<char*>(al.va) + k * chunk, chunk, 0, h, 0);
+    if (e == hipSuccess) al.handles.push_back(h);
+  }
+  if (e == hipSuccess) {
+    hipMemAccessDesc acc = hipMemAccessDesc();
+    acc.location.type = hipMemLocationTypeDevice;
+    acc.location.id = device;
+    acc.flags = hipMemAccessFlagsProtReadWrite;
+    e = hipMemSetAccess(al.va, al.bytes, &acc, 1);
+  }
+  if (e != hipSuccess) {
+    if (!al.handles.empty()) (void)hipMemUnmap(al.va, al.handles.size() * chunk);
+    (void)hipMemAddressFree(al.va, al.bytes);
+    cleanup();
+    return fail_hip(e, "hipMemMap / hipMemSetAccess");
+  }
+  same.clear();
+  other.clear();
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_allocs[al.va] = al;
+  }
+  *out = al.va;
+  return BIKV_OK;
+}
+
+extern "C" int bikv_device_free(void* p) {
+  if (!p) return BIKV_OK;
+  Allocation al;
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_allocs.find(p);
+    if (it == g_allocs.end()) return fail(BIKV_EINVAL, "pointer was not returned by bikv_device_alloc");
+    al = it->second;
+    g_allocs.erase(it);
+  }
+  BIKV_DEVICE(al.device);
+  BIKV_HIP(hipDeviceSynchronize());
+  hipError_t e = hipMemUnmap(al.va, al.bytes);
+  release_all(al.handles);
+  const hipError_t e2 = hipMemAddressFree(al.va, al.bytes);
+  if (e != hipSuccess) return fail_hip(e, "hipMemUnmap");
+  if (e2 != hipSuccess) return fail_hip(e2, "hipMemAddressFree");
+  return BIKV_OK;
+}
+
+extern "C" int bikv_device_alloc_info(const void* p, bikv_alloc_info* info) {
+  if (!p || !info) return fail(BIKV_EINVAL, "null argument");
+  std::lock_guard<std::mutex> lk(g_mu);
+  auto it = g_allocs.find(const_cast<void*>(p));
+  if (it == g_allocs.end()) return fail(BIKV_EINVAL, "pointer was not returned by bikv_device_alloc");
+  info->bytes = (int64_t)it->second.bytes;
+  info->chunk_bytes = (int64_t)it->second.chunk;
+  info->n_chunks = (int32_t)it->second.handles.size();
+  info->n_other_half = it->second.n_other;
+  info->n_fillers = it->second.n_fillers;
+  info->reserved = 0;
+  return BIKV_OK;
+}

@@ -310,6 +310,36 @@ int bikv_d2h_copy(int device, void* host_dst, const void* dev_src, int64_t bytes
 int bikv_h2d_copy(int device, void* dev_dst, const void* host_src, int64_t bytes,
                   int64_t chunk_bytes /* 0 = one copy */, double* seconds_out);
 
+/* --------------------------------------------------------------------------------------------
+ * 3a. Device memory placed for this GPU's memory system (optional; no counterpart in the reference,
+ * which allocates its pools with torch: kvcache.py:38-43, Worker.py:74-78).
+ *
+ * On MI355X the physical address space behaves as two halves: a copy whose random writes all land in
+ * one half runs at 5.6-5.7 TB/s, the same writes spread over both at 6.6-6.7 TB/s; reads and sequential
+ * writes hardly care. Which half memory lies in depends on where the driver put it: a pool that fits one
+ * half (any pool below ~100 GB on an empty GPU) scatters 15-18 % slower than it could, and how a large
+ * hipMalloc straddles the boundary changes from one allocation to the next.
+ * bikv_device_alloc(BIKV_PLACE_SPREAD) builds the allocation from physical chunks (256 MiB - 1 GiB,
+ * hipMemCreate), tells the halves apart with a short timed scatter into pairs of chunks, keeps equal
+ * numbers of both kinds and maps them alternately into one virtual range, so that every window of the
+ * pool spreads its writes over both halves. To reach the second half it may transiently create (and
+ * release again) filler chunks up to the free memory of the device less 2 GiB: call it at start-up,
+ * before other large allocations. BIKV_PLACE_SEQUENTIAL maps the chunks in creation order, unprobed.
+ * The memory behaves like hipMalloc'd memory for kernels and copies; it cannot be exported over HIP IPC.
+ * Sizes are rounded up to whole chunks. ------------------------------------------------------------ */
+enum { BIKV_PLACE_SPREAD = 0, BIKV_PLACE_SEQUENTIAL = 1 };
+typedef struct bikv_alloc_info {
+  int64_t bytes;          /* mapped size (a whole number of chunks) */
+  int64_t chunk_bytes;
+  int32_t n_chunks;
+  int32_t n_other_half;   /* chunks the probe placed in the other half than the first chunk */
+  int32_t n_fillers;      /* chunks created on the way and released again */
+  int32_t reserved;
+} bikv_alloc_info;
+int bikv_device_alloc(int device, int64_t bytes, int32_t placement, void** out);
+int bikv_device_free(void* p);
+int bikv_device_alloc_info(const void* p, bikv_alloc_info* info);
+
 /* Pinned host memory (hipHostMalloc, mapped + portable). */
 int bikv_host_alloc(int64_t bytes, void** out);
 int bikv_host_free(void* p);

@@ -762,3 +762,63 @@ def test_duplicate_scatter_destinations_are_refused_in_debug_mode(bk, cuda):
         nhd.load_token_major(tm, ids)
     nhd.store_token_major(tm, torch.tensor([3, 4], dtype=torch.int64, device=cuda))
     nhd.check()
+
+
+def test_device_alloc_builds_a_pool_out_of_chunks_from_both_halves(bk, oracle, cuda, lib):
+    """bikv_device_alloc: memory made of physical chunks mapped into one range behaves like any device
+    memory — torch writes it, the movers gather from and scatter into it against the oracle — and its
+    bookkeeping adds up. (Whether the probe finds a second half depends on what else the GPU holds; the
+    test only requires that the allocation is complete and correct.)"""
+    import ctypes as C
+    from bikv_pagecopy import _lib
+    _announce("device allocator")
+    n_planes, n_pages, tile = 6, 9000, 16384                         # 885 MB: four chunks of 256 MiB
+    nbytes = n_planes * n_pages * tile
+    for spread in (True, False):
+        buf = bk.DeviceBuffer(nbytes, cuda, spread=spread)
+        info = buf.info
+        assert info["bytes"] >= nbytes and info["bytes"] % info["chunk_bytes"] == 0
+        assert info["n_chunks"] * info["chunk_bytes"] == info["bytes"] and info["chunk_bytes"] >= 256 << 20
+        assert 0 <= info["n_other_half"] <= info["n_chunks"] // 2
+        if not spread:
+            assert info["n_other_half"] == 0 and info["n_fillers"] == 0
+        t = buf.tensor
+        assert t.numel() == nbytes and t.dtype == torch.uint8 and t.device == cuda
+        rng = np.random.default_rng(401)
+        # the pages next to a chunk boundary are among the ones used: the pool is [planes, pages, tile] flat in
+        # memory, so boundary b falls on page (b * tiles_per_chunk) % n_pages of some plane
+        per_chunk = info["chunk_bytes"] // tile
+        edge = [(b * per_chunk) % n_pages for b in range(1, info["n_chunks"])]
+        edge = [p for e in edge for p in (e - 1, e) if 0 <= p < n_pages]
+        ids_all = np.unique(np.concatenate([np.arange(8), edge, rng.integers(0, n_pages, size=52)]))
+        assert ids_all.max() < n_pages and ids_all.min() >= 0
+        pool_h = rng.integers(0, 256, size=(n_planes, len(ids_all), tile), dtype=np.uint8)
+        pool_t = t.view(n_planes, n_pages, tile)
+        pool_t.zero_()
+        pool_t[:, torch.from_numpy(ids_all).to(cuda)] = torch.from_numpy(pool_h[:, : len(ids_all)]).to(cuda)
+        pool = bk.PagedKVPool.from_stacked(pool_t, plane_dims=1)
+        others = np.setdiff1d(ids_all, edge)
+        reqs = [np.concatenate([edge, others[rng.permutation(len(others))[: 20 - len(edge)]]]).astype(np.int64), ids_all[:7]]
+        assert len(reqs[0]) == 20
+        batch = pool.make_batch(reqs)
+        st, _ = pool.gather(batch)
+        pool.check()
+        pos = {int(p): i for i, p in enumerate(ids_all)}
+        want = np.concatenate([np.stack([pool_h[q, [pos[int(p)] for p in r]] for q in range(n_planes)]).reshape(-1) for r in reqs])
+        assert _to_np(st).tobytes() == want.tobytes(), spread
+        # scatter into pages that were zero, read back with torch
+        fresh = np.setdiff1d(np.arange(n_pages), ids_all)[:27]
+        sb = pool.make_batch([fresh[:20], fresh[20:27]], check_unique=True)
+        pool.scatter(sb, st)
+        pool.check()
+        got = pool_t[:, torch.from_numpy(fresh).to(cuda)].cpu().numpy()
+        assert got.tobytes() == np.stack([pool_h[q, [pos[int(p)] for p in np.concatenate(reqs)]] for q in range(n_planes)]).tobytes()
+        pool.close()
+        del pool_t, t, st
+        buf.free()
+        with pytest.raises(RuntimeError, match="freed"):
+            buf.tensor
+    assert lib.bikv_device_free(C.c_void_p(12345)) == _lib.EINVAL
+    p = C.c_void_p()
+    assert lib.bikv_device_alloc(0, 0, 0, C.byref(p)) == _lib.EINVAL
+    assert lib.bikv_device_alloc(0, 1 << 20, 7, C.byref(p)) == _lib.EINVAL
