@@ -63,6 +63,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-layout", dest="no_other_layout", action="store_true",
                     help="skip the second measurement with the other staging layout")
+    ap.add_argument("--pool-form", dest="pool_form", choices=["planar", "worker"], default="planar",
+                    help="planar: one [pages, tile] plane per (layer, K|V); worker: one [tokens, 2, heads, dim] tensor per "
+                         "layer with K and V interleaved token by token, as the reference's Worker holds its cache")
     ap.add_argument("--pool-pages", type=int, default=0, help="override the pool size (pages per plane)")
     ap.add_argument("--pool-alloc", choices=["planes", "stacked", "spread"], default="spread",
                     help="one torch tensor per (layer, K|V) plane, one stacked torch allocation, or one allocation "
@@ -122,11 +125,30 @@ def fill_random_bytes(t):
         flat[off: off + step].random_(0, 256)
 
 
-def make_pool(shape, dev, alloc="planes"):
+def make_pool(shape, dev, alloc="planes", form="planar"):
     """The pool as the serving engine holds it: one tensor per (layer, K|V) plane ("planes", as
     Bi-KV/Worker/Worker.py:74-78 keeps a list of per-layer caches), or one stacked allocation
-    ("stacked"). Returns (planes, scale planes or None); both index as planes[q] -> [n_pages, tile]."""
+    ("stacked"), or memory from bikv_device_alloc ("spread"). Returns (planes, scale planes or None); both
+    index as planes[q] -> [n_pages, tile]. With form "worker" the pool is one [tokens, 2, heads, dim] tensor
+    per layer (Bi-KV/Worker/Worker.py:74-78); the planes are then strided views [n_pages, page_tokens, row]
+    for checking, and the second value is the list of per-layer tensors."""
     import torch
+
+    if form == "worker":
+        # [tokens, 2, heads, dim] per layer; plane (l, k) is the strided view [pages, page_tokens, row] of it
+        import bikv_pagecopy as bk
+        if shape.scales:
+            raise SystemExit("bench: the worker form has no scale planes")
+        L, P = shape.layers, shape.page_tokens
+        row = shape.tile_bytes // P
+        n = L * shape.n_pages * P * 2 * row
+        arena = spread_empty(bk, n, dev, f"{shape.name} pool, worker form") if alloc == "spread" else \
+            torch.empty(n, dtype=torch.uint8, device=dev)
+        fill_random_bytes(arena)
+        a5 = arena.view(L, shape.n_pages, P, 2, row)
+        el = arena.view(torch.float16 if shape.elem_bytes == 2 else torch.uint8)
+        layers = list(el.view(L, shape.n_pages * P, 2, shape.kv_heads, shape.head_dim).unbind(0))
+        return [a5[l, :, :, k] for l in range(L) for k in (0, 1)], layers
 
     def one(tile_bytes):
         if alloc == "spread":
@@ -163,7 +185,7 @@ def verify_on_device(pool_t, staging, batch, requests, n_full=2):
         for q in (range(n_planes) if r in full else some):
             want = torch.index_select(pool_t[q], 0, idt)
             got = view[q] if batch.layout == "layer_major" else view[:, q]
-            if not torch.equal(got, want):
+            if not torch.equal(got.reshape(want.shape), want):
                 return False, checked, len(nonempty) * n_planes
             checked += 1
     return True, checked, len(nonempty) * n_planes
@@ -275,7 +297,7 @@ TRAFFIC_SOURCE = "profiles/*_pmc.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of t
 
 
 def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layout=None, steps=None,
-                       warmup=None, target_s=None, keep_pool=False):
+                       warmup=None, target_s=None, keep_pool=False, pool_form=None):
     """One named configuration at full size: pool resident in HBM, one launch per direction (more when the
     staging image would exceed --staging-cap-gb), `steps` timed steps (or as many as fill `target_s`
     seconds). Returns (json fragment, shape, workload, kept) — kept = (pool_t, pool) when keep_pool."""
@@ -291,11 +313,22 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layo
         shape = shape.scaled(args.pool_pages)
     wl = workloads.named(name, shape)
     log(f"{name}: pool {shape.pool_bytes / 1e9:.2f} GB, tile {shape.tile_bytes} B x {shape.n_planes} planes, layout {layout}")
-    pool_t, scale_t = make_pool(shape, dev, args.pool_alloc)
-    pool = bk.PagedKVPool.from_planes(pool_t, scale_t)
+    pool_form = pool_form or args.pool_form
+    pool_t, scale_t = make_pool(shape, dev, args.pool_alloc, pool_form)
+    if pool_form == "worker":                       # second value = the per-layer tensors, not scale planes
+        pool, scale_t = bk.PagedKVPool.from_token_kv_layers(scale_t, shape.page_tokens), None
+    else:
+        pool = bk.PagedKVPool.from_planes(pool_t, scale_t)
 
     g_reqs = wl["gather"]
     s_reqs = wl.get("scatter") or []
+    if pool_form == "worker" and not s_reqs:
+        # the named workload only gathers; the Worker also writes received pages into this pool, so the same
+        # request lengths are scattered to fresh unique pages as well
+        perm, o = np.random.default_rng(7).permutation(shape.n_pages), 0
+        for r in g_reqs:
+            s_reqs.append(perm[o: o + len(r)].astype(np.int64))
+            o += len(r)
 
     # A launch covers as many whole requests as fit a staging buffer of --staging-cap-gb; the
     # Qwen2-7B-shaped batch fits in one launch per direction, the 70B-shaped one needs a few.
@@ -407,7 +440,7 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layo
     kname = "bikv::tile_move_wave_kernel<0=gather>" if dominant_is_gather else "bikv::tile_move_wave_kernel<1=scatter>"
     dom = g_stat if dominant_is_gather else s_stat
     ratio = MEASURED_TRAFFIC_RATIO.get(name, {}).get("gather" if dominant_is_gather else "scatter")
-    if args.pool_pages or layout != "layer_major":
+    if args.pool_pages or layout != "layer_major" or pool_form == "worker":
         ratio = None                                   # measured on the full-size layer-major workload only
     out = {
         "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
@@ -418,7 +451,10 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layo
                                f"{shape.kv_heads} heads x {shape.head_dim} {shape.dtype}"
                                f"{' + fp32 scales' if shape.scales else ''}; {len(g_reqs)} gather + {len(s_reqs)} "
                                f"scatter requests, {n_pages} pages/step in {len(g_groups)}+{len(s_groups)} launches, "
-                               f"layout {layout}",
+                               f"layout {layout}"
+                               + ("; pool held as one [tokens, 2, heads, dim] tensor per layer (the reference Worker's form: "
+                                  f"a tile is {shape.page_tokens} rows of {shape.tile_bytes // shape.page_tokens} B, two rows apart)"
+                                  if pool_form == "worker" else ""),
                    "pool_GB": round(shape.pool_bytes / 1e9, 2), "tile_bytes": shape.tile_bytes,
                    "planes": shape.n_planes,
                    "pool_alloc": ("bikv_device_alloc (physical chunks alternating between the halves of HBM)"
@@ -535,7 +571,21 @@ def run_staging(args, bk, workloads, dev, kept=None):
                 rates.append(total_bytes / (time.perf_counter() - t0) / 1e9)
         return {"GBps_min": round(min(rates), 2), "GBps_median": round(float(np.median(rates)), 2),
                 "plain_GBps_just_before": round(link, 2),
-                "frac_min": round(min(rates) / link, 4), "frac_median": round(float(np.median(rates)) / link, 4)}
+                "frac_min": round(min(rates) / link, 4), "frac_median": round(float(np.median(rates)) / link, 4),
+                "passes_GBps": [round(r, 2) for r in rates]}
+
+    def warm_up(stager, seconds):
+        """Untimed passes of the first cell's shape for a fixed time. Now and then a process spends its
+        first 7-15 s of staging at about 35 GB/s (seen with 4 MiB chunks out of the pool; the plain copy
+        timed next to it is at full rate) before it settles for good; the rates seen are kept in the record."""
+        seen, t_start = [], time.perf_counter()
+        while time.perf_counter() - t_start < seconds:
+            t0 = time.perf_counter()
+            for b, off, sz in zip(g_batches, offs, sizes):
+                stager.gather_to_host_async(pool, b, host[off: off + int(sz)], "pipelined")
+            stager.wait()
+            seen.append(round(total_bytes / (time.perf_counter() - t0) / 1e9, 2))
+        return {"seconds": seconds, "passes_GBps": seen}
 
     def verify(stager, mode):
         """Three requests (smallest, median, largest below 1 GiB) staged synchronously and compared, every
@@ -569,6 +619,7 @@ def run_staging(args, bk, workloads, dev, kept=None):
         stager = bk.HostStager(dev, chunk_bytes=chunk << 20, n_buffers=lanes, chunks_per_launch=group)
         if (chunk, lanes, group) == grid[0]:
             verify(stager, "pipelined")
+            warm = warm_up(stager, 0 if args.chunk_mib else 15.0)
         row = {"mode": "pipelined", "chunk_MiB": chunk, "lanes": lanes, "copies_per_launch": group}
         for direction in ("gather", "scatter"):
             row[direction + "_to_host" if direction == "gather" else "scatter_from_host"] = cell(stager, "pipelined", direction)
@@ -594,6 +645,7 @@ def run_staging(args, bk, workloads, dev, kept=None):
                        f"{len(reqs)} requests of {int(sizes.min() // shape.page_bytes)}..{int(sizes.max() // shape.page_bytes)} "
                        f"pages ({total_bytes / 1e9:.2f} GB per pass), enqueued back to back, {passes} timed passes per cell",
            "pool_GB": round(shape.pool_bytes / 1e9, 2),
+           "warm_up_before_the_first_cell": warm,
            "plain_d2h_GBps": {"min": round(min(yard["d2h"]), 2), "median": round(float(np.median(yard["d2h"])), 2),
                               "max": round(max(yard["d2h"]), 2), "samples": len(yard["d2h"])},
            "plain_h2d_GBps": {"min": round(min(yard["h2d"]), 2), "median": round(float(np.median(yard["h2d"])), 2),
@@ -801,7 +853,10 @@ def run_layout_change(args, bk, dev, blocks=None, sort=False, pool_alloc=None):
     pool = bk.NHDPool.from_token_kv_layers(layers, P)
     tm = torch.empty((n_pages, P, D, H, L, 2), dtype=torch.float16, device=dev)
     fill_random_bytes(tm)
-    tm_out = torch.empty_like(tm)
+    if pool_alloc == "spread" and args.staging_alloc in ("auto", "spread"):   # the written image, like a gather's
+        tm_out = spread_empty(bk, tm.numel() * 2, dev, "token-major image written by the store").view(torch.float16).view(tm.shape)
+    else:
+        tm_out = torch.empty_like(tm)
     rng = np.random.default_rng(6)
     ids_h = rng.permutation(blocks)[:n_pages].astype(np.int64)       # page i of tm <-> block ids_h[i]
     ids, pages = pool.page_list(ids_h, sort=sort, check_unique=True)
@@ -953,6 +1008,11 @@ def main():
             o, _, _, kept = run_gather_scatter(args, bk, workloads, dev, with_copy=False, name=other, target_s=1.0,
                                                warmup=3, keep_pool=keep)
             out["configs"][other] = config_summary(o)
+            if other == "qwen2_1p5b":
+                # the same shape held the way the reference's Worker holds it: [tokens, 2, heads, dim] per layer
+                o, _, _, _ = run_gather_scatter(args, bk, workloads, dev, with_copy=False, name=other, target_s=0.6,
+                                                warmup=3, pool_form="worker")
+                out["configs"]["qwen2_1p5b_worker_form"] = config_summary(o)
             if keep:
                 log("pinned-host staging on the Llama-3-8B pool")
                 out["staging"] = run_staging(args, bk, workloads, dev, kept)

@@ -203,9 +203,11 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
     if (value < 16 || value > (1 << 20)) return fail(BIKV_EINVAL, "small_run_max must be in [16, 1 MiB]");
     t.small_run_max = (int)value;
   } else if (!strcmp(key, "transpose_block")) {
-    if (value != 128 && value != 256 && value != 512 && value != 1024)
-      return fail(BIKV_EINVAL, "transpose_block must be 128, 256, 512 or 1024");
+    if (value != 0 && value != 128 && value != 256 && value != 512 && value != 1024)
+      return fail(BIKV_EINVAL, "transpose_block must be 0 (chosen per direction), 128, 256, 512 or 1024");
     t.transpose_block = (int)value;
+  } else if (!strcmp(key, "transpose_sc1")) {
+    t.transpose_sc1 = value ? 1 : 0;
   } else if (!strcmp(key, "transpose_pairs")) {
     t.transpose_pairs = value ? 1 : 0;
   } else if (!strcmp(key, "pair_rows")) {

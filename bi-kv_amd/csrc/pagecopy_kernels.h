@@ -64,7 +64,9 @@ struct Tuning {
   int transpose_lds_kib = 60;  // LDS tile budget of the layout-change kernels, KiB
   int transpose_dsplit = 0;    // slices of head_dim per tile; 0 = default (1: whole compute rows)
   int transpose_pairs = 1;     // the K/V-pair kernel where the shape allows (0 = element-wise kernel)
-  int transpose_block = 512;   // lanes per workgroup of the K/V-pair kernel: 128, 256, 512, 1024
+  int transpose_block = 0;     // lanes per workgroup of the K/V-pair kernel: 128, 256, 512, 1024;
+                               // 0 = chosen per direction (256 for the load, 512 for the store)
+  int transpose_sc1 = 1;       // K/V-pair kernel: payload stores are nt with system scope (0 = nt only)
   int debug_unique = 0;        // 1 = scattering entry points check their destination ids on the host first
   int pair_rows = 0;           // 1 = pools whose K and V rows interleave in 512-byte halves use the pair mover
                                // (measured 4-6 % SLOWER than the general wave mover: off by default)
@@ -108,6 +110,11 @@ struct TransposeArgs {
   int32_t chunk_cols, chunk_rows, pitch;      // filled by the launcher
   int32_t swz_mask;                           // pair kernel: XOR mask of the 16-byte groups of an LDS row
   uint32_t n_chunks, n_dchunks, tile_words;
+  // pair kernel, filled by the launcher: multipliers that replace divisions (m = ceil(2^32 / n), 0 for
+  // n = 1) and the per-step advance of its two index walks for the chosen workgroup size
+  uint32_t n_heads, m_heads, m_layers, m_vpr, m_dgs, m_chunks;
+  uint32_t q_tm, r_tm, q_cp, r_cp;
+  uint32_t sys_scope;             // payload stores carry system scope besides nt
   uint32_t* status;
 };
 // dir 0: compute -> token-major, dir 1: token-major -> compute.

@@ -168,24 +168,6 @@ __global__ __launch_bounds__(kBlock) void transpose_pages_kernel(const Transpose
 // above takes 11 and ~105 (three integer divisions per vector).
 // The XOR mask is the largest 2^k - 1 <= 7 with 2^k dividing the groups of a row, so that the permuted
 // index stays inside the row for every head_dim the entry points accept.
-struct Walk {        // (outer, inner) of a linear index that advances by the block size per step
-  int outer, inner;
-};
-__device__ __forceinline__ Walk walk_start(int idx, int n_inner) {
-  Walk w;
-  w.outer = idx / n_inner;
-  w.inner = idx - w.outer * n_inner;
-  return w;
-}
-__device__ __forceinline__ void walk_step(Walk& w, int q, int r, int n_inner) {
-  w.outer += q;
-  w.inner += r;
-  if (w.inner >= n_inner) {
-    w.inner -= n_inner;
-    w.outer += 1;
-  }
-}
-
 // 32 bytes of units {K,V} (g0 = the first 16, g1 = the next 16) -> a K vector and a V vector.
 template <int ES>
 __device__ __forceinline__ void split_kv(const u32x4& g0, const u32x4& g1, u32x4& kx, u32x4& vx) {
@@ -230,20 +212,55 @@ template <> struct UnitOf<1> { using T = uint16_t; };
 template <> struct UnitOf<2> { using T = uint32_t; };
 template <> struct UnitOf<4> { using T = uint64_t; };
 
+// Division of a small index by a divisor fixed at launch: the launcher passes m = ceil(2^32 / n) (0 when
+// n == 1) and the quotient is the high word of x * m, exact for x, n < 2^16. An integer division costs
+// ~25 instructions; a lane of this kernel moves only a handful of vectors, so three or four divisions
+// in its prologue were a third of all the vector instructions it issued.
+__device__ __forceinline__ uint32_t udiv_small(uint32_t x, uint32_t m) {
+  return m ? __umulhi(x, m) : x;
+}
+struct UWalk {       // (outer, inner) of a linear index that advances by the block size per step
+  uint32_t outer, inner;
+};
+__device__ __forceinline__ UWalk uwalk_start(uint32_t idx, uint32_t n_inner, uint32_t m) {
+  UWalk w;
+  w.outer = udiv_small(idx, m);
+  w.inner = idx - w.outer * n_inner;
+  return w;
+}
+__device__ __forceinline__ void uwalk_step(UWalk& w, uint32_t q, uint32_t r, uint32_t n_inner) {
+  w.outer += q;
+  w.inner += r;
+  if (w.inner >= n_inner) {
+    w.inner -= n_inner;
+    w.outer += 1;
+  }
+}
+
+// 16-byte payload store: nt, or nt with system scope (sc1), which has no C++ spelling for 16-byte accesses.
+__device__ __forceinline__ void store16(uint64_t p, const u32x4& v, bool sys) {
+  if (sys)
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(p), "v"(v) : "memory");
+  else
+    __builtin_nontemporal_store(v, (BIKV_GLOBAL u32x4*)p);
+}
+
 template <int DIR, int ES, int B>
 __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs a) {
   using Unit = typename UnitOf<ES>::T;
-  constexpr int UB = 2 * ES;               // bytes of a unit
-  constexpr int UPV = 16 / UB;             // units in a 16-byte vector
-  constexpr int UPV_SHIFT = ES == 1 ? 3 : (ES == 2 ? 2 : 1);
-  constexpr int DPV = 16 / ES;             // values of d in a compute-side vector
+  constexpr uint32_t UB = 2 * ES;               // bytes of a unit
+  constexpr uint32_t UPV = 16 / UB;             // units in a 16-byte vector
+  constexpr uint32_t UPV_SHIFT = ES == 1 ? 3 : (ES == 2 ? 2 : 1);
+  constexpr uint32_t DPV = 16 / ES;             // values of d in a compute-side vector
   extern __shared__ uint32_t lds_words[];
   u32x4* lds_vec = reinterpret_cast<u32x4*>(lds_words);
   Unit* lds_unit = reinterpret_cast<Unit*>(lds_words);
   uint64_t* row_addr = reinterpret_cast<uint64_t*>(lds_words + a.tile_words);  // K row of each pair
 
-  const uint32_t chunk = blockIdx.x % a.n_chunks;              // column chunk
-  const uint32_t t = blockIdx.x / a.n_chunks;                  // token within the page
+  const uint32_t tid = threadIdx.x;
+  const bool sys = a.sys_scope != 0;
+  const uint32_t t = udiv_small(blockIdx.x, a.m_chunks);       // token within the page
+  const uint32_t chunk = blockIdx.x - t * a.n_chunks;          // column chunk
   const uint64_t i = (uint64_t)blockIdx.y + (uint64_t)blockIdx.z * gridDim.y;
   if (i >= (uint64_t)a.n_pages) return;
   const int64_t blk = tload(a.block_ids + i);
@@ -251,145 +268,149 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
   const bool bad_blk = (uint64_t)blk >= (uint64_t)a.n_blocks;
   const bool bad_tm = (uint64_t)tmp >= (uint64_t)a.n_tm_pages;
   if (bad_blk || bad_tm) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
+    if (tid == 0 && blockIdx.x == 0) {
       if (bad_blk) *reinterpret_cast<volatile uint32_t*>(a.status + ST_SLOT_PAGE) = 1u;
       if (bad_tm) *reinterpret_cast<volatile uint32_t*>(a.status + (DIR == 0 ? ST_SLOT_DST : ST_SLOT_SRC)) = 1u;
     }
     return;
   }
-  const int D = a.head_dim, C = a.n_cols;
-  const int Cw = a.chunk_cols >> 1;        // column pairs in the tile
-  const int vpr = Cw >> UPV_SHIFT;         // 16-byte vectors per token-major row piece
-  const int dgs = D / DPV;                 // 16-byte vectors per compute row
-  const int gpr = (D * UB) >> 4;           // 16-byte groups per LDS row (even)
-  const int sm = a.swz_mask;               // 2^k - 1 with 2^k dividing gpr, at most 7
-  const int cp0 = (int)chunk * Cw;
+  const uint32_t D = (uint32_t)a.head_dim, C = (uint32_t)a.n_cols, L = (uint32_t)a.n_layers;
+  const uint32_t Cw = (uint32_t)a.chunk_cols >> 1;   // column pairs in the tile
+  const uint32_t vpr = Cw >> UPV_SHIFT;              // 16-byte vectors per token-major row piece
+  const uint32_t dgs = D / DPV;                      // 16-byte vectors per compute row
+  const uint32_t gpr = (D * UB) >> 4;                // 16-byte groups per LDS row (even)
+  const uint32_t sm = (uint32_t)a.swz_mask;          // 2^k - 1 with 2^k dividing gpr, at most 7
+  const uint32_t cp0 = chunk * Cw;
   // The compute side is walked layer by layer (all heads of a layer, K rows then V rows, are
   // neighbours in memory), the LDS tile is indexed by column pair (head-major): entry j of the table
   // holds the K row address of the j-th pair in walking order and, in its top 16 bits, that pair's
   // index in the tile. A tile that is only a column chunk of the token is walked in column order.
-  const int n_heads = C / (2 * a.n_layers);
-  for (int j = threadIdx.x; j < Cw; j += B) {
-    int h, l, cp;
+  const uint64_t tok_off = (uint64_t)(blk * a.block_stride + (int64_t)t * a.token_stride) * ES;   // uniform
+  auto pair_of = [&](uint32_t j, uint32_t& l, uint32_t& h, uint32_t& cp) {
     if (a.n_chunks == 1) {
-      l = j / n_heads;
-      h = j - l * n_heads;
-      cp = h * a.n_layers + l;
+      l = udiv_small(j, a.m_heads);
+      h = j - l * a.n_heads;
+      cp = h * L + l;
     } else {
       cp = j;
-      h = (cp0 + cp) / a.n_layers;
-      l = (cp0 + cp) - h * a.n_layers;
+      h = udiv_small(cp0 + cp, a.m_layers);
+      l = (cp0 + cp) - h * L;
     }
-    const int64_t off = blk * a.block_stride + (int64_t)t * a.token_stride + (int64_t)h * a.head_dim;
-    row_addr[j] = ((uint64_t)a.layer_base[l] + (uint64_t)off * ES) | ((uint64_t)cp << 48);
+  };
+  for (uint32_t j = tid; j < Cw; j += B) {
+    uint32_t h, l, cp;
+    pair_of(j, l, h, cp);
+    row_addr[j] = ((uint64_t)a.layer_base[l] + tok_off + (uint64_t)(h * D * ES)) | ((uint64_t)cp << 48);
   }
   const uint64_t kv_bytes = (uint64_t)a.kv_stride * ES;
-  const uint64_t tm_tok = (uint64_t)a.tm_base +
-                          (((uint64_t)(tmp * a.block_tokens + t) * D) * C + (uint64_t)cp0 * 2) * ES;
-  const uint64_t tm_row_bytes = (uint64_t)C * ES;
-  const int n_tm = D * vpr;                // vectors on the token-major side
-  const int n_cp = Cw * dgs;               // (pair, 16/ES values of d) items on the compute side
+  // token-major side: a uniform base and 32-bit offsets inside the token (a token is far below 4 GiB)
+  BIKV_GLOBAL char* tm_tok = (BIKV_GLOBAL char*)(uint64_t)a.tm_base +
+                             (((uint64_t)(tmp * a.block_tokens + t) * D) * C + (uint64_t)cp0 * 2) * ES;
+  const uint32_t tm_row_bytes = C * ES;
+  const uint32_t n_tm = D * vpr;                // vectors on the token-major side
+  const uint32_t n_cp = Cw * dgs;               // (pair, 16/ES values of d) items on the compute side
   // Unit (pair cp, d) sits in group (d / UPV) ^ s of row cp, s = (cp / UPV) & sm = the index of the
   // token-major vector the pair belongs to, mod 8 (mod a smaller power of two when the row has fewer
   // aligned groups, e.g. head_dim 80 at 2 bytes: 20 groups, mod 4).
 
   if (DIR == 1) {
     // token-major rows -> LDS, the units of a vector to as many pair rows
-    constexpr int U = 8;
-    const int q = B / vpr, r = B - q * vpr;
-    Walk w = walk_start(threadIdx.x, vpr);                     // (d, vector within the row piece)
-    for (int base = 0; base < n_tm; base += B * U) {
+    constexpr uint32_t U = 8;
+    UWalk w = uwalk_start(tid, vpr, a.m_vpr);                  // (d, vector within the row piece)
+    for (uint32_t base = 0; base < n_tm; base += B * U) {
       u32x4 x[U];
-      Walk wu = w;
+      UWalk wu = w;
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const bool ok = wu.outer < D;                          // a lane past the end re-reads row 0
-        const int d = ok ? wu.outer : 0;
-        x[u] = __builtin_nontemporal_load(
-            (const BIKV_GLOBAL u32x4*)(tm_tok + (uint64_t)d * tm_row_bytes + (uint64_t)wu.inner * 16));
-        walk_step(wu, q, r, vpr);
+      for (uint32_t u = 0; u < U; ++u) {
+        if (base + u * B >= n_tm) break;                       // whole workgroup past the end: nothing to load
+        const uint32_t d = wu.outer < D ? wu.outer : 0;        // a lane past the end re-reads row 0
+        x[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(tm_tok + (d * tm_row_bytes + wu.inner * 16)));
+        uwalk_step(wu, a.q_tm, a.r_tm, vpr);
       }
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
+      for (uint32_t u = 0; u < U; ++u) {
+        if (base + u * B >= n_tm) break;
         if (w.outer < D) {
-          const int cv = w.inner, d = w.outer;
+          const uint32_t cv = w.inner, d = w.outer;
           // unit index inside row (cv*UPV + j): group (d/UPV ^ s) * UPV + d % UPV
           Unit* row = lds_unit + (cv * UPV) * D + ((((d >> UPV_SHIFT) ^ (cv & sm)) << UPV_SHIFT) | (d & (UPV - 1)));
           Unit e[UPV];
           __builtin_memcpy(e, &x[u], 16);
 #pragma unroll
-          for (int j = 0; j < UPV; ++j) row[j * D] = e[j];
+          for (uint32_t j = 0; j < UPV; ++j) row[j * D] = e[j];
         }
-        walk_step(w, q, r, vpr);
+        uwalk_step(w, a.q_tm, a.r_tm, vpr);
       }
     }
     __syncthreads();
     // LDS -> compute rows: 32 bytes of units become one K vector and one V vector
-    const int q2 = B / dgs, r2 = B - q2 * dgs;
-    Walk o = walk_start(threadIdx.x, dgs);                     // (pair, group of d)
-    for (int base = 0; base < n_cp; base += B) {
+    UWalk o = uwalk_start(tid, dgs, a.m_dgs);                  // (pair, group of d)
+    for (uint32_t base = 0; base < n_cp; base += B) {
       if (o.outer < Cw) {
         const uint64_t entry = row_addr[o.outer];
-        const int cp = (int)(entry >> 48), dg = o.inner;
-        const int s = (cp >> UPV_SHIFT) & sm;
-        const int flip = (dg >> 2) & 1;                        // lanes 0-3 and 4-7 start on different halves
+        const uint32_t cp = (uint32_t)(entry >> 48), dg = o.inner;
+        const uint32_t s = (cp >> UPV_SHIFT) & sm;
+        const uint32_t flip = (dg >> 2) & 1;                   // lanes 0-3 and 4-7 start on different halves
         const u32x4 lo = lds_vec[cp * gpr + ((2 * dg + flip) ^ s)];
         const u32x4 hi = lds_vec[cp * gpr + ((2 * dg + 1 - flip) ^ s)];
         const u32x4 g0 = flip ? hi : lo, g1 = flip ? lo : hi;
         u32x4 kx, vx;
         split_kv<ES>(g0, g1, kx, vx);
-        const uint64_t ra = (entry & 0xFFFFFFFFFFFFull) + (uint64_t)dg * 16;
-        __builtin_nontemporal_store(kx, (BIKV_GLOBAL u32x4*)ra);
-        __builtin_nontemporal_store(vx, (BIKV_GLOBAL u32x4*)(ra + kv_bytes));
+        const uint64_t ra = (entry & 0xFFFFFFFFFFFFull) + (uint64_t)(dg * 16);
+        store16(ra, kx, sys);
+        store16(ra + kv_bytes, vx, sys);
       }
-      walk_step(o, q2, r2, dgs);
+      uwalk_step(o, a.q_cp, a.r_cp, dgs);
     }
   } else {
     // compute rows -> LDS: a K vector and a V vector interleave into 32 bytes of units
     __syncthreads();                                            // row_addr
-    constexpr int U = 4;
-    const int q2 = B / dgs, r2 = B - q2 * dgs;
-    Walk o = walk_start(threadIdx.x, dgs);
-    for (int base = 0; base < n_cp; base += B * U) {
+    constexpr uint32_t U = 4;
+    UWalk o = uwalk_start(tid, dgs, a.m_dgs);
+    for (uint32_t base = 0; base < n_cp; base += B * U) {
       u32x4 kx[U], vx[U];
-      Walk ou = o;
+      uint32_t cps[U];
+      UWalk ou = o;
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const bool ok = ou.outer < Cw;
-        const uint64_t ra = (row_addr[ok ? ou.outer : 0] & 0xFFFFFFFFFFFFull) + (uint64_t)ou.inner * 16;
+      for (uint32_t u = 0; u < U; ++u) {
+        if (base + u * B >= n_cp) break;                       // whole workgroup past the end: nothing to load
+        const uint32_t jj = ou.outer < Cw ? ou.outer : 0;      // a lane past the end re-reads row 0
+        const uint64_t entry = row_addr[jj];
+        cps[u] = (uint32_t)(entry >> 48);
+        const uint64_t ra = (entry & 0xFFFFFFFFFFFFull) + (uint64_t)(ou.inner * 16);
         kx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)ra);
         vx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(ra + kv_bytes));
-        walk_step(ou, q2, r2, dgs);
+        uwalk_step(ou, a.q_cp, a.r_cp, dgs);
       }
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
+      for (uint32_t u = 0; u < U; ++u) {
+        if (base + u * B >= n_cp) break;
         if (o.outer < Cw) {
-          const int cp = (int)(row_addr[o.outer] >> 48), dg = o.inner;
-          const int s = (cp >> UPV_SHIFT) & sm;
+          const uint32_t cp = cps[u], dg = o.inner;
+          const uint32_t s = (cp >> UPV_SHIFT) & sm;
+          const uint32_t flip = (dg >> 2) & 1;                 // as in the load: lanes 0-3 and 4-7 on different halves
           u32x4 g0, g1;
           join_kv<ES>(kx[u], vx[u], g0, g1);
-          lds_vec[cp * gpr + ((2 * dg) ^ s)] = g0;
-          lds_vec[cp * gpr + ((2 * dg + 1) ^ s)] = g1;
+          lds_vec[cp * gpr + ((2 * dg + flip) ^ s)] = flip ? g1 : g0;
+          lds_vec[cp * gpr + ((2 * dg + 1 - flip) ^ s)] = flip ? g0 : g1;
         }
-        walk_step(o, q2, r2, dgs);
+        uwalk_step(o, a.q_cp, a.r_cp, dgs);
       }
     }
     __syncthreads();
-    const int q = B / vpr, r = B - q * vpr;
-    Walk w = walk_start(threadIdx.x, vpr);
-    for (int base = 0; base < n_tm; base += B) {
+    UWalk w = uwalk_start(tid, vpr, a.m_vpr);
+    for (uint32_t base = 0; base < n_tm; base += B) {
       if (w.outer < D) {
-        const int cv = w.inner, d = w.outer;
+        const uint32_t cv = w.inner, d = w.outer;
         const Unit* row = lds_unit + (cv * UPV) * D + ((((d >> UPV_SHIFT) ^ (cv & sm)) << UPV_SHIFT) | (d & (UPV - 1)));
         Unit e[UPV];
 #pragma unroll
-        for (int j = 0; j < UPV; ++j) e[j] = row[j * D];
+        for (uint32_t j = 0; j < UPV; ++j) e[j] = row[j * D];
         u32x4 x;
         __builtin_memcpy(&x, e, 16);
-        __builtin_nontemporal_store(
-            x, (BIKV_GLOBAL u32x4*)(tm_tok + (uint64_t)d * tm_row_bytes + (uint64_t)cv * 16));
+        store16((uint64_t)(tm_tok + (d * tm_row_bytes + cv * 16)), x, sys);
       }
-      walk_step(w, q, r, vpr);
+      uwalk_step(w, a.q_tm, a.r_tm, vpr);
     }
   }
 }
@@ -440,9 +461,28 @@ hipError_t launch_transpose_pages(int dir, TransposeArgs& a, hipStream_t stream)
       const int64_t gx = (int64_t)a.n_chunks * a.block_tokens;
       const int64_t gy = a.n_pages < 32768 ? a.n_pages : 32768;
       const int64_t gz = (a.n_pages + gy - 1) / gy;
-      if (gx >= (int64_t(1) << 24) || gz > 65535) return hipErrorInvalidValue;
+      if (gx >= (int64_t(1) << 24) || gx * a.n_chunks > (int64_t(1) << 32) || gz > 65535) return hipErrorInvalidValue;
       const dim3 grid((uint32_t)gx, (uint32_t)gy, (uint32_t)gz);
-      const int block = tuning().transpose_block;
+      // The load writes the pool in KiB pieces and does best with many small workgroups in flight; the store
+      // reads them and does best with the waves of a tile sharing one workgroup (measured: 256 / 512 lanes).
+      const int block = tuning().transpose_block > 0 ? tuning().transpose_block : (dir == 1 ? 256 : 512);
+      // divisors of the kernel's index arithmetic as multipliers (see udiv_small); all are far below 2^16
+      const uint32_t cw = (uint32_t)best / 2, upv = 16u / (2u * (uint32_t)ES);
+      const uint32_t vpr = cw / upv, dgs = (uint32_t)D / (uint32_t)VE;
+      const uint32_t n_heads = (uint32_t)C / (2u * (uint32_t)a.n_layers);
+      if (vpr == 0 || dgs == 0 || n_heads == 0 || C >= 65536 || D >= 65536) return hipErrorInvalidValue;
+      auto magic = [](uint32_t n) { return n <= 1 ? 0u : (uint32_t)(((uint64_t(1) << 32) + n - 1) / n); };
+      a.n_heads = n_heads;
+      a.m_heads = magic(n_heads);
+      a.m_layers = magic((uint32_t)a.n_layers);
+      a.m_vpr = magic(vpr);
+      a.m_dgs = magic(dgs);
+      a.m_chunks = magic(a.n_chunks);
+      a.sys_scope = (uint32_t)tuning().transpose_sc1;
+      a.q_tm = (uint32_t)block / vpr;
+      a.r_tm = (uint32_t)block % vpr;
+      a.q_cp = (uint32_t)block / dgs;
+      a.r_cp = (uint32_t)block % dgs;
 #define BIKV_LAUNCH_PAIRS(DIR_, ES_, B_) \
   hipLaunchKernelGGL((transpose_pairs_kernel<DIR_, ES_, B_>), grid, dim3(B_), lds, stream, a)
 #define BIKV_LAUNCH_PAIRS_B(DIR_, ES_)                         \

@@ -76,7 +76,9 @@ int bikv_check_status(int device, void* stream, uint32_t* bits_out);
  * many bytes use one lane per 16-byte piece instead of one wave per KiB), "run_group" (1 = several
  * short runs share a row of the launch grid, default; 0 = one row per run), "transpose_lds_kib" and
  * "transpose_dsplit" (LDS tile budget and head_dim slices of the layout-change kernel),
- * "transpose_pairs" (1 = the K/V-pair kernel, default; 0 = the element-wise kernel) and "transpose_block" (its lanes per workgroup: 128, 256, 512, 1024),
+ * "transpose_pairs" (1 = the K/V-pair kernel, default; 0 = the element-wise kernel), "transpose_block"
+ * (its lanes per workgroup: 128, 256, 512, 1024; 0 = default: 256 for the load, 512 for the store) and
+ * "transpose_sc1" (1 = its payload stores are nt with system scope, default; 0 = nt only),
  * "debug_unique" (1 = what BIKV_DEBUG_UNIQUE=1 in the environment switches on, see bikv_find_duplicate),
  * "pair_rows" (1 = pools whose K and V rows interleave in 512-byte halves, the Worker's own tensors at
  * 2 KV heads x 128 x fp16, are moved two tokens at a time with the halves exchanged between lanes, so

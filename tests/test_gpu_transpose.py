@@ -93,7 +93,7 @@ def test_word_pair_kernel_at_other_workgroup_sizes(lib, oracle, cuda, block):
         oracle.transpose_pages_c(layers_h, "block_kv", tm_h, ids2, pages2, "store")
         assert _to_np(tm_d).tobytes() == tm_h.tobytes()
     finally:
-        bk.set_tuning(transpose_block=512)
+        bk.reset_tuning()
 
 
 def test_default_tm_pages_is_a_dense_received_buffer(lib, oracle, cuda):
