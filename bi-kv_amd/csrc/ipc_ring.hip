@@ -162,6 +162,43 @@ void ring_publish(bikv_shared_control* c, size_t at, size_t data_size, const int
 
 }  // namespace
 
+// Maps the named control block into this process: `create` makes a fresh object of the block's size
+// (replacing a stale one of the same name, exclusive, mode 0666 as ipc_service.cpp:33-35 does), otherwise an
+// existing object is opened and must be at least that large. On failure nothing is left open, and a
+// created object is removed again.
+static int map_control(const char* name, bool create, const char* who, Role* r) {
+  if (create) shm_unlink(name);
+  r->fd = shm_open(name, create ? (O_CREAT | O_RDWR | O_EXCL) : O_RDWR, 0666);
+  if (r->fd == -1) return fail(BIKV_ESYS, "%s shm_open failed: %s", who, strerror(errno));
+  const char* what = nullptr;
+  int err = 0;
+  if (create) {
+    if (ftruncate(r->fd, sizeof(bikv_shared_control)) == -1) what = "ftruncate", err = errno;
+  } else {
+    struct stat sb;
+    if (fstat(r->fd, &sb) == -1 || (size_t)sb.st_size < sizeof(bikv_shared_control)) {
+      close(r->fd);
+      r->fd = -1;
+      return fail(BIKV_ESYS, "%s: shared object is smaller than the control block", who);
+    }
+  }
+  if (!what) {
+    void* m = mmap(nullptr, sizeof(bikv_shared_control), PROT_READ | PROT_WRITE, MAP_SHARED, r->fd, 0);
+    if (m == MAP_FAILED) what = "mmap", err = errno;
+    else r->ctrl = static_cast<bikv_shared_control*>(m);
+  }
+  if (what) {
+    close(r->fd);
+    r->fd = -1;
+    if (create) shm_unlink(name);
+    return fail(BIKV_ESYS, "%s %s failed: %s", who, what, strerror(err));
+  }
+  return BIKV_OK;
+}
+
+// The consumer owns the ring: device memory first, then the control block that describes it. The block is
+// filled in one go from a local image, so a producer that opens it early sees either zeros (refused: ring
+// size 0) or the finished description, never half of one.
 extern "C" int bikv_consumer_init(int device, const char* shm_name, size_t buffer_bytes) {
   if (!shm_name || !*shm_name) return fail(BIKV_EINVAL, "shm_name is empty");
   if (strlen(shm_name) >= sizeof(g_consumer.shm_name)) return fail(BIKV_EINVAL, "shm_name too long");
@@ -172,114 +209,84 @@ extern "C" int bikv_consumer_init(int device, const char* shm_name, size_t buffe
   r.device = device;
   strncpy(r.shm_name, shm_name, sizeof(r.shm_name) - 1);
 
-  shm_unlink(shm_name);  // make sure no stale object is left, as the reference does
-  r.fd = shm_open(shm_name, O_CREAT | O_RDWR | O_EXCL, 0666);
-  if (r.fd == -1) return fail(BIKV_ESYS, "consumer_init shm_open failed: %s", strerror(errno));
-  if (ftruncate(r.fd, sizeof(bikv_shared_control)) == -1) {
-    const int e = errno;
-    close(r.fd);
-    shm_unlink(shm_name);
-    return fail(BIKV_ESYS, "consumer_init ftruncate failed: %s", strerror(e));
-  }
-  void* m = mmap(nullptr, sizeof(bikv_shared_control), PROT_READ | PROT_WRITE, MAP_SHARED, r.fd, 0);
-  if (m == MAP_FAILED) {
-    const int e = errno;
-    close(r.fd);
-    shm_unlink(shm_name);
-    return fail(BIKV_ESYS, "consumer_init mmap failed: %s", strerror(e));
-  }
-  r.ctrl = static_cast<bikv_shared_control*>(m);
-  memset(r.ctrl, 0, sizeof(bikv_shared_control));
-  sem_init(sem_of(r.ctrl->sem_start), 1, 0);
-  sem_init(sem_of(r.ctrl->sem_complete), 1, 0);
-  gethostname(r.ctrl->hostname, sizeof(r.ctrl->hostname));
-  r.ctrl->current_offset = 0;
-  r.ctrl->last_valid_offset = 0;
-  r.ctrl->device_id = device;
-  r.ctrl->buffer_size = buffer_bytes;
-
+  bikv_shared_control image;
+  memset(&image, 0, sizeof(image));
+  image.device_id = device;
+  image.buffer_size = buffer_bytes;
+  gethostname(image.hostname, sizeof(image.hostname));
   hipError_t e = hipMalloc(&r.mem, buffer_bytes);
-  if (e != hipSuccess) {
-    unmap_role(r);
-    shm_unlink(shm_name);
-    return fail(BIKV_EHIP, "consumer_init hipMalloc failed: %s", hipGetErrorString(e));
-  }
+  if (e != hipSuccess) return fail(BIKV_EHIP, "consumer_init hipMalloc failed: %s", hipGetErrorString(e));
   // A ring of 2 GiB or more is never exported: IPC mappings that large have been seen not to return
   // on some ROCm hosts. Its handle stays zeroed, a producer in another process is refused
   // (bikv_producer_init), and a producer in this process uses the pointer directly.
   if (buffer_bytes < kMaxIpcBytes) {
+    static_assert(sizeof(hipIpcMemHandle_t) <= sizeof(image.ipc_handle), "IPC handle does not fit the control block");
     hipIpcMemHandle_t handle;
     memset(&handle, 0, sizeof(handle));
     e = hipIpcGetMemHandle(&handle, r.mem);
     if (e != hipSuccess) {
       (void)hipFree(r.mem);
-      unmap_role(r);
-      shm_unlink(shm_name);
       return fail(BIKV_EHIP, "consumer_init hipIpcGetMemHandle failed: %s", hipGetErrorString(e));
     }
-    memcpy(r.ctrl->ipc_handle, &handle, sizeof(handle));
+    memcpy(image.ipc_handle, &handle, sizeof(handle));
   }
+  const int rc = map_control(shm_name, true, "consumer_init", &r);
+  if (rc != BIKV_OK) {
+    (void)hipFree(r.mem);
+    return rc;
+  }
+  memcpy(r.ctrl, &image, sizeof(image));
+  sem_init(sem_of(r.ctrl->sem_start), 1, 0);
+  sem_init(sem_of(r.ctrl->sem_complete), 1, 0);
   g_consumer = r;
   return BIKV_OK;
 }
 
+// The producer attaches to a ring some consumer described: the control block is opened and checked before
+// the GPU is touched, so that a missing object or a foreign host is reported as such whatever the state of
+// the device.
 extern "C" int bikv_producer_init(int device, const char* shm_name) {
   if (!shm_name || !*shm_name) return fail(BIKV_EINVAL, "shm_name is empty");
   if (g_producer.ctrl) return fail(BIKV_ESTATE, "producer already initialised (call producer_cleanup first)");
-  // The control block is opened and checked before the GPU is touched, so that a missing object
-  // or a foreign host is reported as such whatever the state of the device.
   Role r;
   r.device = device;
   strncpy(r.shm_name, shm_name, sizeof(r.shm_name) - 1);
-  r.fd = shm_open(shm_name, O_RDWR, 0666);
-  if (r.fd == -1) return fail(BIKV_ESYS, "producer_init shm_open failed: %s", strerror(errno));
-  struct stat sb;
-  if (fstat(r.fd, &sb) == -1 || (size_t)sb.st_size < sizeof(bikv_shared_control)) {
-    close(r.fd);
-    return fail(BIKV_ESYS, "producer_init: shared object is smaller than the control block");
-  }
-  void* m = mmap(nullptr, sizeof(bikv_shared_control), PROT_READ | PROT_WRITE, MAP_SHARED, r.fd, 0);
-  if (m == MAP_FAILED) {
-    const int e = errno;
-    close(r.fd);
-    return fail(BIKV_ESYS, "producer_init mmap failed: %s", strerror(e));
-  }
-  r.ctrl = static_cast<bikv_shared_control*>(m);
-  char host[256];
+  int rc = map_control(shm_name, false, "producer_init", &r);
+  if (rc != BIKV_OK) return rc;
+  const bool same_process = g_consumer.ctrl && strcmp(g_consumer.shm_name, shm_name) == 0;
+  const size_t ring_bytes = r.ctrl->buffer_size;
+  char host[sizeof(r.ctrl->hostname)];
   memset(host, 0, sizeof(host));
   gethostname(host, sizeof(host));
-  if (strncmp(host, r.ctrl->hostname, sizeof(host)) != 0) {
-    unmap_role(r);
-    return fail(BIKV_ESTATE, "Processes must run on the same host");
+  const bool foreign = strncmp(host, r.ctrl->hostname, sizeof(host)) != 0;
+  if (ring_bytes == 0 && (r.ctrl->hostname[0] == '\0' || !foreign))
+    rc = fail(BIKV_ESTATE, "producer_init: the control block describes no ring yet (the consumer is still initialising)");
+  else if (foreign)
+    rc = fail(BIKV_ESTATE, "Processes must run on the same host");
+  else if (!same_process && ring_bytes >= kMaxIpcBytes)
+    // Mapping another process's allocation of 2 GiB or more has been seen not to return on some ROCm
+    // hosts; the consumer does not export a handle for such a ring and it is refused here.
+    rc = fail(BIKV_ERANGE, "the consumer's ring is %zu bytes: IPC mappings of 2 GiB or more are refused "
+                           "(use a ring below 2 GiB, or run producer and consumer in one process)", ring_bytes);
+  if (rc == BIKV_OK) {
+    const hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) rc = fail_hip(e, "hipSetDevice");
   }
-  const bool same_process = g_consumer.ctrl && strcmp(g_consumer.shm_name, shm_name) == 0;
-  // Mapping another process's allocation of 2 GiB or more has been seen not to return on some
-  // ROCm hosts; the consumer does not export a handle for such a ring and it is refused here.
-  if (!same_process && r.ctrl->buffer_size >= kMaxIpcBytes) {
-    const size_t bytes = r.ctrl->buffer_size;
-    unmap_role(r);
-    return fail(BIKV_ERANGE, "the consumer's ring is %zu bytes: IPC mappings of 2 GiB or more are refused "
-                             "(use a ring below 2 GiB, or run producer and consumer in one process)", bytes);
-  }
-  {
-    hipError_t e = hipSetDevice(device);
-    if (e != hipSuccess) {
-      unmap_role(r);
-      return fail_hip(e, "hipSetDevice");
+  if (rc == BIKV_OK) {
+    if (same_process) {
+      r.mem = g_consumer.mem;  // same process: no IPC mapping needed (or possible)
+      r.ipc_mapped = false;
+    } else {
+      hipIpcMemHandle_t handle;
+      memcpy(&handle, r.ctrl->ipc_handle, sizeof(handle));
+      const hipError_t e = hipIpcOpenMemHandle(&r.mem, handle, hipIpcMemLazyEnablePeerAccess);
+      if (e != hipSuccess) rc = fail(BIKV_EHIP, "producer_init hipIpcOpenMemHandle failed: %s", hipGetErrorString(e));
+      r.ipc_mapped = e == hipSuccess;
     }
   }
-  if (same_process) {
-    r.mem = g_consumer.mem;  // same process: no IPC mapping needed (or possible)
-    r.ipc_mapped = false;
-  } else {
-    hipIpcMemHandle_t handle;
-    memcpy(&handle, r.ctrl->ipc_handle, sizeof(handle));
-    hipError_t e = hipIpcOpenMemHandle(&r.mem, handle, hipIpcMemLazyEnablePeerAccess);
-    if (e != hipSuccess) {
-      unmap_role(r);
-      return fail(BIKV_EHIP, "producer_init hipIpcOpenMemHandle failed: %s", hipGetErrorString(e));
-    }
-    r.ipc_mapped = true;
+  if (rc != BIKV_OK) {
+    unmap_role(r);
+    return rc;
   }
   g_producer = r;
   return BIKV_OK;

@@ -443,11 +443,14 @@ typedef struct bikv_tensor_dims {
   int64_t kv_pair;
 } bikv_tensor_dims;
 
-/* consumer_init (ipc_service.cpp:20-74): unlink+create shm, init semaphores, record hostname and
- * device, allocate the device ring, publish its IPC handle. A ring of 2 GiB or more is not exported
- * (its handle stays zeroed): only a producer in the consumer's own process can use it. */
+/* consumer_init (ipc_service.cpp:20-74): allocates the device ring and its IPC handle, then creates the
+ * named control block (a stale object of that name is replaced) and fills it in one go: hostname, device,
+ * ring size, handle, both semaphores at 0. Unlike the reference, which creates the block first and fills it
+ * field by field around the allocation, a producer never finds a half-described ring. A ring of 2 GiB or
+ * more is not exported (its handle stays zeroed): only a producer in the consumer's own process can use it. */
 int bikv_consumer_init(int device, const char* shm_name, size_t buffer_bytes);
-/* producer_init (ipc_service.cpp:77-110): open shm, same-host check, map the ring. A producer in
+/* producer_init (ipc_service.cpp:77-110): open shm, same-host check, map the ring. A control block that
+ * describes no ring yet (all zeros: the consumer is between creating and filling it) is BIKV_ESTATE. A producer in
  * ANOTHER process than the consumer refuses a ring of 2 GiB or more with BIKV_ERANGE (opening an IPC
  * mapping that large has been seen not to return on some ROCm hosts). */
 int bikv_producer_init(int device, const char* shm_name);

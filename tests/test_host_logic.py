@@ -122,6 +122,10 @@ def test_producer_init_rejects_a_control_block_from_another_host(lib):
         with pytest.raises(RuntimeError, match="same host"):
             ipc_service.producer_init(0, name.encode())
         with open(path, "wb") as f:
+            f.write(bytes(SharedControl()))  # created but not filled in yet: no ring to attach to
+        with pytest.raises(RuntimeError, match="describes no ring yet"):
+            ipc_service.producer_init(0, name)
+        with open(path, "wb") as f:
             f.write(b"\0" * 100)  # too small to be a control block
         with pytest.raises(RuntimeError, match="smaller than the control block"):
             ipc_service.producer_init(0, name)
