@@ -39,6 +39,8 @@ def _make(rng, form, es, P, D, H, L, blocks, n_tm, cuda):
     (1, 3, 64, 2, 4),        # 1-byte elements, the smallest pair-kernel shape (one vector per row)
     (4, 2, 16, 3, 2),        # 4-byte elements, head_dim 16
     (4, 3, 128, 4, 16),      # fp32, 128 columns: chunked
+    (2, 4, 64, 4, 1),        # a single layer
+    (2, 64, 128, 8, 32),     # 64 tokens per block x four column chunks: 256 workgroups per page
 ])
 @pytest.mark.parametrize("pairs", [1, 0])
 def test_load_and_store_match_oracle(lib, oracle, cuda, form, es, P, D, H, L, pairs):
