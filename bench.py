@@ -49,7 +49,7 @@ MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9948, "scatter": 1.0002},
                           "qwen2_1p5b": {"gather": 1.0009},
                           "llama3_8b": {"gather": 0.9967},
                           "llama3_70b_fp8": {"gather": 1.0142, "scatter": 1.0001},
-                          "qwen2_7b_token_major": {"gather": 0.9997, "scatter": 1.0002},
+                          "qwen2_7b_token_major": {"gather": 0.9998, "scatter": 1.0002},
                           "layout_change": {"load": 1.0029, "store": 1.0035}}
 
 
@@ -293,7 +293,7 @@ def cpu_baseline(shape, wl, budget_s=12.0):
 # Where the `traffic` figures come from: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, kept as
 # summaries under profiles/. They are NOT measured by the run that prints them (counters need the
 # profiler); a run only multiplies its own algorithmic bytes by the ratio recorded there.
-TRAFFIC_SOURCE = "profiles/*_pmc.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this command; not measured in this run)"
+TRAFFIC_SOURCE = "profiles/<kernel>_<workload>.md (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this workload; not measured in this run)"
 
 
 def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layout=None, steps=None,
@@ -756,12 +756,18 @@ def run_token_major(args, bk, workloads, dev):
         shape = shape.scaled(args.pool_pages)
     wl = workloads.named("qwen2_7b", shape)
     page_elems = shape.page_bytes // 2
-    pool = torch.empty(shape.n_pages * page_elems, dtype=torch.bfloat16, device=dev)
-    fill_random_bytes(pool)
     g_ids = np.concatenate(wl["gather"]).astype(np.int64)
     s_ids = np.concatenate(wl["scatter"]).astype(np.int64)
     n_g, n_s = len(g_ids), len(s_ids)
-    dense = torch.empty(max(n_g, n_s) * page_elems, dtype=torch.bfloat16, device=dev)
+    if args.pool_alloc == "spread":
+        pool = spread_empty(bk, shape.n_pages * page_elems * 2, dev, "token-major pool").view(torch.bfloat16)
+    else:
+        pool = torch.empty(shape.n_pages * page_elems, dtype=torch.bfloat16, device=dev)
+    fill_random_bytes(pool)
+    if args.staging_alloc in ("auto", "spread"):     # the gather writes it, the scatter reads it
+        dense = spread_empty(bk, max(n_g, n_s) * page_elems * 2, dev, "dense buffer").view(torch.bfloat16)
+    else:
+        dense = torch.empty(max(n_g, n_s) * page_elems, dtype=torch.bfloat16, device=dev)
     g_src = torch.from_numpy(g_ids * page_elems).to(dev)
     s_dst = torch.from_numpy(s_ids * page_elems).to(dev)
     g_dst = torch.arange(n_g, dtype=torch.int64, device=dev) * page_elems
@@ -814,11 +820,12 @@ def run_token_major(args, bk, workloads, dev):
         "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": f"qwen2_7b_token_major: {shape.n_pages} pages x {shape.page_bytes} B (16 tok x (128,4,28,2) bf16), "
                                f"{n_g} pages gathered + {n_s} scattered per step, one run per page",
-                   "pool_GB": round(shape.pool_bytes / 1e9, 2)},
+                   "pool_GB": round(shape.pool_bytes / 1e9, 2),
+                   "pool_alloc": "bikv_device_alloc" if args.pool_alloc == "spread" else "torch"},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "pages_per_s": round((n_g + n_s) / (wall / args.steps), 1), "bit_exact": True,
-        "kernels": {"gather": {"GBps": round(alg_g / g_ms / 1e6, 1), "avg_ms": round(g_ms, 4)},
-                    "scatter": {"GBps": round(alg_s / s_ms / 1e6, 1), "avg_ms": round(s_ms, 4)}},
+        "kernels": {"gather": {"GBps": round(alg_g / g_ms / 1e6, 1), "avg_ms": round(g_ms, 4), "alg_bytes": alg_g},
+                    "scatter": {"GBps": round(alg_s / s_ms / 1e6, 1), "avg_ms": round(s_ms, 4), "alg_bytes": alg_s}},
         "roofline": {"bound": "hbm", "kernel": "bikv::copy_runs_wave_kernel", "achieved": round(alg / ms / 1e6, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(alg / ms / 1e6 / HBM_PEAK_GBPS, 4),
                      "traffic": (int(alg * MEASURED_TRAFFIC_RATIO["qwen2_7b_token_major"]["gather" if slow_g else "scatter"])
