@@ -172,7 +172,6 @@ extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, v
   // they only push the driver's allocator on towards the other half and are released at the end. A
   // failed creation (memory exhausted) ends the search with whatever balance was reached.
   size_t free_b = 0, total_b = 0;
-  BIKV_HIP(hipMemGetInfo(&free_b, &total_b));
   const size_t reserve = size_t(2) << 30;     // never take the last 2 GiB of the device
   while (same.size() < want_same || other.size() < want_other) {
     if (hipMemGetInfo(&free_b, &total_b) != hipSuccess || free_b < chunk + reserve) break;
