@@ -619,7 +619,7 @@ def run_staging(args, bk, workloads, dev, kept=None):
         stager = bk.HostStager(dev, chunk_bytes=chunk << 20, n_buffers=lanes, chunks_per_launch=group)
         if (chunk, lanes, group) == grid[0]:
             verify(stager, "pipelined")
-            warm = warm_up(stager, 0 if args.chunk_mib else 15.0)
+            warm = warm_up(stager, 0 if args.chunk_mib else 20.0)
         row = {"mode": "pipelined", "chunk_MiB": chunk, "lanes": lanes, "copies_per_launch": group}
         for direction in ("gather", "scatter"):
             row[direction + "_to_host" if direction == "gather" else "scatter_from_host"] = cell(stager, "pipelined", direction)
