@@ -621,6 +621,8 @@ def run_staging(args, bk, workloads, dev, kept=None):
             verify(stager, "pipelined")
             warm = warm_up(stager, 0 if args.chunk_mib else 20.0)
         row = {"mode": "pipelined", "chunk_MiB": chunk, "lanes": lanes, "copies_per_launch": group}
+        if group == 1 and chunk < 16:
+            row["contrast_case"] = "one kernel per small copy: the shape that makes small chunks slow, shown for contrast only"
         for direction in ("gather", "scatter"):
             row[direction + "_to_host" if direction == "gather" else "scatter_from_host"] = cell(stager, "pipelined", direction)
         log(f"staging {row}")
@@ -656,6 +658,12 @@ def run_staging(args, bk, workloads, dev, kept=None):
            "scatter_from_host_GBps": auto["scatter_from_host"]["GBps_median"],
            "scatter_frac_of_plain_h2d": auto["scatter_from_host"]["frac_median"],
            "cells": cells, "per_request_blocking_calls": per_call, "bit_exact": True}
+    real = [c for c in cells if "contrast_case" not in c]
+    out["min_frac_over_cells"] = {
+        "gather_to_host": min(c["gather_to_host"]["frac_min"] for c in real),
+        "scatter_from_host": min(c["scatter_from_host"]["frac_min"] for c in real),
+        "what": "lowest single pass of any cell, as a fraction of the plain copy timed just before that cell "
+                "(every chunk size, lane count and mode above except the contrast case)"}
     if kept is None:
         pool.close()
         del pool_t
