@@ -551,14 +551,14 @@ def run_staging(args, bk, workloads, dev, kept=None):
     yard = {"d2h": [], "h2d": []}
 
     def cell(stager, mode, direction, synchronous=False):
+        untimed = 2 if stager.n_buffers <= 2 else 4     # a stager with four new lanes takes longer to settle
         d2h, h2d = link_yardstick(bk, dev, host[: dev_buf.numel()], dev_buf)
         yard["d2h"].append(d2h)
         yard["h2d"].append(h2d)
         link = d2h if direction == "gather" else h2d
         batches = g_batches if direction == "gather" else s_batches
         rates = []
-        for p in range(passes + 2):                      # the first two passes are a warm-up (a stager with
-                                                         # four new lanes needs more than one to settle)
+        for p in range(passes + untimed):
             t0 = time.perf_counter()
             for b, off, sz in zip(batches, offs, sizes):
                 win = host[off: off + int(sz)]
@@ -568,7 +568,7 @@ def run_staging(args, bk, workloads, dev, kept=None):
                     (stager.gather_to_host_async if direction == "gather" else stager.scatter_from_host_async)(pool, b, win, mode)
             if not synchronous:
                 stager.wait()
-            if p > 1:
+            if p >= untimed:
                 rates.append(total_bytes / (time.perf_counter() - t0) / 1e9)
         return {"GBps_min": round(min(rates), 2), "GBps_median": round(float(np.median(rates)), 2),
                 "plain_GBps_just_before": round(link, 2),
@@ -629,7 +629,7 @@ def run_staging(args, bk, workloads, dev, kept=None):
         log(f"staging {row}")
         cells.append(row)
         stager.close()
-    stager = bk.HostStager(dev)          # the library's defaults: 8 MiB x 4 per launch x 2 lanes
+    stager = bk.HostStager(dev)          # the library's defaults: 16 MiB x 2 per launch x 2 lanes
     verify(stager, "direct")
     for mode in ("direct", "auto"):
         row = {"mode": mode, "chunk_MiB": stager.chunk_bytes >> 20, "lanes": stager.n_buffers,
@@ -646,7 +646,7 @@ def run_staging(args, bk, workloads, dev, kept=None):
     auto = cells[-1]
     out = {"workload": f"llama3_8b: {shape.n_pages} pages x {shape.n_planes} planes x {shape.tile_bytes} B, "
                        f"{len(reqs)} requests of {int(sizes.min() // shape.page_bytes)}..{int(sizes.max() // shape.page_bytes)} "
-                       f"pages ({total_bytes / 1e9:.2f} GB per pass), enqueued back to back, {passes} timed passes per cell after two untimed ones",
+                       f"pages ({total_bytes / 1e9:.2f} GB per pass), enqueued back to back, {passes} timed passes per cell after two untimed ones (four for a stager with four lanes)",
            "pool_GB": round(shape.pool_bytes / 1e9, 2),
            "warm_up_before_the_first_cell": warm,
            "plain_d2h_GBps": {"min": round(min(yard["d2h"]), 2), "median": round(float(np.median(yard["d2h"])), 2),

@@ -26,11 +26,13 @@ def pinned_empty(nbytes: int) -> torch.Tensor:
 
 class HostStager:
     """`n_buffers` lanes (HIP stream + HBM buffer of `chunks_per_launch` x `chunk_bytes`). Mode "auto"
-    sends with the kernel storing straight into the pinned image ("direct") and receives through the
-    DMA engine ("pipelined"): on MI355X the device -> host DMA path runs at either ~30 or ~57 GB/s
-    depending on a platform state the library cannot see, kernel stores hold ~55 GB/s in both."""
+    sends with the kernel storing straight into the pinned image ("direct", a steady ~55.7 GB/s) and
+    receives through the DMA engine ("pipelined"): a hipMemcpyAsync device -> host behind a kernel is run by
+    the HIP runtime as a shader copy of its own, whose rate has been seen to start at 35 GB/s for seconds.
+    The defaults (two copies of 16 MiB per kernel launch, two lanes) measured 98.8 % of a plain pinned
+    copy host -> device; 8 MiB x 4 gives 97.7 %, 4 MiB x 4 95.6 %."""
 
-    def __init__(self, device, chunk_bytes: int = 8 << 20, n_buffers: int = 2, chunks_per_launch: int = 4):
+    def __init__(self, device, chunk_bytes: int = 16 << 20, n_buffers: int = 2, chunks_per_launch: int = 2):
         self.device = torch.device(device)
         self.chunk_bytes = int(chunk_bytes)
         self.n_buffers = int(n_buffers)
