@@ -154,6 +154,14 @@ extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, v
   const size_t want_other = placement == BIKV_PLACE_SPREAD ? n / 2 : 0;
   const size_t want_same = n - want_other;
 
+  const size_t reserve = size_t(2) << 30;     // never take the last 2 GiB of the device
+  {
+    size_t free_now = 0, total_now = 0;
+    BIKV_HIP(hipMemGetInfo(&free_now, &total_now));
+    if (n * chunk + reserve > free_now)
+      return fail(BIKV_EHIP, "out of device memory: %zu bytes asked for (%zu chunks of %zu), %zu free, 2 GiB kept back",
+                  (size_t)bytes, n, chunk, free_now);
+  }
   std::vector<hipMemGenericAllocationHandle_t> same, other, fillers;
   Prober pr;
   int rc = BIKV_OK;
@@ -172,7 +180,6 @@ extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, v
   // they only push the driver's allocator on towards the other half and are released at the end. A
   // failed creation (memory exhausted) ends the search with whatever balance was reached.
   size_t free_b = 0, total_b = 0;
-  const size_t reserve = size_t(2) << 30;     // never take the last 2 GiB of the device
   while (same.size() < want_same || other.size() < want_other) {
     if (hipMemGetInfo(&free_b, &total_b) != hipSuccess || free_b < chunk + reserve) break;
     hipMemGenericAllocationHandle_t h;

@@ -822,3 +822,6 @@ def test_device_alloc_builds_a_pool_out_of_chunks_from_both_halves(bk, oracle, c
     p = C.c_void_p()
     assert lib.bikv_device_alloc(0, 0, 0, C.byref(p)) == _lib.EINVAL
     assert lib.bikv_device_alloc(0, 1 << 20, 7, C.byref(p)) == _lib.EINVAL
+    # more than the device holds: refused at once, nothing created
+    assert lib.bikv_device_alloc(0, 1 << 42, 0, C.byref(p)) == _lib.EHIP and not p.value
+    assert b"out of device memory" in lib.bikv_last_error()
