@@ -825,3 +825,66 @@ def test_device_alloc_builds_a_pool_out_of_chunks_from_both_halves(bk, oracle, c
     # more than the device holds: refused at once, nothing created
     assert lib.bikv_device_alloc(0, 1 << 42, 0, C.byref(p)) == _lib.EHIP and not p.value
     assert b"out of device memory" in lib.bikv_last_error()
+
+
+# ---- several host threads -----------------------------------------------------------------------
+def test_four_host_threads_move_pages_through_one_pool(bk, oracle, cuda):
+    """The reference's callers are thread pools (20 gRPC workers per process, config.yml:53,60). Four host
+    threads, each on its own stream with its own batches, staging buffers and host stager, gather from and
+    scatter into one pool at the same time; every thread's results are checked against the oracle."""
+    import threading
+    _announce("four host threads on one pool")
+    n_planes, n_pages, tile, n_threads, rounds = 6, 4096, 4096, 4, 12
+    rng = np.random.default_rng(77)
+    pool_h = _rand_pool(rng, n_planes, n_pages, tile)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    perm = rng.permutation(n_pages)
+    half = n_pages // 2
+    # pages [0, half) of the permutation are only read, the rest only written: each thread owns a slice of both
+    per = half // n_threads
+    jobs = []
+    for t in range(n_threads):
+        src = perm[t * per: (t + 1) * per]
+        dst = perm[half + t * per: half + (t + 1) * per]
+        reqs = [src[i: i + 37].astype(np.int64) for i in range(0, per, 37)]
+        dreqs = [dst[i: i + 37].astype(np.int64) for i in range(0, per, 37)]
+        jobs.append((reqs, dreqs))
+    errors, host_images = [], [None] * n_threads
+
+    def work(t):
+        try:
+            reqs, dreqs = jobs[t]
+            stream = torch.cuda.Stream(cuda)
+            stager = bk.HostStager(cuda, chunk_bytes=16 * tile, n_buffers=2, chunks_per_launch=2)
+            with torch.cuda.stream(stream):
+                gb = pool.make_batch(reqs, "layer_major")
+                sb = pool.make_batch(dreqs, "layer_major", check_unique=True)
+                staging, _ = pool.empty_staging(gb)
+                for _ in range(rounds):
+                    pool.gather(gb, staging)
+                    pool.scatter(sb, staging)          # the gathered pages land in this thread's own pages
+                host = bk.pinned_empty(gb.n_slots * tile)
+                stager.gather_to_host(pool, gb, host, "auto")
+                stream.synchronize()
+            want = oracle.gather_layered_c(pool_h, reqs, "layer_major")
+            if _to_np(staging).tobytes() != want.tobytes():
+                errors.append(f"thread {t}: gathered image differs")
+            if host.numpy().tobytes() != want.tobytes():
+                errors.append(f"thread {t}: host image differs")
+            host_images[t] = want
+            stager.close()
+        except Exception as e:                          # noqa: BLE001 - reported below
+            errors.append(f"thread {t}: {type(e).__name__}: {e}")
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(n_threads)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    torch.cuda.synchronize(cuda)
+    pool.check()
+    assert not errors, errors
+    for t in range(n_threads):
+        oracle.scatter_layered_c(pool_h, jobs[t][1], host_images[t], "layer_major")
+    assert _to_np(pool_d).tobytes() == pool_h.tobytes()
