@@ -374,8 +374,9 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layo
     log(f"gather {g_pages} pages in {len(g_groups)} launch(es) ({alg_g / 1e9:.2f} GB r+w), scatter {s_pages} pages in "
         f"{len(s_groups)} launch(es) ({alg_s / 1e9:.2f} GB r+w)")
 
-    def step(events=None):
-        if events is not None:
+    def step(events=None, first=True):
+        # events[0] is recorded for the first step only: a later step starts where the one before it ended
+        if events is not None and first:
             events[0].record()
         for b, _ in g_groups:
             pool.gather(b, *views(b, g_st, g_sc))
@@ -398,10 +399,12 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layo
     torch.cuda.synchronize(dev)
     t0 = time.perf_counter()
     for k in range(steps):
-        step(evs[k])
+        step(evs[k], first=(k == 0))
     torch.cuda.synchronize(dev)
     wall = time.perf_counter() - t0
     pool.check()
+    for k in range(1, steps):
+        evs[k][0] = evs[k - 1][2]
 
     # per-launch durations (a direction's launches are back to back between two events)
     g_ms = [e[0].elapsed_time(e[1]) / len(g_groups) for e in evs]
