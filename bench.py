@@ -2,7 +2,8 @@
 """Benchmark of the KV page-copy hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload qwen2_7b|qwen2_1p5b|llama3_8b|
-                    llama3_70b_fp8|reference_200x50]
+                    llama3_70b_fp8|qwen2_7b_token_major|layout_change|staging|reference_200x50]
+                    [--pool-form planar|worker] [--pool-alloc spread|stacked|planes] [--layout layer_major|page_major]
 
 Default workload = the configuration the headline target is quoted on: the Qwen2-7B-shaped bf16 pool
 (28 layers x K/V, 131072 pages of 16 tokens x 4 heads x 128, ~120 GB resident in HBM) with 64
