@@ -13,13 +13,14 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libbikv_pagecopy.so")
 
 MAX_DIM = 5
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 OK, EINVAL, EHIP, ESYS, ESTATE, EBOUNDS, ERANGE = 0, -1, -2, -3, -4, -5, -6
 ST_SRC_RANGE, ST_DST_RANGE, ST_PAGE_ID = 1, 2, 4
 LAYOUT_LAYER_MAJOR, LAYOUT_PAGE_MAJOR = 0, 1
 HINT_NONE, HINT_LAYER_MAJOR, HINT_PAGE_MAJOR = 0, 1, 2
-STAGE_PIPELINED, STAGE_DIRECT, STAGE_AUTO = 0, 1, 2
+STAGE_PIPELINED, STAGE_DIRECT, STAGE_AUTO, STAGE_PIPELINED_KERNEL = 0, 1, 2, 3
+TRACE_KINDS = ("kernel", "copy_d2h", "copy_h2d", "copy_kernel")
 PLACE_SPREAD, PLACE_SEQUENTIAL = 0, 1
 
 
@@ -78,6 +79,11 @@ class StageStats(C.Structure):
     _fields_ = [("bytes", C.c_int64), ("n_chunks", C.c_int64), ("wall_seconds", C.c_double)]
 
 
+class TraceStep(C.Structure):
+    _fields_ = [("lane", C.c_int32), ("kind", C.c_int32), ("bytes", C.c_int64), ("start_ms", C.c_float),
+                ("end_ms", C.c_float)]
+
+
 class TensorDimsC(C.Structure):
     _fields_ = [
         ("total_tokens", C.c_int64),
@@ -132,6 +138,8 @@ _SIGNATURES = {
                                      C.c_void_p, C.c_int64, C.c_void_p]),
     "bikv_stager_create": (C.c_int, [C.c_int, C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_void_p)]),
     "bikv_stager_wait": (C.c_int, [C.c_void_p, C.POINTER(StageStats)]),
+    "bikv_stager_trace": (C.c_int, [C.c_void_p, C.c_int64]),
+    "bikv_stager_trace_read": (C.c_int64, [C.c_void_p, C.POINTER(TraceStep), C.c_int64]),
     "bikv_gather_to_host_async": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PageBatchDesc),
                                             C.POINTER(C.c_int64), C.c_int64, C.c_int32, C.c_void_p,
                                             C.c_int64, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]),

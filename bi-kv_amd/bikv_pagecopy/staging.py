@@ -16,7 +16,8 @@ import torch
 from . import _lib
 from .pool import PagedKVPool, PageBatch, _LAYOUT_CODE
 
-_MODES = {"pipelined": _lib.STAGE_PIPELINED, "direct": _lib.STAGE_DIRECT, "auto": _lib.STAGE_AUTO}
+_MODES = {"pipelined": _lib.STAGE_PIPELINED, "direct": _lib.STAGE_DIRECT, "auto": _lib.STAGE_AUTO,
+          "pipelined_kernel": _lib.STAGE_PIPELINED_KERNEL}
 
 
 def pinned_empty(nbytes: int) -> torch.Tensor:
@@ -111,6 +112,23 @@ class HostStager:
         finally:
             self._keep.clear()
         return stats.bytes, stats.n_chunks, stats.wall_seconds
+
+    def trace(self, max_steps: int):
+        """Switches the per-step trace on (up to `max_steps` kernel launches and host copies, each between two
+        timing events on its lane) or, with 0, off. A diagnostic: it costs a few percent of throughput."""
+        _lib.check(_lib.load().bikv_stager_trace(self._h, int(max_steps)))
+
+    def trace_read(self):
+        """The steps recorded since trace(n), in issue order, as a list of dicts {lane, kind, bytes, start_ms,
+        end_ms}; times count from the start of the first recorded step. Call after wait()."""
+        lib = _lib.load()
+        n = _lib.check(lib.bikv_stager_trace_read(self._h, None, 0))
+        if n == 0:
+            return []
+        buf = (_lib.TraceStep * n)()
+        _lib.check(lib.bikv_stager_trace_read(self._h, buf, n))
+        return [{"lane": s.lane, "kind": _lib.TRACE_KINDS[s.kind], "bytes": s.bytes, "start_ms": s.start_ms,
+                 "end_ms": s.end_ms} for s in buf]
 
     def close(self):
         if getattr(self, "_h", None):

@@ -39,7 +39,8 @@ int fail_hip(hipError_t e, const char* what) {
 // below) and that pointer is what kernels and copies are given.
 constexpr int64_t kScratchPayload = int64_t(16) << 20;
 constexpr int64_t kScratchScale = int64_t(64) << 10;
-constexpr int64_t kScratchCopy = int64_t(8) << 20;     // bytes per hipMemcpyAsync out of the scratch
+constexpr int64_t kScratchCopy = int64_t(8) << 20;     // bytes per hipMemcpyAsync out of the scratch (only when an
+                                                        // address is not 16-byte aligned and the copy kernel cannot be used)
 static __device__ __align__(256) unsigned char scratch[kScratchPayload + kScratchScale];
 
 // ---- per-device context: the host-mapped status block and the scratch address ---------------
@@ -47,6 +48,7 @@ struct DevCtx {
   uint32_t* status_host = nullptr;  // pinned, mapped
   uint32_t* status_dev = nullptr;   // the same memory as the device sees it
   char* scratch_dev = nullptr;      // this device's copy of `scratch`
+  bool bank_used[ST_BANKS] = {};    // banks handed out to stagers (the fixed ones are never marked)
 };
 static std::mutex g_ctx_mu;
 static DevCtx g_ctx[64];
@@ -80,6 +82,30 @@ int device_status(int device, int bank, uint32_t** dev_ptr) {
   }
   *dev_ptr = c.status_dev + bank * ST_SLOTS;
   return BIKV_OK;
+}
+
+int acquire_bank(int device, int* bank_out) {
+  uint32_t* st = nullptr;
+  const int rc = device_status(device, ST_BANK_SHARED, &st);   // creates the block on first use
+  if (rc) return rc;
+  std::lock_guard<std::mutex> lk(g_ctx_mu);
+  DevCtx& c = g_ctx[device];
+  for (int b = ST_BANK_DYNAMIC; b < ST_BANKS; ++b) {
+    if (c.bank_used[b]) continue;
+    c.bank_used[b] = true;
+    volatile uint32_t* s = c.status_host + b * ST_SLOTS;
+    for (int i = 0; i < ST_SLOTS; ++i) s[i] = 0;
+    *bank_out = b;
+    return BIKV_OK;
+  }
+  return fail(BIKV_ERANGE, "device %d already has %d host stagers: no status words are left for another",
+              device, ST_BANKS - ST_BANK_DYNAMIC);
+}
+
+void release_bank(int device, int bank) {
+  if (device < 0 || device >= 64 || bank < ST_BANK_DYNAMIC || bank >= ST_BANKS) return;
+  std::lock_guard<std::mutex> lk(g_ctx_mu);
+  g_ctx[device].bank_used[bank] = false;
 }
 
 // The scratch address of a device whose context already exists; never creates one (the allocation-free
@@ -146,7 +172,6 @@ struct bikv_pool {
   const char** d_plane_base;        // device table: payload planes, then scale planes
   uint64_t align_bits;              // OR of every base, stride and tile size (payload)
   uint64_t scale_align_bits;
-  bool kv_rows;                     // planes 2l and 2l+1 interleave in 512-byte rows (the pair mover's shape)
 };
 
 extern "C" int bikv_abi_version(void) { return BIKV_ABI_VERSION; }
@@ -166,11 +191,15 @@ extern "C" int bikv_check_status(int device, void* stream, uint32_t* bits_out) {
   return status_error(bits);
 }
 
-extern "C" void bikv_reset_tuning(void) { tuning() = Tuning(); }
+extern "C" void bikv_reset_tuning(void) {
+  std::lock_guard<std::mutex> lk(tuning_mutex());
+  tuning_shared() = Tuning();
+}
 
 extern "C" int bikv_set_tuning(const char* key, int64_t value) {
   if (!key) return fail(BIKV_EINVAL, "null tuning key");
-  Tuning& t = tuning();
+  std::lock_guard<std::mutex> lk(tuning_mutex());
+  Tuning& t = tuning_shared();
   if (!strcmp(key, "seg")) {
     if (value < 0 || value > kMaxSeg) return fail(BIKV_EINVAL, "seg must be in [0, %d]", kMaxSeg);
     t.seg = (int)value;
@@ -210,13 +239,8 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
     t.transpose_sc1 = value ? 1 : 0;
   } else if (!strcmp(key, "transpose_pairs")) {
     t.transpose_pairs = value ? 1 : 0;
-  } else if (!strcmp(key, "pair_rows")) {
-    t.pair_rows = value ? 1 : 0;
   } else if (!strcmp(key, "debug_unique")) {
     t.debug_unique = value ? 1 : 0;
-  } else if (!strcmp(key, "run_chunk_kib")) {
-    if (value < 0 || value > 1 << 20) return fail(BIKV_EINVAL, "run_chunk_kib out of range");
-    t.run_chunk_kib = (int)value;
   } else {
     return fail(BIKV_EINVAL, "unknown tuning key '%s'", key);
   }
@@ -286,12 +310,6 @@ extern "C" int bikv_pool_create(const bikv_pool_desc* d, bikv_pool** out) {
   p->d_plane_base = static_cast<const char**>(dtab);
   p->align_bits = ab;
   p->scale_align_bits = sab;
-  // The Worker's [tokens, 2, heads, dim] tensors at 512 bytes per row: K and V rows of a token are the two
-  // halves of one KiB, plane 2l+1 starts one row after plane 2l.
-  p->kv_rows = !has_scale && row_bytes == 512 && row_stride == 1024 && d->tile_bytes % 1024 == 0 &&
-               d->n_planes % 2 == 0 && (ab & 15) == 0;
-  for (int q = 0; q + 1 < d->n_planes && p->kv_rows; q += 2)
-    if (table[q + 1] != table[q] + 512) p->kv_rows = false;
   *out = p;
   return BIKV_OK;
 }
@@ -350,7 +368,6 @@ static int build_move(int bank, const bikv_pool* pool, const bikv_page_batch* b,
   if ((pool->row_bytes & (pool->row_bytes - 1)) == 0)
     for (m->payload.log2_row = 0; (int64_t(1) << m->payload.log2_row) < pool->row_bytes;) ++m->payload.log2_row;
   m->payload.vec_width = lowbit_width(pool->align_bits | (uint64_t)staging);
-  m->kv_rows = pool->kv_rows && m->payload.vec_width == 16 && (pb & 1) == 0 && (pc & 1) == 0;
   if (has_scale) {
     m->scale.plane_base = pool->d_plane_base + pool->n_planes;
     m->scale.staging = static_cast<char*>(const_cast<void*>(scale_staging));
@@ -416,6 +433,7 @@ static bool debug_unique() {
     const char* e = getenv("BIKV_DEBUG_UNIQUE");
     return e && e[0] && e[0] != '0';
   }();
+  refresh_tuning();
   return env_on || tuning().debug_unique != 0;
 }
 
@@ -583,8 +601,16 @@ extern "C" int bikv_h2d_copy(int device, void* dev_dst, const void* host_src, in
 //     sit in either for minutes (the host -> device path and kernels storing into mapped pinned memory
 //     do not show it): BIKV_STAGE_DIRECT keeps 55 GB/s in both states, which is why BIKV_STAGE_AUTO
 //     sends with the kernel and receives with the DMA engine.
+// One step of a lane as the optional trace records it: two events around the launch or copy.
+struct TraceOp {
+  hipEvent_t e0, e1;
+  int32_t lane, kind;
+  int64_t bytes;
+};
+
 struct bikv_stager {
   int device;
+  int bank;                  // this stager's own status words
   int64_t chunk_bytes;       // bytes of one host copy
   int group;                 // copies per kernel launch
   int64_t lane_bytes;        // chunk_bytes * group: HBM buffer of one lane
@@ -599,6 +625,9 @@ struct bikv_stager {
   int64_t pending_bytes, pending_copies;
   bool timing;
   std::chrono::steady_clock::time_point t_first;
+  // opt-in trace (bikv_stager_trace): up to trace_cap steps, each between two timing events
+  int64_t trace_cap = 0;
+  std::vector<TraceOp> trace;
 };
 
 extern "C" int bikv_stager_create(int device, int64_t chunk_bytes, int32_t chunks_per_launch,
@@ -608,12 +637,17 @@ extern "C" int bikv_stager_create(int device, int64_t chunk_bytes, int32_t chunk
   if (chunk_bytes < 4096 || n_buffers < 1 || n_buffers > 16 || chunks_per_launch < 1 || chunks_per_launch > 64)
     return fail(BIKV_EINVAL, "need chunk_bytes >= 4096, 1 <= chunks_per_launch <= 64 and 1 <= n_buffers <= 16");
   if (chunk_bytes > (int64_t(1) << 36) / chunks_per_launch) return fail(BIKV_EINVAL, "lane buffer too large");
-  uint32_t* st_ptr = nullptr;
-  int rc = device_status(device, ST_BANK_STAGER, &st_ptr);
+  int bank = -1;
+  int rc = acquire_bank(device, &bank);
   if (rc) return rc;
-  BIKV_DEVICE(device);
+  DeviceGuard guard_(device);
+  if (guard_.error() != hipSuccess) {
+    release_bank(device, bank);
+    return fail_hip(guard_.error(), "hipSetDevice");
+  }
   bikv_stager* st = new bikv_stager();
   st->device = device;
+  st->bank = bank;
   st->chunk_bytes = chunk_bytes;
   st->group = chunks_per_launch;
   st->lane_bytes = chunk_bytes * chunks_per_launch;
@@ -650,6 +684,11 @@ extern "C" int bikv_stager_destroy(bikv_stager* st) {
   if (st->after) (void)hipEventDestroy(st->after);
   if (st->ring) (void)hipFree(st->ring);
   if (st->scale_ring) (void)hipFree(st->scale_ring);
+  for (TraceOp& op : st->trace) {
+    (void)hipEventDestroy(op.e0);
+    (void)hipEventDestroy(op.e1);
+  }
+  release_bank(st->device, st->bank);
   delete st;
   return BIKV_OK;
 }
@@ -736,7 +775,36 @@ struct LaneSet {
   int64_t lane_bytes, scale_lane_bytes, chunk_bytes;
   uint64_t* next_launch;
   int bank;
+  // device -> host hop done by the library's copy kernel through these device views of the two pinned
+  // images (null: hipMemcpyAsync)
+  char* host_dev = nullptr;
+  char* host_scale_dev = nullptr;
+  // opt-in trace: steps are appended to *trace while it holds fewer than trace_cap
+  std::vector<TraceOp>* trace = nullptr;
+  int64_t trace_cap = 0;
 };
+
+enum : int { TRACE_KERNEL = 0, TRACE_COPY_D2H = 1, TRACE_COPY_H2D = 2, TRACE_COPY_KERNEL = 3 };
+
+// Records the first event of a traced step on `s`; returns its index in the trace or -1 (not traced).
+static int trace_begin(const LaneSet& L, int lane, int kind, int64_t bytes, hipStream_t s) {
+  if (!L.trace || (int64_t)L.trace->size() >= L.trace_cap) return -1;
+  TraceOp op;
+  op.lane = lane;
+  op.kind = kind;
+  op.bytes = bytes;
+  if (hipEventCreate(&op.e0) != hipSuccess) return -1;
+  if (hipEventCreate(&op.e1) != hipSuccess) {
+    (void)hipEventDestroy(op.e0);
+    return -1;
+  }
+  (void)hipEventRecord(op.e0, s);
+  L.trace->push_back(op);
+  return (int)L.trace->size() - 1;
+}
+static void trace_end(const LaneSet& L, int idx, hipStream_t s) {
+  if (idx >= 0) (void)hipEventRecord((*L.trace)[(size_t)idx].e1, s);
+}
 
 static int validate_stage_args(const bikv_pool* pool, const bikv_page_batch* batch, const int64_t* req_pages,
                                int64_t n_requests, int32_t layout, const void* host, int64_t host_bytes,
@@ -804,21 +872,48 @@ static int issue_pipelined(int dir, const bikv_pool* pool, const bikv_page_batch
     char* host_chunk = host + ch.first_slot * T;
     char* host_scale_chunk = has_scale ? host_scale + ch.first_slot * S : nullptr;
     if (dir == 0) {
+      const int t = trace_begin(L, lane, TRACE_KERNEL, bytes, stream);
       const int rc = move_pages(L.bank, 0, pool, &sub, dev_chunk, bytes, dev_scale, ch.n_slots * S, stream);
       if (rc) return rc;
+      trace_end(L, t, stream);
     }
-    for (int64_t off = 0; off < bytes; off += L.chunk_bytes) {
-      const int64_t n = bytes - off < L.chunk_bytes ? bytes - off : L.chunk_bytes;
-      BIKV_HIP(dir == 0 ? hipMemcpyAsync(host_chunk + off, dev_chunk + off, (size_t)n, hipMemcpyDeviceToHost, stream)
-                        : hipMemcpyAsync(dev_chunk + off, host_chunk + off, (size_t)n, hipMemcpyHostToDevice, stream));
+    // the hop between lane buffer and pinned image: the library's copy kernel through the mapped image when
+    // the call asked for it and both ends are 16-byte aligned, else one hipMemcpyAsync per chunk_bytes
+    char* img_dev = L.host_dev ? L.host_dev + ch.first_slot * T : nullptr;
+    const bool kernel_hop = img_dev && (((uint64_t)img_dev | (uint64_t)dev_chunk) & 15) == 0;
+    if (kernel_hop) {
+      // one launch moves the whole lane buffer: thousands of waves' accesses are in flight at once, and
+      // no copy engine is involved
+      const int t = trace_begin(L, lane, TRACE_COPY_KERNEL, bytes, stream);
+      BIKV_HIP(dir == 0 ? launch_linear_copy(dev_chunk, img_dev, bytes, stream)
+                        : launch_linear_copy(img_dev, dev_chunk, bytes, stream));
+      trace_end(L, t, stream);
       ++*n_copies;
+    } else {
+      for (int64_t off = 0; off < bytes; off += L.chunk_bytes) {
+        const int64_t n = bytes - off < L.chunk_bytes ? bytes - off : L.chunk_bytes;
+        const int t = trace_begin(L, lane, dir == 0 ? TRACE_COPY_D2H : TRACE_COPY_H2D, n, stream);
+        BIKV_HIP(dir == 0 ? hipMemcpyAsync(host_chunk + off, dev_chunk + off, (size_t)n, hipMemcpyDeviceToHost, stream)
+                          : hipMemcpyAsync(dev_chunk + off, host_chunk + off, (size_t)n, hipMemcpyHostToDevice, stream));
+        trace_end(L, t, stream);
+        ++*n_copies;
+      }
     }
-    if (has_scale)
-      BIKV_HIP(dir == 0 ? hipMemcpyAsync(host_scale_chunk, dev_scale, (size_t)(ch.n_slots * S), hipMemcpyDeviceToHost, stream)
-                        : hipMemcpyAsync(dev_scale, host_scale_chunk, (size_t)(ch.n_slots * S), hipMemcpyHostToDevice, stream));
+    if (has_scale) {
+      const int64_t sb = ch.n_slots * S;
+      char* simg_dev = L.host_scale_dev ? L.host_scale_dev + ch.first_slot * S : nullptr;
+      if (kernel_hop && simg_dev && (((uint64_t)simg_dev | (uint64_t)dev_scale) & 15) == 0)
+        BIKV_HIP(dir == 0 ? launch_linear_copy(dev_scale, simg_dev, sb, stream)
+                          : launch_linear_copy(simg_dev, dev_scale, sb, stream));
+      else
+        BIKV_HIP(dir == 0 ? hipMemcpyAsync(host_scale_chunk, dev_scale, (size_t)sb, hipMemcpyDeviceToHost, stream)
+                          : hipMemcpyAsync(dev_scale, host_scale_chunk, (size_t)sb, hipMemcpyHostToDevice, stream));
+    }
     if (dir == 1) {
+      const int t = trace_begin(L, lane, TRACE_KERNEL, bytes, stream);
       const int rc = move_pages(L.bank, 1, pool, &sub, dev_chunk, bytes, dev_scale, ch.n_slots * S, stream);
       if (rc) return rc;
+      trace_end(L, t, stream);
     }
   }
   return BIKV_OK;
@@ -862,8 +957,8 @@ static int stage_issue(int dir, bikv_stager* st, const bikv_pool* pool, const bi
                                host_scale_bytes, &total_pages);
   if (rc) return rc;
   if (pool->device != st->device) return fail(BIKV_EINVAL, "pool and stager are on different devices");
-  if (mode == BIKV_STAGE_AUTO) mode = dir == 0 ? BIKV_STAGE_DIRECT : BIKV_STAGE_PIPELINED;
-  if (mode != BIKV_STAGE_DIRECT && mode != BIKV_STAGE_PIPELINED)
+  if (mode == BIKV_STAGE_AUTO) mode = BIKV_STAGE_DIRECT;
+  if (mode != BIKV_STAGE_DIRECT && mode != BIKV_STAGE_PIPELINED && mode != BIKV_STAGE_PIPELINED_KERNEL)
     return fail(BIKV_EINVAL, "unknown staging mode %d", mode);
   if (total_pages == 0) return BIKV_OK;
   const bool has_scale = pool->scale_tile_bytes > 0;
@@ -895,8 +990,13 @@ static int stage_issue(int dir, bikv_stager* st, const bikv_pool* pool, const bi
     BIKV_HIP(hipHostGetDevicePointer(&dptr, host, 0));
     if (has_scale) BIKV_HIP(hipHostGetDevicePointer(&sptr, host_scale, 0));
     const int lane = (int)(st->next_launch++ % (uint64_t)st->n_buf);
-    rc = move_pages(ST_BANK_STAGER, dir, pool, batch, dptr, image_bytes, sptr, scale_image_bytes, st->lanes[lane]);
+    LaneSet T0;                       // only the trace fields are used
+    T0.trace = st->trace_cap > 0 ? &st->trace : nullptr;
+    T0.trace_cap = st->trace_cap;
+    const int t = trace_begin(T0, lane, TRACE_KERNEL, image_bytes, st->lanes[lane]);
+    rc = move_pages(st->bank, dir, pool, batch, dptr, image_bytes, sptr, scale_image_bytes, st->lanes[lane]);
     if (rc) return rc;
+    trace_end(T0, t, st->lanes[lane]);
   } else {
     // the scale tiles of a launch ride in a second, much smaller buffer per lane
     const int64_t max_slots = st->lane_bytes / T;
@@ -918,7 +1018,18 @@ static int stage_issue(int dir, bikv_stager* st, const bikv_pool* pool, const bi
     L.scale_lane_bytes = has_scale ? st->scale_ring_bytes / st->n_buf : 0;
     L.chunk_bytes = st->chunk_bytes;
     L.next_launch = &st->next_launch;
-    L.bank = ST_BANK_STAGER;
+    L.bank = st->bank;
+    L.trace = st->trace_cap > 0 ? &st->trace : nullptr;
+    L.trace_cap = st->trace_cap;
+    if (mode == BIKV_STAGE_PIPELINED_KERNEL) {
+      void* dptr = nullptr;
+      BIKV_HIP(hipHostGetDevicePointer(&dptr, host, 0));
+      L.host_dev = static_cast<char*>(dptr);
+      if (has_scale) {
+        BIKV_HIP(hipHostGetDevicePointer(&dptr, host_scale, 0));
+        L.host_scale_dev = static_cast<char*>(dptr);
+      }
+    }
     rc = issue_pipelined(dir, pool, batch, req_pages, n_requests, layout, static_cast<char*>(host),
                          static_cast<char*>(host_scale), L, &copies);
     if (rc) {
@@ -948,7 +1059,48 @@ extern "C" int bikv_stager_wait(bikv_stager* st, bikv_stage_stats* stats) {
   st->pending_bytes = st->pending_copies = 0;
   st->timing = false;
   if (es != hipSuccess) return fail_hip(es, "hipStreamSynchronize(lane)");
-  return check_bank(st->device, ST_BANK_STAGER);
+  return check_bank(st->device, st->bank);
+}
+
+// Opt-in trace of a stager's lanes: while it is on, every kernel launch and host copy the stager enqueues is
+// bracketed by two timing events on its lane, up to `max_steps` steps (0 switches it off and drops what was
+// recorded). bikv_stager_trace_read, after bikv_stager_wait, turns the events into start / end times in
+// milliseconds relative to the first recorded step.
+extern "C" int bikv_stager_trace(bikv_stager* st, int64_t max_steps) {
+  if (!st || max_steps < 0 || max_steps > (int64_t(1) << 20)) return fail(BIKV_EINVAL, "bad stager_trace arguments");
+  BIKV_DEVICE(st->device);
+  drain_lanes(st);
+  for (TraceOp& op : st->trace) {
+    (void)hipEventDestroy(op.e0);
+    (void)hipEventDestroy(op.e1);
+  }
+  st->trace.clear();
+  st->trace_cap = max_steps;
+  if (max_steps > 0) st->trace.reserve((size_t)max_steps);
+  return BIKV_OK;
+}
+
+extern "C" int64_t bikv_stager_trace_read(bikv_stager* st, bikv_trace_step* out, int64_t cap) {
+  if (!st || cap < 0 || (cap > 0 && !out)) return fail(BIKV_EINVAL, "bad stager_trace_read arguments");
+  if (st->trace.empty()) return 0;
+  BIKV_DEVICE(st->device);
+  drain_lanes(st);
+  const hipEvent_t base = st->trace[0].e0;
+  int64_t n = 0;
+  for (const TraceOp& op : st->trace) {
+    if (n >= cap) break;
+    float a = -1.0f, b = -1.0f;
+    // a step whose launch failed has no second event: it is reported with end_ms = -1
+    if (hipEventElapsedTime(&a, base, op.e0) != hipSuccess) { a = -1.0f; (void)hipGetLastError(); }
+    if (hipEventElapsedTime(&b, base, op.e1) != hipSuccess) { b = -1.0f; (void)hipGetLastError(); }
+    out[n].lane = op.lane;
+    out[n].kind = op.kind;
+    out[n].bytes = op.bytes;
+    out[n].start_ms = a;
+    out[n].end_ms = b;
+    ++n;
+  }
+  return (int64_t)st->trace.size();
 }
 
 extern "C" int bikv_gather_to_host_async(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
@@ -1007,8 +1159,9 @@ extern "C" int bikv_scatter_from_host(bikv_stager* st, const bikv_pool* pool,
                     const_cast<void*>(host_scale_src), host_scale_bytes, mode, stats);
 }
 
-// The allocation-free form of bikv_gather_to_host: the same pipeline on ONE lane — the caller's stream —
-// whose buffer is this device's `scratch` array. Enqueue only. Nothing here allocates or frees: the
+// The allocation-free form of bikv_gather_to_host: the lane pipeline on ONE lane — the caller's stream —
+// whose buffer is this device's `scratch` array, with the library's copy kernel as the hop to the host
+// (BIKV_STAGE_PIPELINED_KERNEL's shape). Enqueue only. Nothing here allocates or frees: the
 // device context (status block, scratch address) was set up by bikv_init / bikv_pool_create, the planner
 // is an iterator, errors go to a thread-local buffer.
 extern "C" int bikv_gather_to_host_noalloc(const bikv_pool* pool, const bikv_page_batch* batch,
@@ -1042,6 +1195,15 @@ extern "C" int bikv_gather_to_host_noalloc(const bikv_pool* pool, const bikv_pag
   L.chunk_bytes = kScratchCopy;
   L.next_launch = &launches;
   L.bank = ST_BANK_SHARED;
+  // the hop to the host is the library's copy kernel storing through the mapped image: kernels only, so the
+  // call can be captured into a HIP graph, and no copy engine is involved
+  void* dptr = nullptr;
+  BIKV_HIP(hipHostGetDevicePointer(&dptr, host_dst, 0));
+  L.host_dev = static_cast<char*>(dptr);
+  if (pool->scale_tile_bytes > 0) {
+    BIKV_HIP(hipHostGetDevicePointer(&dptr, host_scale_dst, 0));
+    L.host_scale_dev = static_cast<char*>(dptr);
+  }
   return issue_pipelined(0, pool, batch, req_pages, n_requests, layout, static_cast<char*>(host_dst),
                          static_cast<char*>(host_scale_dst), L, &copies);
 }

@@ -10,19 +10,23 @@ namespace bikv {
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int fail_hip(hipError_t e, const char* what);
 
-// The host-mapped status block of a device is cut into banks, one per kind of caller, so that the
-// synchronous entry points (ring producer, host stager) judge their own launches only: a flag left
-// behind by somebody's unchecked asynchronous launch cannot fail them, and bikv_check_status() from
-// another thread cannot clear a flag they are about to read.
+// The host-mapped status block of a device is cut into banks of ST_SLOTS words. Two are fixed, one per
+// kind of caller; the rest are handed out one per host stager, so that a wait judges the launches of its
+// own stager only: a flag left behind by somebody's unchecked asynchronous launch cannot fail it,
+// bikv_check_status() from another thread cannot clear a flag it is about to read, and a page id
+// rejected in one stager's launch is never reported (or cleared) by another stager's wait.
 enum : int {
   ST_BANK_SHARED = 0,   // the asynchronous entry points; read and cleared by bikv_check_status()
   ST_BANK_RING = 1,     // copies issued by the ring producer
-  ST_BANK_STAGER = 2,   // launches of the host staging pipeline
-  ST_BANKS = 8
+  ST_BANK_DYNAMIC = 2,  // first bank that acquire_bank() hands out (one per bikv_stager)
+  ST_BANKS = 256        // 256 banks x 8 words x 4 bytes = 8 KiB of pinned memory per device
 };
 
 // Device-side pointer of bank `bank` of the status block of `device` (created on first use).
 int device_status(int device, int bank, uint32_t** dev_ptr);
+// A bank of its own for a new stager (cleared), or BIKV_ERANGE when all are taken; release_bank() returns it.
+int acquire_bank(int device, int* bank_out);
+void release_bank(int device, int bank);
 
 // Synchronises `stream`, then converts raised status slots of `bank` into BIKV_EBOUNDS (and clears them).
 int sync_and_check(int device, int bank, hipStream_t stream);

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 namespace bikv {
 
 // Status slots written by kernels (one 32-bit word per condition, plain stores of 1, so no
@@ -43,8 +45,6 @@ struct MoveArgs {
   int32_t order;                  // wave mover: 0 = plane by plane, 1 = page chunk by page chunk
   int32_t log2_chunk;             // order 1: pages per chunk = 2^log2_chunk
   int32_t layout_hint;            // host side only: 0 none, 1 layer-major, 2 page-major staging
-  int32_t kv_rows;                // 1 = K and V rows of a token are adjacent 512-byte halves of one KiB of the
-                                  // pool (planes 2l and 2l+1 interleave row by row): the pair mover may be used
   uint32_t* status;
 };
 
@@ -58,7 +58,6 @@ struct Tuning {
   int unroll = 4;       // 16-byte vectors in flight per lane (1, 2, 4 or 8)
   int nontemporal = -1; // cache policy of payload accesses: 0 none, 1 nt, 4 nt + system scope,
                         // -1 = chosen per direction and layout (run copy also: 2 loads, 3 stores only)
-  int run_chunk_kib = 0;       // bytes of a run handled by one workgroup, KiB; 0 = choose
   int run_group = 1;           // wave run kernel: several short runs share one grid row (0 = off)
   int small_run_max = 1023;    // runs up to this many bytes go to the one-lane-per-piece kernel
   int transpose_lds_kib = 60;  // LDS tile budget of the layout-change kernels, KiB
@@ -68,10 +67,14 @@ struct Tuning {
                                // 0 = chosen per direction (256 for the load, 512 for the store)
   int transpose_sc1 = 1;       // K/V-pair kernel: payload stores are nt with system scope (0 = nt only)
   int debug_unique = 0;        // 1 = scattering entry points check their destination ids on the host first
-  int pair_rows = 0;           // 1 = pools whose K and V rows interleave in 512-byte halves use the pair mover
-                               // (measured 4-6 % SLOWER than the general wave mover: off by default)
 };
-Tuning& tuning();
+// The knobs are process-wide and may be set from any thread. Setters change the shared copy under
+// tuning_mutex(); every launch first copies it into a snapshot of the calling thread (refresh_tuning) and
+// reads only that (tuning()), so one launch sees one consistent set of knobs whatever is set meanwhile.
+std::mutex& tuning_mutex();
+Tuning& tuning_shared();
+const Tuning& tuning();
+void refresh_tuning();
 
 constexpr int kBlock = 256;      // 4 wavefronts
 constexpr int kMaxSeg = 256;     // LDS descriptor slots per workgroup
@@ -94,6 +97,9 @@ struct RunArgs {
   uint32_t* status;
 };
 hipError_t launch_copy_runs(const RunArgs& a, hipStream_t stream);
+// Plain copy of `bytes` bytes between two 16-byte aligned device-visible addresses (either may be mapped
+// pinned host memory).
+hipError_t launch_linear_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
 
 // Fused page move + layout change between token-major pages and a per-layer paged NHD pool.
 struct TransposeArgs {

@@ -15,6 +15,8 @@
 // wave movers do not: tiles that are not 16-byte aligned, tiny tiles, misaligned pools.
 #include "pagecopy_kernels.h"
 
+#include <mutex>
+
 namespace bikv {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -356,94 +358,6 @@ __global__ __launch_bounds__(B) void tile_move_wave_kernel(const MoveArgs a) {
   }
 }
 
-// ---------------------------------------------------------------------------------------------
-// Pair mover: the Worker's per-layer tensors [tokens, 2, heads, dim] (Bi-KV/Worker/Worker.py:74-78) at
-// the reference's own shape (2 KV heads x 128 x fp16) have rows of 512 bytes, K and V of a token adjacent:
-// one KiB of the pool is {K row, V row} of one token, and the K tile and the V tile of a page are two
-// different tiles of the staging image. A wave that moves 1 KiB of ONE tile therefore touches two
-// half-KiB pieces of the pool, which costs the scatter 10-15 %. Here a wave takes the two KiB of two
-// consecutive tokens instead — {K0 V0}, {K1 V1}: two 1 KiB accesses on the pool side — and exchanges the
-// upper half of the first vector with the lower half of the second between lanes i and i+32
-// (v_permlane32_swap), which turns them into {K0 K1} and {V0 V1}: two 1 KiB accesses on the staging side,
-// one in the K tile and one in the V tile. The exchange is its own inverse, so the scatter is the same
-// sequence backwards. Grid and walks are those of the wave mover with "plane" meaning layer.
-// MEASURED (MI355X, Qwen2-1.5B-shaped pool in the Worker's form, 30 GB): gather 5.85 / scatter 5.20 TB/s
-// against 6.07 / 5.51 for the general wave mover with its two half-KiB pool pieces per wave: two vectors in
-// flight per lane cost more than the contiguity gains, as they do in a plain copy. Kept selectable
-// ("pair_rows" = 1) and tested; not the default.
-// ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ void load2(uint64_t a, uint64_t b, u32x4& x, u32x4& y) {
-  asm volatile("global_load_dwordx4 %0, %2, off sc1 nt\n\t"
-               "global_load_dwordx4 %1, %3, off sc1 nt\n\t"
-               "s_waitcnt vmcnt(0)"
-               : "=&v"(x), "=&v"(y) : "v"(a), "v"(b) : "memory");
-}
-__device__ __forceinline__ void store2(uint64_t a, uint64_t b, const u32x4& x, const u32x4& y) {
-  asm volatile("global_store_dwordx4 %0, %2, off sc1 nt\n\t"
-               "global_store_dwordx4 %1, %3, off sc1 nt"
-               : : "v"(a), "v"(b), "v"(x), "v"(y) : "memory");
-}
-// lanes 32-63 of x <-> lanes 0-31 of y, all four dwords
-__device__ __forceinline__ void swap_halves(u32x4& x, u32x4& y) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const auto r = __builtin_amdgcn_permlane32_swap(x[i], y[i], false, false);
-    x[i] = r[0];
-    y[i] = r[1];
-  }
-}
-
-template <int DIR>
-__global__ __launch_bounds__(64) void tile_move_pair_kernel(const MoveArgs a) {
-  const uint32_t bx = blockIdx.x;
-  const int32_t lp = a.payload.log2_rows;       // pieces (token pairs) per tile: 2^lp or n_parts
-  const uint32_t np = a.payload.n_parts;
-  const uint32_t bt = lp >= 0 ? bx >> lp : bx / np;
-  const uint32_t part = lp >= 0 ? (bx & ((1u << lp) - 1u)) : bx - bt * np;
-  const uint32_t lc = (uint32_t)a.log2_chunk;
-  int64_t layer;
-  uint32_t i;
-  if (a.order == 0) {
-    layer = blockIdx.y;
-    i = bt;
-  } else {
-    const uint64_t chunk = (uint64_t)blockIdx.y + (uint64_t)blockIdx.z * gridDim.y;
-    const uint64_t page = (chunk << lc) + (bt & ((1u << lc) - 1u));
-    if (page >= (uint64_t)a.n_batch) return;
-    i = (uint32_t)page;
-    layer = (int64_t)(bt >> lc);
-  }
-  const int64_t qk = a.plane_begin + 2 * layer;                      // the K plane; V is qk + 1
-  const int64_t pid = cload(a.page_ids + i);
-  const int64_t s0 = cload(a.slots + i) - a.slot_bias;
-  const int64_t ss = cload(a.slot_strides + i);
-  const uint64_t plane = (uint64_t)cload(a.payload.plane_base + qk);
-  const int64_t slot_k = s0 + qk * ss, slot_v = slot_k + ss;
-  const bool bad_page = (uint64_t)pid >= (uint64_t)a.n_pool_pages;
-  const bool bad_slot = (uint64_t)slot_k >= (uint64_t)a.payload.n_slots || (uint64_t)slot_v >= (uint64_t)a.payload.n_slots;
-  if (bad_page || bad_slot) {
-    if (threadIdx.x == 0 && part == 0) {
-      if (bad_page) raise(a.status, ST_SLOT_PAGE);
-      if (bad_slot) raise(a.status, DIR == 0 ? ST_SLOT_DST : ST_SLOT_SRC);
-    }
-    return;
-  }
-  const uint64_t lane = threadIdx.x * 16u;
-  const uint64_t pool = plane + (uint64_t)(pid * a.payload.page_stride) + (uint64_t)part * 2048u + lane;
-  const uint64_t sk = (uint64_t)a.payload.staging + (uint64_t)(slot_k * a.payload.tile_bytes) + (uint64_t)part * 1024u + lane;
-  const uint64_t sv = (uint64_t)a.payload.staging + (uint64_t)(slot_v * a.payload.tile_bytes) + (uint64_t)part * 1024u + lane;
-  u32x4 x, y;
-  if (DIR == 0) {
-    load2(pool, pool + 1024u, x, y);      // {K0 V0}, {K1 V1}
-    swap_halves(x, y);                    // {K0 K1}, {V0 V1}
-    store2(sk, sv, x, y);
-  } else {
-    load2(sk, sv, x, y);
-    swap_halves(x, y);
-    store2(pool, pool + 1024u, x, y);
-  }
-}
-
 // How the wave mover walks a batch, and whether it marks its accesses non-temporal. Measured on
 // MI355X with 8-64 KiB tiles and 56-160 planes of 2 GiB each:
 //   * random accesses confined to ONE plane's few GiB run ~10 % slower than the same accesses spread
@@ -581,20 +495,7 @@ static bool finish_class(TileClass& c, int forced_seg, int64_t n_batch, int plan
 
 hipError_t launch_tile_move(int dir, MoveArgs& a, hipStream_t stream) {
   if (a.n_batch <= 0 || a.plane_count <= 0) return hipSuccess;
-  if (tuning().seg == 0 && tuning().pair_rows != 0 && a.kv_rows != 0 && tuning().wave_block == 64) {
-    // K and V rows interleave in half-KiB pieces: the pair mover, planned as a wave mover over layers
-    // whose pieces are token pairs (1 KiB of each of the two staging tiles, 2 KiB of the pool)
-    dim3 grid;
-    const WavePolicy pol = choose_wave_policy(dir, a.layout_hint);
-    MoveArgs b = a;
-    b.plane_count = a.plane_count / 2;
-    if (plan_wave(b, 64, pol.order, pol.log2_chunk, &grid)) {
-      b.plane_count = a.plane_count;
-      if (dir == 0) hipLaunchKernelGGL(tile_move_pair_kernel<0>, grid, dim3(64), 0, stream, b);
-      else hipLaunchKernelGGL(tile_move_pair_kernel<1>, grid, dim3(64), 0, stream, b);
-      return hipGetLastError();
-    }
-  }
+  refresh_tuning();
   if (tuning().seg == 0) {
     // default: the wave mover, whenever the payload shape qualifies
     dim3 grid;
@@ -637,67 +538,6 @@ __device__ __forceinline__ void copy_span_vw(uint64_t s, uint64_t d, int64_t byt
   const int64_t done = n * VW;
   for (int64_t i = done + threadIdx.x; i < bytes; i += kBlock)
     st<false, uint8_t>(d + (uint64_t)i, ld<false, uint8_t>(s + (uint64_t)i));
-}
-
-// Large runs: workgroup b handles chunk (b % chunks_per_run) of run (b / chunks_per_run). The
-// run's two offsets are fetched once by lane 0, parked in LDS and broadcast.
-template <int UNROLL, bool NT>
-__global__ __launch_bounds__(kBlock) void copy_runs_kernel(const RunArgs a, int64_t chunk_bytes,
-                                                           uint32_t chunks_per_run) {
-  __shared__ int64_t s_off[2];
-  const uint32_t run = blockIdx.x / chunks_per_run;
-  const uint32_t ch = blockIdx.x - run * chunks_per_run;
-  if (threadIdx.x == 0) {
-    s_off[0] = a.src_off[run];
-    s_off[1] = a.dst_off[run];
-  }
-  __syncthreads();
-  const int64_t so_u = (int64_t)uniform64((uint64_t)s_off[0]);
-  const int64_t do_u = (int64_t)uniform64((uint64_t)s_off[1]);
-  const int64_t so = so_u * a.unit_bytes;
-  const int64_t dof = do_u * a.unit_bytes;
-  const bool bad_src = so_u < 0 || so < 0 || so > a.src_bytes - a.run_bytes;
-  const bool bad_dst = do_u < 0 || dof < 0 || dof > a.dst_bytes - a.run_bytes;
-  if (bad_src || bad_dst) {
-    if (threadIdx.x == 0) {
-      if (bad_src) raise(a.status, ST_SLOT_SRC);
-      if (bad_dst) raise(a.status, ST_SLOT_DST);
-    }
-    return;
-  }
-  const int64_t lo = (int64_t)ch * chunk_bytes;
-  const int64_t hi = lo + chunk_bytes < a.run_bytes ? lo + chunk_bytes : a.run_bytes;
-  const uint64_t s = (uint64_t)(a.src + so + lo);
-  const uint64_t d = (uint64_t)(a.dst + dof + lo);
-  const int64_t bytes = hi - lo;
-  const uint64_t al = s | d;
-  if ((al & 15) == 0) {
-    const int64_t nvec = bytes >> 4;
-    for (int64_t base = 0; base < nvec; base += (int64_t)kBlock * UNROLL) {
-      u32x4 v[UNROLL];
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        const int64_t i = base + u * kBlock + threadIdx.x;
-        if (i < nvec) v[u] = ld<NT, u32x4>(s + ((uint64_t)i << 4));
-      }
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        const int64_t i = base + u * kBlock + threadIdx.x;
-        if (i < nvec) st<NT, u32x4>(d + ((uint64_t)i << 4), v[u]);
-      }
-    }
-    const int64_t done = nvec << 4;
-    for (int64_t i = done + threadIdx.x; i < bytes; i += kBlock)
-      st<false, uint8_t>(d + (uint64_t)i, ld<false, uint8_t>(s + (uint64_t)i));
-  } else if ((al & 7) == 0) {
-    copy_span_vw<8>(s, d, bytes);
-  } else if ((al & 3) == 0) {
-    copy_span_vw<4>(s, d, bytes);
-  } else if ((al & 1) == 0) {
-    copy_span_vw<2>(s, d, bytes);
-  } else {
-    copy_span_vw<1>(s, d, bytes);
-  }
 }
 
 // Small runs (below 1 KiB by default): one lane per 16-byte piece, many runs per workgroup.
@@ -831,51 +671,63 @@ static hipError_t launch_runs_wave(const RunArgs& a, hipStream_t stream) {
 
 hipError_t launch_copy_runs(const RunArgs& a, hipStream_t stream) {
   if (a.n_runs <= 0 || a.run_bytes <= 0) return hipSuccess;
+  refresh_tuning();
   const int64_t small_max = tuning().small_run_max;
-  if (a.run_lens || (a.run_bytes > small_max && tuning().run_chunk_kib == 0)) {
+  if (a.run_lens || a.run_bytes > small_max) {
     switch (tuning().wave_block) {
       case 128: return launch_runs_wave<128>(a, stream);
       case 256: return launch_runs_wave<256>(a, stream);
       default: return launch_runs_wave<64>(a, stream);
     }
   }
-  if (a.run_bytes <= small_max) {
-    const int64_t ppr = (a.run_bytes + 15) >> 4;
-    const int64_t total = ppr * a.n_runs;
-    const int64_t grid = (total + kBlock - 1) / kBlock;
-    if (grid >= (int64_t(1) << 24)) return hipErrorInvalidValue;
-    if (tuning().nontemporal != 0)
-      hipLaunchKernelGGL(copy_small_runs_kernel<true>, dim3((uint32_t)grid), dim3(kBlock), 0, stream, a,
-                         (uint32_t)ppr, total);
-    else
-      hipLaunchKernelGGL(copy_small_runs_kernel<false>, dim3((uint32_t)grid), dim3(kBlock), 0, stream, a,
-                         (uint32_t)ppr, total);
-    return hipGetLastError();
-  }
-  int64_t chunk = (int64_t)tuning().run_chunk_kib * 1024;
-  if (chunk <= 0) {
-    // ~4096 workgroups when the batch is big enough, 16 KiB..256 KiB each
-    const int64_t total = a.run_bytes * a.n_runs;
-    chunk = 16 * 1024;
-    while (chunk < 256 * 1024 && total / (chunk * 2) >= 4096) chunk *= 2;
-  }
-  chunk = (chunk + 4095) & ~int64_t(4095);
-  const int64_t cpr = (a.run_bytes + chunk - 1) / chunk;
-  const int64_t grid = cpr * a.n_runs;
-  if (cpr >= (int64_t(1) << 31) || grid >= (int64_t(1) << 24)) return hipErrorInvalidValue;
-  const bool nt = tuning().nontemporal != 0;
-  if (nt)
-    hipLaunchKernelGGL((copy_runs_kernel<4, true>), dim3((uint32_t)grid), dim3(kBlock), 0, stream,
-                       a, chunk, (uint32_t)cpr);
+  const int64_t ppr = (a.run_bytes + 15) >> 4;
+  const int64_t total = ppr * a.n_runs;
+  const int64_t grid = (total + kBlock - 1) / kBlock;
+  if (grid >= (int64_t(1) << 24)) return hipErrorInvalidValue;
+  if (tuning().nontemporal != 0)
+    hipLaunchKernelGGL(copy_small_runs_kernel<true>, dim3((uint32_t)grid), dim3(kBlock), 0, stream, a,
+                       (uint32_t)ppr, total);
   else
-    hipLaunchKernelGGL((copy_runs_kernel<4, false>), dim3((uint32_t)grid), dim3(kBlock), 0, stream,
-                       a, chunk, (uint32_t)cpr);
+    hipLaunchKernelGGL(copy_small_runs_kernel<false>, dim3((uint32_t)grid), dim3(kBlock), 0, stream, a,
+                       (uint32_t)ppr, total);
   return hipGetLastError();
 }
 
-Tuning& tuning() {
-  static Tuning t;
-  return t;
+// A plain copy of `bytes` bytes between two 16-byte aligned addresses in the wave movers' shape (one
+// 16-byte vector per lane, 64-lane workgroups, nt + system scope): the hop between a stager's lane buffer
+// and the mapped pinned image when the library moves those bytes itself.
+__global__ __launch_bounds__(64) void linear_copy_kernel(const char* src, char* dst, int64_t bytes) {
+  const int64_t lo = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * 1024 + threadIdx.x * 16;
+  if (lo >= bytes) return;
+  const int64_t left = bytes - lo;
+  if (left >= 16) move16<2>((uint64_t)(src + lo), (uint64_t)(dst + lo));
+  else move_upto16((uint64_t)(src + lo), (uint64_t)(dst + lo), (int)left);
+}
+
+hipError_t launch_linear_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream) {
+  if (bytes <= 0) return hipSuccess;
+  if ((((uint64_t)src | (uint64_t)dst) & 15) != 0) return hipErrorInvalidValue;
+  const int64_t groups = (bytes + 1023) / 1024;
+  const int64_t gx = groups < 65536 ? groups : 65536;
+  const int64_t gy = (groups + gx - 1) / gx;
+  if (gy > 65535) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(linear_copy_kernel, dim3((uint32_t)gx, (uint32_t)gy), dim3(64), 0, stream,
+                     static_cast<const char*>(src), static_cast<char*>(dst), bytes);
+  return hipGetLastError();
+}
+
+// Launch knobs: one shared copy that the setters change under a mutex, and one snapshot per thread that
+// a launch takes when it begins and reads from then on.
+static std::mutex g_tuning_mu;
+static Tuning g_tuning;
+static thread_local Tuning t_tuning;
+
+std::mutex& tuning_mutex() { return g_tuning_mu; }
+Tuning& tuning_shared() { return g_tuning; }
+const Tuning& tuning() { return t_tuning; }
+void refresh_tuning() {
+  std::lock_guard<std::mutex> lk(g_tuning_mu);
+  t_tuning = g_tuning;
 }
 
 }  // namespace bikv

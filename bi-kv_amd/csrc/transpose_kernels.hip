@@ -431,6 +431,7 @@ static hipError_t launch_transpose_dir(const TransposeArgs& a, dim3 grid, size_t
 // take (the caller has already validated them; this is a second line of defence).
 hipError_t launch_transpose_pages(int dir, TransposeArgs& a, hipStream_t stream) {
   if (a.n_pages <= 0) return hipSuccess;
+  refresh_tuning();
   const int ES = a.elem_bytes;
   if (ES != 1 && ES != 2 && ES != 4) return hipErrorInvalidValue;
   const int VE = 16 / ES;

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define BIKV_ABI_VERSION 3
+#define BIKV_ABI_VERSION 4
 
 enum {
   BIKV_OK = 0,
@@ -72,18 +72,16 @@ int bikv_check_status(int device, void* stream, uint32_t* bits_out);
  * "unroll" (segment mover: 16-byte vectors in flight per lane: 1, 2, 4, 8), "nontemporal" (nt hint on
  * payload accesses: 1 on, 0 off, 4 = nt with system scope, -1 = default: chosen per direction and
  * layout; the run copy also takes 2 = loads only, 3 = stores only),
- * "run_chunk_kib" (bytes of a run per workgroup, KiB; 0 = automatic), "small_run_max" (runs up to this
+ * "small_run_max" (runs up to this
  * many bytes use one lane per 16-byte piece instead of one wave per KiB), "run_group" (1 = several
  * short runs share a row of the launch grid, default; 0 = one row per run), "transpose_lds_kib" and
  * "transpose_dsplit" (LDS tile budget and head_dim slices of the layout-change kernel),
  * "transpose_pairs" (1 = the K/V-pair kernel, default; 0 = the element-wise kernel), "transpose_block"
  * (its lanes per workgroup: 128, 256, 512, 1024; 0 = default: 256 for the load, 512 for the store) and
  * "transpose_sc1" (1 = its payload stores are nt with system scope, default; 0 = nt only),
- * "debug_unique" (1 = what BIKV_DEBUG_UNIQUE=1 in the environment switches on, see bikv_find_duplicate),
- * "pair_rows" (1 = pools whose K and V rows interleave in 512-byte halves, the Worker's own tensors at
- * 2 KV heads x 128 x fp16, are moved two tokens at a time with the halves exchanged between lanes, so
- * that both sides see 1 KiB accesses; 0 = default: the general wave mover, which measures 4-6 % faster).
- * Process-wide. */
+ * "debug_unique" (1 = what BIKV_DEBUG_UNIQUE=1 in the environment switches on, see bikv_find_duplicate).
+ * Process-wide and safe to set from any thread: a launch works on the snapshot of the knobs it took
+ * when it began. */
 int bikv_set_tuning(const char* key, int64_t value);
 /* Every knob back to its default. */
 void bikv_reset_tuning(void);
@@ -222,15 +220,25 @@ int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* batch,
  * scale tiles of a pool with a scale class go, slot for slot, into a second pinned image.
  *
  * Modes: BIKV_STAGE_PIPELINED as above; BIKV_STAGE_DIRECT lets the kernel store into (read from) the
- * mapped pinned image itself, no HBM hop and no DMA engine; BIKV_STAGE_AUTO picks DIRECT for
- * pool -> host and PIPELINED for host -> pool, the faster and steadier choice per direction on MI355X
- * (the device -> host DMA path runs at either ~30 or ~57 GB/s there, whichever state the platform is
- * in, while kernel stores to pinned memory hold ~55 GB/s).
+ * mapped pinned image itself, no HBM hop and no copy engine; BIKV_STAGE_PIPELINED_KERNEL keeps lanes and
+ * lane buffers but makes the hop between lane buffer and pinned image with the library's own copy kernel
+ * (one launch per lane buffer, through the mapped image) instead of hipMemcpyAsync; BIKV_STAGE_AUTO is
+ * DIRECT in both directions. Why: on MI355X every hipMemcpyAsync between device and host, in either
+ * direction, drops from ~57 to ~30 GB/s for as long as the driver is scrubbing device memory that some
+ * hipFree (this process's or, at start-up, bikv_device_alloc's released filler chunks) has given back —
+ * about one second per 15 GB freed, and hipFree itself returns at once, so nothing announces it. Kernels
+ * that store to or load from mapped pinned memory hold 54-56 GB/s through it. PIPELINED is 1-2 % faster
+ * than the other modes while nothing is being scrubbed and half as fast while something is.
+ *
+ * Every stager has status words of its own: a page id or slot that one stager's kernel rejects is
+ * reported by THAT stager's wait (or synchronous call) and by no other's, so stagers are independent
+ * objects that different host threads can drive on one GPU at the same time. A device serves up to 254
+ * stagers at once (BIKV_ERANGE beyond). One stager is not re-entrant: one thread at a time per stager.
  * ------------------------------------------------------------------------------------------ */
 typedef struct bikv_stager bikv_stager; /* opaque; owns n_buffers HIP streams, each with an HBM buffer */
 
 enum { BIKV_LAYOUT_LAYER_MAJOR = 0, BIKV_LAYOUT_PAGE_MAJOR = 1 };
-enum { BIKV_STAGE_PIPELINED = 0, BIKV_STAGE_DIRECT = 1, BIKV_STAGE_AUTO = 2 };
+enum { BIKV_STAGE_PIPELINED = 0, BIKV_STAGE_DIRECT = 1, BIKV_STAGE_AUTO = 2, BIKV_STAGE_PIPELINED_KERNEL = 3 };
 
 int bikv_stager_create(int device, int64_t chunk_bytes, int32_t chunks_per_launch, int32_t n_buffers,
                        bikv_stager** out);
@@ -243,7 +251,7 @@ typedef struct bikv_stage_stats {
 } bikv_stage_stats;
 
 /* Synchronous: returns when all bytes are in host memory; BIKV_EBOUNDS if a page id or slot was
- * rejected by a kernel of THIS call (the stager's launches have a status word of their own). */
+ * rejected by a kernel of THIS call (every stager has status words of its own). */
 int bikv_gather_to_host(bikv_stager* st, const bikv_pool* pool, const bikv_page_batch* batch,
                         const int64_t* req_pages, int64_t n_requests, int32_t layout,
                         void* host_dst, int64_t host_bytes,
@@ -281,15 +289,35 @@ int bikv_scatter_from_host_async(bikv_stager* st, const bikv_pool* pool, const b
                                  int64_t host_scale_bytes, int32_t mode, void* after_stream);
 int bikv_stager_wait(bikv_stager* st, bikv_stage_stats* stats);
 
+/* Opt-in trace of a stager's lanes, for finding out where the time of a transfer goes (no counterpart in
+ * the reference; its stage timers are host-side prints, kvcache.py:155-238). While it is on, every kernel
+ * launch and every host copy the stager enqueues is bracketed by two timing events on its lane, up to
+ * `max_steps` steps; max_steps = 0 switches it off and drops what was recorded. bikv_stager_trace_read
+ * (after bikv_stager_wait) writes up to `cap` steps in issue order and returns how many were recorded;
+ * times are milliseconds from the start of the first recorded step. Tracing allocates events as it goes
+ * and costs a few percent of throughput: a diagnostic, not a mode to serve in. */
+enum { BIKV_TRACE_KERNEL = 0, BIKV_TRACE_COPY_D2H = 1, BIKV_TRACE_COPY_H2D = 2, BIKV_TRACE_COPY_KERNEL = 3 };
+typedef struct bikv_trace_step {
+  int32_t lane;
+  int32_t kind;       /* BIKV_TRACE_*: gather/scatter kernel, hipMemcpyAsync out, hipMemcpyAsync in, copy kernel */
+  int64_t bytes;
+  float start_ms;
+  float end_ms;       /* -1 when the step was never completed (its launch failed) */
+} bikv_trace_step;
+int bikv_stager_trace(bikv_stager* st, int64_t max_steps);
+int64_t bikv_stager_trace_read(bikv_stager* st, bikv_trace_step* out, int64_t cap);
+
 /* bikv_gather_to_host for callers that cannot allocate: code under HIP graph capture, serving loops and
- * harnesses that forbid hipMalloc. It has no counterpart in the reference. The pipeline is the
- * pipelined mode of bikv_gather_to_host on ONE lane, the caller's `stream`: gather kernel into a buffer,
- * hipMemcpyAsync of at most 8 MiB each to `host_dst`, piece after piece in stream order. The buffer is
- * not a stager's: it is a static array inside the library's device code, 16 MiB for payload tiles plus
- * 64 KiB for scale tiles, which every GPU the library runs on holds until the process ends. The call
- * allocates and frees nothing (no hipMalloc, no stream or event creation) and only enqueues: it returns
- * when kernels and copies are queued on `stream`; rejected page ids / slots are reported by
- * bikv_check_status like those of bikv_gather_pages.
+ * harnesses that forbid hipMalloc. It has no counterpart in the reference. The pipeline is that of
+ * BIKV_STAGE_PIPELINED_KERNEL on ONE lane, the caller's `stream`: gather kernel into a buffer, then the
+ * library's copy kernel from the buffer into `host_dst` through its device mapping, piece after piece in
+ * stream order — kernel launches only, so a capturing stream records nothing but kernel nodes. (Only when a
+ * tile size is not a multiple of 16 bytes does the hop fall back to hipMemcpyAsync calls of at most 8 MiB.)
+ * The buffer is not a stager's: it is a static array inside the library's device code, 16 MiB for payload
+ * tiles plus 64 KiB for scale tiles, which every GPU the library runs on holds until the process ends. The
+ * call allocates and frees nothing (no hipMalloc, no stream or event creation) and only enqueues: it returns
+ * when the kernels are queued on `stream`; rejected page ids / slots are reported by bikv_check_status
+ * like those of bikv_gather_pages.
  * Limits: tile_bytes <= 16 MiB and scale_tile_bytes <= 64 KiB (BIKV_ERANGE otherwise); the device must
  * have been set up by bikv_init or any bikv_pool_create (BIKV_ESTATE otherwise — a valid pool implies it).
  * All calls on one GPU share that GPU's array: calls whose work overlaps in time (two streams, or two

@@ -299,11 +299,11 @@ def test_worker_token_interleaved_layers(bk, oracle, cuda, P, H, D, dtype, layou
 
 
 @pytest.mark.parametrize("layout", ["layer_major", "page_major"])
-def test_pair_mover_for_half_kib_rows_matches_the_general_mover_and_the_oracle(bk, oracle, cuda, layout):
-    """The Worker's own shape (2 KV heads x 128 x fp16: 512-byte rows, K and V of a token adjacent) takes the
-    pair mover, which exchanges half-waves between lanes; every walk of it against the oracle and against
-    the general wave mover on the same pool, and a rejected page id."""
-    _announce(f"pair mover {layout}")
+def test_half_kib_rows_of_the_worker_shape_match_the_oracle_in_every_walk(bk, oracle, cuda, layout):
+    """The Worker's own shape (2 KV heads x 128 x fp16: 512-byte rows, K and V of a token adjacent, so that a
+    wave's KiB of a tile is two half-KiB pieces of the pool): every walk of the wave mover against the oracle,
+    and a rejected page id."""
+    _announce(f"half-KiB rows {layout}")
     rng = np.random.default_rng(311)
     P, H, D, L, blocks = 16, 2, 128, 5, 70
     layers_h = [rng.integers(0, 65536, size=(blocks * P, 2, H, D), dtype=np.uint16) for _ in range(L)]
@@ -312,14 +312,14 @@ def test_pair_mover_for_half_kib_rows_matches_the_general_mover_and_the_oracle(b
     want = oracle.gather_layered_c(planes_h, reqs, layout).tobytes()
     perm = rng.permutation(blocks)
     sreqs = [perm[:21], perm[21:40]]
-    for pair_rows, order, lc in ((1, -1, -1), (1, 0, 0), (1, 1, 0), (1, 1, 2), (1, 1, 5), (0, -1, -1)):
-        bk.set_tuning(pair_rows=pair_rows, order=order, log2_chunk=lc)
+    for order, lc in ((-1, -1), (0, 0), (1, 0), (1, 2), (1, 5)):
+        bk.set_tuning(order=order, log2_chunk=lc)
         layers_d = [torch.from_numpy(a.view(np.int16)).to(cuda).view(torch.float16) for a in layers_h]
         pool = bk.PagedKVPool.from_token_kv_layers(layers_d, P)
         batch = pool.make_batch(reqs, layout)
         st, _ = pool.gather(batch)
         pool.check()
-        assert _to_np(st).tobytes() == want, (pair_rows, order, lc)
+        assert _to_np(st).tobytes() == want, (order, lc)
         sb = pool.make_batch(sreqs, layout, check_unique=True)
         src = rng.integers(0, 256, size=sb.n_slots * pool.tile_bytes, dtype=np.uint8)
         pool.scatter(sb, torch.from_numpy(src).to(cuda))
@@ -328,7 +328,7 @@ def test_pair_mover_for_half_kib_rows_matches_the_general_mover_and_the_oracle(b
         oracle.scatter_layered_c(ph, sreqs, src, layout)
         back = oracle.token_kv_layers_of_planes(ph.view(np.uint16), P, H, D)
         for l in range(L):
-            assert _to_np(layers_d[l]).tobytes() == back[l].tobytes(), (pair_rows, order, lc, l)
+            assert _to_np(layers_d[l]).tobytes() == back[l].tobytes(), (order, lc, l)
         # a page id outside the pool: that page is skipped and reported, its neighbours still move
         bad = pool.make_batch([[2, blocks + 3, 7]], layout)
         st2 = torch.full((bad.n_slots * pool.tile_bytes,), 0xA5, dtype=torch.uint8, device=cuda)

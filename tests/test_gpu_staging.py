@@ -7,7 +7,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("layout", ["layer_major", "page_major"])
-@pytest.mark.parametrize("mode", ["pipelined", "direct"])
+@pytest.mark.parametrize("mode", ["pipelined", "direct", "pipelined_kernel"])
 def test_gather_to_host_matches_oracle(lib, oracle, cuda, layout, mode):
     import bikv_pagecopy as bk
     print(f"[case] gather_to_host {layout} {mode}", flush=True)
@@ -31,13 +31,16 @@ def test_gather_to_host_matches_oracle(lib, oracle, cuda, layout, mode):
             # one launch per piece of the plan, one host copy per chunk_bytes of a piece
             plan = bk.plan_chunks(batch.req_pages, n_planes, layout, chunk_tiles * group)
             assert n_chunks == sum(-(-int(p[5]) // chunk_tiles) for p in plan)
+        elif mode == "pipelined_kernel":
+            # one gather launch and one copy launch per piece of the plan
+            assert n_chunks == len(bk.plan_chunks(batch.req_pages, n_planes, layout, chunk_tiles * group))
         else:
             assert n_chunks == 1
         stager.close()
 
 
 @pytest.mark.parametrize("layout", ["layer_major", "page_major"])
-@pytest.mark.parametrize("mode", ["pipelined", "direct"])
+@pytest.mark.parametrize("mode", ["pipelined", "direct", "pipelined_kernel"])
 def test_gather_to_host_moves_scales_with_the_payload(lib, oracle, cuda, layout, mode):
     """fp8-style pool: 16 KiB payload tiles + 32-byte scale tiles go to two pinned images."""
     import bikv_pagecopy as bk
@@ -253,3 +256,111 @@ def test_llama3_8b_requests_staged_in_4_to_16_mib_chunks(lib, oracle, cuda, chun
     assert np.array_equal(pool_d.cpu().numpy(), pool_h)
     stager.close()
     pool.close()
+
+
+def test_a_rejected_page_id_is_reported_by_its_own_stager_only(lib, oracle, cuda):
+    """Two stagers work on one pool at once; the batch given to the first names a page outside the pool.
+    Only that stager's wait raises (every stager has status words of its own); the other's image equals the
+    oracle's, and so do the good pages of the bad batch (the kernel skips the rejected page, nothing faults).
+    Both orders of waiting, both sending modes."""
+    import bikv_pagecopy as bk
+    print("[case] per-stager status words", flush=True)
+    rng = np.random.default_rng(401)
+    n_planes, n_pages, tile = 4, 50, 4096
+    pool_h = rng.integers(0, 256, size=(n_planes, n_pages, tile), dtype=np.uint8)
+    pool = bk.PagedKVPool.from_stacked(torch.from_numpy(pool_h).to(cuda), plane_dims=1)
+    good_req = [rng.permutation(n_pages)[:20]]
+    bad_req = [np.array([3, n_pages + 5, 9, 11], dtype=np.int64)]
+    good, bad = pool.make_batch(good_req), pool.make_batch(bad_req)
+    want_good = oracle.gather_layered_c(pool_h, good_req).tobytes()
+    want_bad = oracle.gather_layered_c(pool_h, [np.array([3, 9, 11])]).reshape(n_planes, 3, tile)
+    for mode in ("direct", "pipelined", "pipelined_kernel"):
+        for bad_waits_first in (True, False):
+            a = bk.HostStager(cuda, chunk_bytes=4 * tile, n_buffers=2, chunks_per_launch=1)
+            b = bk.HostStager(cuda, chunk_bytes=4 * tile, n_buffers=2, chunks_per_launch=1)
+            host_a = bk.pinned_empty(bad.n_slots * tile).fill_(0xA5)
+            host_b = bk.pinned_empty(good.n_slots * tile).fill_(0xA5)
+            a.gather_to_host_async(pool, bad, host_a, mode)
+            b.gather_to_host_async(pool, good, host_b, mode)
+            if bad_waits_first:
+                with pytest.raises(RuntimeError, match="page-id"):
+                    a.wait()
+                b.wait()
+            else:
+                b.wait()
+                with pytest.raises(RuntimeError, match="page-id"):
+                    a.wait()
+            a.wait()                       # the report was consumed: a second wait is clean
+            assert host_b.numpy().tobytes() == want_good, (mode, bad_waits_first)
+            got = host_a.numpy().reshape(n_planes, 4, tile)
+            assert np.array_equal(got[:, [0, 2, 3]], want_bad)
+            if mode == "direct":           # the other modes copy whole lane buffers, skipped slots included
+                assert (got[:, 1] == 0xA5).all()
+            # neither report leaked into the words bikv_check_status reads
+            pool.check()
+            a.close()
+            b.close()
+
+
+def test_stager_banks_are_returned_when_a_stager_is_destroyed(lib, cuda):
+    """A device hands out one set of status words per live stager; closing a stager gives its set back, so
+    creating and closing many stagers one after the other never runs out."""
+    import bikv_pagecopy as bk
+    print("[case] stager banks recycled", flush=True)
+    for _ in range(600):
+        bk.HostStager(cuda, chunk_bytes=4096, n_buffers=1, chunks_per_launch=1).close()
+    live = [bk.HostStager(cuda, chunk_bytes=4096, n_buffers=1, chunks_per_launch=1) for _ in range(8)]
+    for s in live:
+        s.close()
+
+
+def test_stager_trace_records_every_step_of_a_transfer(lib, oracle, cuda):
+    """The opt-in trace brackets every kernel launch and host copy with events: the steps it reports are those
+    of the plan, in issue order, each with end >= start, and the transfer is still bit-exact."""
+    import bikv_pagecopy as bk
+    print("[case] stager trace", flush=True)
+    rng = np.random.default_rng(409)
+    n_planes, n_pages, tile = 6, 64, 16384
+    pool_h = rng.integers(0, 256, size=(n_planes, n_pages, tile), dtype=np.uint8)
+    pool = bk.PagedKVPool.from_stacked(torch.from_numpy(pool_h).to(cuda), plane_dims=1)
+    reqs = [rng.permutation(n_pages)[:m] for m in (7, 30)]
+    batch = pool.make_batch(reqs)
+    want = oracle.gather_layered_c(pool_h, reqs).tobytes()
+    stager = bk.HostStager(cuda, chunk_bytes=4 * tile, n_buffers=2, chunks_per_launch=2)
+    plan = bk.plan_chunks(batch.req_pages, n_planes, "layer_major", 8)
+    host = bk.pinned_empty(batch.n_slots * tile)
+    for mode, copy_kind in (("pipelined", "copy_d2h"), ("pipelined_kernel", "copy_kernel")):
+        stager.trace(4096)
+        host.fill_(0xA5)
+        stager.gather_to_host(pool, batch, host, mode)
+        steps = stager.trace_read()
+        assert host.numpy().tobytes() == want
+        kernels = [s for s in steps if s["kind"] == "kernel"]
+        copies = [s for s in steps if s["kind"] == copy_kind]
+        assert len(kernels) == len(plan) and len(kernels) + len(copies) == len(steps)
+        assert [s["bytes"] for s in kernels] == [int(p[5]) * tile for p in plan]
+        assert sum(s["bytes"] for s in copies) == batch.n_slots * tile
+        assert all(s["end_ms"] >= s["start_ms"] >= 0 for s in steps)
+        assert {s["lane"] for s in steps} == {0, 1}
+    # direct mode: one kernel step
+    stager.trace(8)
+    host.fill_(0)
+    stager.gather_to_host(pool, batch, host, "direct")
+    assert [s["kind"] for s in stager.trace_read()] == ["kernel"]
+    assert host.numpy().tobytes() == want
+    # a cap smaller than the transfer: the trace stops, the transfer does not
+    stager.trace(3)
+    host.fill_(0)
+    stager.gather_to_host(pool, batch, host, "pipelined")
+    assert len(stager.trace_read()) == 3
+    assert host.numpy().tobytes() == want
+    # the receiving direction (this changes the pool, hence last)
+    stager.trace(64)
+    perm = rng.permutation(n_pages)
+    sb = pool.make_batch([perm[:9]], check_unique=True)
+    stager.scatter_from_host(pool, sb, host[: sb.n_slots * tile], "pipelined")
+    kinds = [s["kind"] for s in stager.trace_read()]
+    assert kinds.count("copy_h2d") >= 1 and kinds.count("kernel") >= 1 and set(kinds) == {"copy_h2d", "kernel"}
+    stager.trace(0)
+    assert stager.trace_read() == []
+    stager.close()
