@@ -18,6 +18,7 @@
 // half) and maps them alternately into one virtual range (hipMemAddressReserve / hipMemMap). Every
 // window of such a pool, however small, then spreads its writes over both halves.
 #include "../../include/bikv_pagecopy.h"
+#include "host_logic/host_checks.h"
 #include "pagecopy_internal.h"
 
 #include <algorithm>
@@ -236,10 +237,10 @@ extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, v
   al.n_fillers = n_fillers;
   hipError_t e = hipMemAddressReserve(&al.va, al.bytes, 0, nullptr, 0);
   if (e != hipSuccess) { cleanup(); return fail_hip(e, "hipMemAddressReserve"); }
+  const std::vector<bool> order = interleave_order(same.size(), other.size());
   size_t is = 0, io = 0;
   for (size_t k = 0; k < n && e == hipSuccess; ++k) {
-    const bool take_other = io < other.size() && (is >= same.size() || (io + 1) * n <= (k + 1) * other.size() + n / 2);
-    hipMemGenericAllocationHandle_t h = take_other ? other[io++] : same[is++];
+    hipMemGenericAllocationHandle_t h = order[k] ? other[io++] : same[is++];
     e = hipMemMap(static_cast<char*>(al.va) + k * chunk, chunk, 0, h, 0);
     if (e == hipSuccess) al.handles.push_back(h);
   }

@@ -11,17 +11,16 @@
 //     IPC handle (a process cannot open its own handle);
 //   - consumer_receive can time out.
 #include "../../include/bikv_pagecopy.h"
+#include "host_logic/ring_logic.h"
 #include "pagecopy_internal.h"
 #include "pagecopy_kernels.h"
 
 #include <cerrno>
 #include <cstdlib>
 #include <cstring>
-#include <ctime>
-#include <deque>
-#include <utility>
+#include <mutex>
+#include <shared_mutex>
 #include <fcntl.h>
-#include <semaphore.h>
 #include <sys/mman.h>
 #include <sys/stat.h>
 #include <unistd.h>
@@ -33,6 +32,7 @@ static_assert(sizeof(hipIpcMemHandle_t) <= BIKV_IPC_HANDLE_SIZE, "IPC handle mus
 
 namespace {
 
+// What a role has mapped: the control block and the ring.
 struct Role {
   int fd = -1;
   bikv_shared_control* ctrl = nullptr;
@@ -40,17 +40,21 @@ struct Role {
   int device = 0;
   bool ipc_mapped = false;  // producer only: mem came from hipIpcOpenMemHandle
   char shm_name[256] = "";
-  // producer only, back-pressure: transfers published and not yet released by the consumer, oldest
-  // first, as (ring offset, bytes)
-  bool backpressure = false;
-  int64_t bp_timeout_ms = -1;
-  std::deque<std::pair<size_t, size_t>> in_flight;
-  // producer only: window handed out by bikv_producer_reserve and not published yet
-  bool reserved = false;
-  size_t reserved_at = 0, reserved_bytes = 0;
 };
 
+// One producer role and one consumer role per process, as in the reference (ipc_service.cpp:9-17), whose
+// callers are gRPC thread pools: every entry point takes its role's lock, so concurrent callers are
+// serialised instead of interleaving their bookkeeping.
+//   g_prod.mu (inside ring::Producer)  held for the whole of a producer call, GPU copy included: the
+//                                      ring's write offset only moves at publication
+//   g_cons_mu                          exclusive for init / cleanup, shared for receive / release (a
+//                                      receive blocked on the semaphore must not keep the release that
+//                                      a producer under back-pressure is waiting for from running)
+// Where both are needed (a producer attaching to the ring of a consumer in its own process, a consumer
+// retiring such a producer) the consumer's lock is taken first.
 Role g_producer, g_consumer;
+ring::Producer g_prod;
+std::shared_mutex g_cons_mu;
 
 // Rings of this many bytes or more are neither exported nor mapped across processes.
 constexpr size_t kMaxIpcBytes = size_t(2) << 30;
@@ -59,7 +63,7 @@ constexpr size_t kMaxIpcBytes = size_t(2) << 30;
 // reservation: any other producer call would be handed the same window.
 const char kReservedMsg[] = "a reserved ring window is waiting for bikv_producer_publish (or bikv_producer_cancel)";
 
-sem_t* sem_of(unsigned char* raw) { return reinterpret_cast<sem_t*>(raw); }
+using ring::sem_of;
 
 void unmap_role(Role& r) {
   if (r.ctrl) {
@@ -72,92 +76,35 @@ void unmap_role(Role& r) {
   }
 }
 
-// The reference's ring advance (copy_kernel.cu:87-89): a batch that does not fit behind the
-// current offset restarts at 0. Returns the write offset.
-size_t ring_reserve(bikv_shared_control* c, size_t data_size) {
-  if (c->current_offset + data_size > c->buffer_size) c->current_offset = 0;
-  return c->current_offset;
-}
-
-int wait_ms(sem_t* s, int64_t timeout_ms) {
-  int rc;
-  if (timeout_ms < 0) {
-    do { rc = sem_wait(s); } while (rc == -1 && errno == EINTR);
-    return rc;
-  }
-  struct timespec ts;
-  clock_gettime(CLOCK_REALTIME, &ts);
-  ts.tv_sec += timeout_ms / 1000;
-  ts.tv_nsec += (timeout_ms % 1000) * 1000000L;
-  if (ts.tv_nsec >= 1000000000L) {
-    ts.tv_sec += 1;
-    ts.tv_nsec -= 1000000000L;
-  }
-  do { rc = sem_timedwait(s, &ts); } while (rc == -1 && errno == EINTR);
-  return rc;
-}
-
-// Ring advance for the producer. Without back-pressure this is ring_reserve. With it, the write
-// window [at, at+data_size) must not touch a transfer the consumer still holds: the consumer posts
-// sem_complete once per transfer it is done with, in order, and the producer blocks here until
-// every overlapping transfer has been released (the reference declares sem_complete,
-// ipc_wrapper.h:16, initialises it, ipc_service.cpp:47, and never uses it: a wrapping producer
-// overwrites tensors the consumer may still read).
-int producer_reserve(Role& p, size_t data_size, size_t* at_out) {
-  bikv_shared_control* c = p.ctrl;
-  const size_t at = ring_reserve(c, data_size);
-  *at_out = at;
-  if (!p.backpressure) return BIKV_OK;
-  sem_t* done = sem_of(c->sem_complete);
-  while (!p.in_flight.empty() && sem_trywait(done) == 0) p.in_flight.pop_front();
-  for (;;) {
-    bool overlap = false;
-    for (const auto& t : p.in_flight)
-      if (t.second > 0 && data_size > 0 && t.first < at + data_size && at < t.first + t.second) overlap = true;
-    if (!overlap) return BIKV_OK;
-    if (wait_ms(done, p.bp_timeout_ms) != 0) {
-      if (errno == ETIMEDOUT)
-        return fail(BIKV_ESTATE, "producer timed out after %lld ms waiting for the consumer to release the ring space it needs",
-                    (long long)p.bp_timeout_ms);
-      return fail(BIKV_ESYS, "sem_wait(sem_complete) failed: %s", strerror(errno));
-    }
-    p.in_flight.pop_front();
-  }
-}
-
-// The control block has ONE slot for the published offset and shape (ipc_wrapper.h:21-27), so with
-// back-pressure a transfer is published only once the consumer has released the previous one: the
-// copy of transfer k+1 overlaps the consumer's use of transfer k, its publication does not.
-int producer_wait_slot(Role& p) {
-  if (!p.backpressure) return BIKV_OK;
-  sem_t* done = sem_of(p.ctrl->sem_complete);
-  while (!p.in_flight.empty()) {
-    if (wait_ms(done, p.bp_timeout_ms) != 0) {
-      if (errno == ETIMEDOUT)
-        return fail(BIKV_ESTATE, "producer timed out after %lld ms waiting for the consumer to release the previous transfer",
-                    (long long)p.bp_timeout_ms);
-      return fail(BIKV_ESYS, "sem_wait(sem_complete) failed: %s", strerror(errno));
-    }
-    p.in_flight.pop_front();
-  }
+// ring::reserve_window with the producer's messages (caller holds g_prod.mu)
+int producer_reserve(size_t data_size, size_t* at_out) {
+  const int rc = ring::reserve_window(g_prod, data_size, at_out);
+  if (rc == ring::WAIT_TIMEOUT)
+    return fail(BIKV_ESTATE, "producer timed out after %lld ms waiting for the consumer to release the ring space it needs",
+                (long long)g_prod.bp_timeout_ms);
+  if (rc == ring::WAIT_ERROR) return fail(BIKV_ESYS, "sem_wait(sem_complete) failed: %s", strerror(errno));
   return BIKV_OK;
 }
 
-void producer_published(Role& p, size_t at, size_t data_size) {
-  if (p.backpressure) p.in_flight.emplace_back(at, data_size);
+int producer_wait_slot() {
+  const int rc = ring::wait_slot(g_prod);
+  if (rc == ring::WAIT_TIMEOUT)
+    return fail(BIKV_ESTATE, "producer timed out after %lld ms waiting for the consumer to release the previous transfer",
+                (long long)g_prod.bp_timeout_ms);
+  if (rc == ring::WAIT_ERROR) return fail(BIKV_ESYS, "sem_wait(sem_complete) failed: %s", strerror(errno));
+  return BIKV_OK;
 }
 
-// The reference's publish step (copy_kernel.cu:116-128, ipc_service.cpp:130-142) for the transfer
-// written at offset `at` (the value ring_reserve returned for it).
-void ring_publish(bikv_shared_control* c, size_t at, size_t data_size, const int64_t* shape, size_t ndim,
-                  int32_t dtype_code) {
-  c->last_valid_offset = at;
-  c->current_offset = at + data_size;
-  c->tensor_dim = ndim;
-  for (size_t i = 0; i < ndim && i < BIKV_MAX_DIM; ++i) c->tensor_shape[i] = shape[i];
-  c->data_size = data_size;
-  c->dtype_code = dtype_code;
-  sem_post(sem_of(c->sem_start));
+void producer_cleanup_locked() {
+  if (g_producer.mem && g_producer.ipc_mapped) (void)hipIpcCloseMemHandle(g_producer.mem);
+  g_producer.mem = nullptr;
+  unmap_role(g_producer);
+  g_producer = Role();
+  g_prod.ctrl = nullptr;
+  g_prod.backpressure = false;
+  g_prod.bp_timeout_ms = -1;
+  g_prod.in_flight.clear();
+  g_prod.reserved = false;
 }
 
 }  // namespace
@@ -197,12 +144,13 @@ static int map_control(const char* name, bool create, const char* who, Role* r) 
 }
 
 // The consumer owns the ring: device memory first, then the control block that describes it. The block is
-// filled in one go from a local image, so a producer that opens it early sees either zeros (refused: ring
-// size 0) or the finished description, never half of one.
+// filled from a local image with its ring size stored last (ring::describe_ring), so a producer that opens
+// it early sees either "no ring yet" (refused) or the finished description, never half of one.
 extern "C" int bikv_consumer_init(int device, const char* shm_name, size_t buffer_bytes) {
   if (!shm_name || !*shm_name) return fail(BIKV_EINVAL, "shm_name is empty");
   if (strlen(shm_name) >= sizeof(g_consumer.shm_name)) return fail(BIKV_EINVAL, "shm_name too long");
   if (buffer_bytes == 0) return fail(BIKV_EINVAL, "buffer_size must be positive");
+  std::unique_lock<std::shared_mutex> lk(g_cons_mu);
   if (g_consumer.ctrl) return fail(BIKV_ESTATE, "consumer already initialised (call consumer_cleanup first)");
   BIKV_HIP(hipSetDevice(device));
   Role r;
@@ -235,9 +183,7 @@ extern "C" int bikv_consumer_init(int device, const char* shm_name, size_t buffe
     (void)hipFree(r.mem);
     return rc;
   }
-  memcpy(r.ctrl, &image, sizeof(image));
-  sem_init(sem_of(r.ctrl->sem_start), 1, 0);
-  sem_init(sem_of(r.ctrl->sem_complete), 1, 0);
+  ring::describe_ring(r.ctrl, image);
   g_consumer = r;
   return BIKV_OK;
 }
@@ -247,6 +193,8 @@ extern "C" int bikv_consumer_init(int device, const char* shm_name, size_t buffe
 // the device.
 extern "C" int bikv_producer_init(int device, const char* shm_name) {
   if (!shm_name || !*shm_name) return fail(BIKV_EINVAL, "shm_name is empty");
+  std::shared_lock<std::shared_mutex> lkc(g_cons_mu);     // the consumer of this process, if any, stays put
+  std::lock_guard<std::mutex> lk(g_prod.mu);
   if (g_producer.ctrl) return fail(BIKV_ESTATE, "producer already initialised (call producer_cleanup first)");
   Role r;
   r.device = device;
@@ -254,7 +202,7 @@ extern "C" int bikv_producer_init(int device, const char* shm_name) {
   int rc = map_control(shm_name, false, "producer_init", &r);
   if (rc != BIKV_OK) return rc;
   const bool same_process = g_consumer.ctrl && strcmp(g_consumer.shm_name, shm_name) == 0;
-  const size_t ring_bytes = r.ctrl->buffer_size;
+  const size_t ring_bytes = ring::describes_ring(r.ctrl);   // acquire: what follows it in the block is complete
   char host[sizeof(r.ctrl->hostname)];
   memset(host, 0, sizeof(host));
   gethostname(host, sizeof(host));
@@ -289,20 +237,21 @@ extern "C" int bikv_producer_init(int device, const char* shm_name) {
     return rc;
   }
   g_producer = r;
+  g_prod.ctrl = r.ctrl;
   return BIKV_OK;
 }
 
 extern "C" void bikv_producer_cleanup(void) {
-  if (g_producer.mem && g_producer.ipc_mapped) (void)hipIpcCloseMemHandle(g_producer.mem);
-  g_producer.mem = nullptr;
-  unmap_role(g_producer);
-  g_producer = Role();
+  std::lock_guard<std::mutex> lk(g_prod.mu);
+  producer_cleanup_locked();
 }
 
 extern "C" void bikv_consumer_cleanup(void) {
-  if (g_producer.ctrl && !g_producer.ipc_mapped && g_producer.mem == g_consumer.mem) {
+  std::unique_lock<std::shared_mutex> lkc(g_cons_mu);
+  {
+    std::lock_guard<std::mutex> lk(g_prod.mu);
     // a same-process producer borrows the consumer's buffer: retire it first
-    bikv_producer_cleanup();
+    if (g_producer.ctrl && !g_producer.ipc_mapped && g_producer.mem == g_consumer.mem) producer_cleanup_locked();
   }
   if (g_consumer.mem) {
     DeviceGuard guard_(g_consumer.device);
@@ -323,8 +272,9 @@ static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_
                          const int64_t* dst_off, const int64_t* run_tokens, int64_t n_runs,
                          int64_t page_size, int64_t total_tokens, const bikv_tensor_dims* dims,
                          int64_t elem_bytes, int32_t dtype_code, void* stream) {
+  std::lock_guard<std::mutex> lk(g_prod.mu);
   if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
-  if (g_producer.reserved) return fail(BIKV_ESTATE, kReservedMsg);
+  if (g_prod.reserved) return fail(BIKV_ESTATE, kReservedMsg);
   if (!dims) return fail(BIKV_EINVAL, "dims is null");
   if (n_runs < 0 || page_size <= 0 || elem_bytes <= 0) return fail(BIKV_EINVAL, "bad n_runs, page_size or elem_bytes");
   if (dims->head_size <= 0 || dims->num_kv_heads <= 0 || dims->num_layers <= 0 || dims->kv_pair <= 0)
@@ -341,7 +291,7 @@ static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_
   BIKV_DEVICE(g_producer.device);
   size_t at = 0;
   {
-    const int rc = producer_reserve(g_producer, (size_t)data_size, &at);
+    const int rc = producer_reserve((size_t)data_size, &at);
     if (rc) return rc;
   }
   if (n_runs > 0) {
@@ -360,11 +310,10 @@ static int producer_copy(const void* src, int64_t src_bytes, const int64_t* src_
   }
   const int64_t shape[5] = {total_tokens, dims->head_size, dims->num_kv_heads, dims->num_layers, dims->kv_pair};
   {
-    const int rc = producer_wait_slot(g_producer);
+    const int rc = producer_wait_slot();
     if (rc) return rc;
   }
-  ring_publish(c, at, (size_t)data_size, shape, 5, dtype_code);
-  producer_published(g_producer, at, (size_t)data_size);
+  ring::publish_transfer(g_prod, at, (size_t)data_size, shape, 5, dtype_code);
   return BIKV_OK;
 }
 
@@ -389,8 +338,9 @@ extern "C" int bikv_producer_copy_tokens(const void* src, int64_t src_bytes, con
 
 extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64_t* shape,
                                   size_t ndim, int32_t dtype_code, void* stream) {
+  std::lock_guard<std::mutex> lk(g_prod.mu);
   if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
-  if (g_producer.reserved) return fail(BIKV_ESTATE, kReservedMsg);
+  if (g_prod.reserved) return fail(BIKV_ESTATE, kReservedMsg);
   if (ndim > BIKV_MAX_DIM) return fail(BIKV_EINVAL, "at most %d dimensions can be published", BIKV_MAX_DIM);
   if ((bytes > 0 && !dev_src) || (ndim > 0 && !shape)) return fail(BIKV_EINVAL, "null pointer argument");
   bikv_shared_control* c = g_producer.ctrl;
@@ -399,7 +349,7 @@ extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64
   BIKV_DEVICE(g_producer.device);
   size_t at = 0;
   {
-    const int rc = producer_reserve(g_producer, bytes, &at);
+    const int rc = producer_reserve(bytes, &at);
     if (rc) return rc;
   }
   if (bytes > 0) {
@@ -408,11 +358,10 @@ extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64
     BIKV_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   }
   {
-    const int rc = producer_wait_slot(g_producer);
+    const int rc = producer_wait_slot();
     if (rc) return rc;
   }
-  ring_publish(c, at, bytes, shape, ndim, dtype_code);
-  producer_published(g_producer, at, bytes);
+  ring::publish_transfer(g_prod, at, bytes, shape, ndim, dtype_code);
   return BIKV_OK;
 }
 
@@ -421,25 +370,27 @@ extern "C" int bikv_producer_send(const void* dev_src, size_t bytes, const int64
 // buffer, copy_kernel.cu:92-113): reserve applies the reference's wrap rule and hands out the write
 // pointer; publish performs the reference's bookkeeping for exactly the reserved bytes.
 extern "C" int bikv_producer_reserve(size_t bytes, void** ptr) {
+  std::lock_guard<std::mutex> lk(g_prod.mu);
   if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
-  if (g_producer.reserved) return fail(BIKV_ESTATE, kReservedMsg);
+  if (g_prod.reserved) return fail(BIKV_ESTATE, kReservedMsg);
   if (!ptr) return fail(BIKV_EINVAL, "null pointer argument");
   bikv_shared_control* c = g_producer.ctrl;
   if (bytes > c->buffer_size)
     return fail(BIKV_ERANGE, "reservation of %zu bytes does not fit the %zu-byte ring", bytes, c->buffer_size);
   size_t at = 0;
-  const int rc = producer_reserve(g_producer, bytes, &at);
+  const int rc = producer_reserve(bytes, &at);
   if (rc) return rc;
-  g_producer.reserved = true;
-  g_producer.reserved_at = at;
-  g_producer.reserved_bytes = bytes;
+  g_prod.reserved = true;
+  g_prod.reserved_at = at;
+  g_prod.reserved_bytes = bytes;
   *ptr = static_cast<char*>(g_producer.mem) + at;
   return BIKV_OK;
 }
 
 extern "C" int bikv_producer_publish(const int64_t* shape, size_t ndim, int32_t dtype_code, void* stream) {
+  std::lock_guard<std::mutex> lk(g_prod.mu);
   if (!g_producer.ctrl || !g_producer.mem) return fail(BIKV_ESTATE, "producer is not initialised");
-  if (!g_producer.reserved) return fail(BIKV_ESTATE, "nothing is reserved (call bikv_producer_reserve first)");
+  if (!g_prod.reserved) return fail(BIKV_ESTATE, "nothing is reserved (call bikv_producer_reserve first)");
   if (ndim > BIKV_MAX_DIM) return fail(BIKV_EINVAL, "at most %d dimensions can be published", BIKV_MAX_DIM);
   if (ndim > 0 && !shape) return fail(BIKV_EINVAL, "null pointer argument");
   BIKV_DEVICE(g_producer.device);
@@ -447,31 +398,33 @@ extern "C" int bikv_producer_publish(const int64_t* shape, size_t ndim, int32_t 
   // (the caller's own launches report into the shared status bank: a flag raised by ANY unchecked
   // launch on this device since the last bikv_check_status fails the publication)
   int rc = sync_and_check(g_producer.device, ST_BANK_SHARED, static_cast<hipStream_t>(stream));
-  if (rc == BIKV_EBOUNDS) g_producer.reserved = false;   // the window is incomplete: it is never published
+  if (rc == BIKV_EBOUNDS) g_prod.reserved = false;   // the window is incomplete: it is never published
   if (rc) return rc;
-  rc = producer_wait_slot(g_producer);
+  rc = producer_wait_slot();
   if (rc) return rc;
-  g_producer.reserved = false;
-  ring_publish(g_producer.ctrl, g_producer.reserved_at, g_producer.reserved_bytes, shape, ndim, dtype_code);
-  producer_published(g_producer, g_producer.reserved_at, g_producer.reserved_bytes);
+  g_prod.reserved = false;
+  ring::publish_transfer(g_prod, g_prod.reserved_at, g_prod.reserved_bytes, shape, ndim, dtype_code);
   return BIKV_OK;
 }
 
 extern "C" int bikv_producer_cancel(void) {
+  std::lock_guard<std::mutex> lk(g_prod.mu);
   if (!g_producer.ctrl) return fail(BIKV_ESTATE, "producer is not initialised");
-  g_producer.reserved = false;   // nothing was published: the window is handed out again next time
+  g_prod.reserved = false;   // nothing was published: the window is handed out again next time
   return BIKV_OK;
 }
 
 extern "C" int bikv_producer_set_backpressure(int enabled, int64_t timeout_ms) {
+  std::lock_guard<std::mutex> lk(g_prod.mu);
   if (!g_producer.ctrl) return fail(BIKV_ESTATE, "producer is not initialised");
-  g_producer.backpressure = enabled != 0;
-  g_producer.bp_timeout_ms = timeout_ms;
-  if (!enabled) g_producer.in_flight.clear();
+  g_prod.backpressure = enabled != 0;
+  g_prod.bp_timeout_ms = timeout_ms;
+  if (!enabled) g_prod.in_flight.clear();
   return BIKV_OK;
 }
 
 extern "C" int bikv_consumer_release(void) {
+  std::shared_lock<std::shared_mutex> lk(g_cons_mu);
   if (!g_consumer.ctrl) return fail(BIKV_ESTATE, "consumer is not initialised");
   if (sem_post(sem_of(g_consumer.ctrl->sem_complete)) != 0)
     return fail(BIKV_ESYS, "sem_post(sem_complete) failed: %s", strerror(errno));
@@ -481,15 +434,14 @@ extern "C" int bikv_consumer_release(void) {
 extern "C" int bikv_consumer_receive(int64_t timeout_ms, void** ptr, int64_t shape[BIKV_MAX_DIM],
                                      size_t* ndim, size_t* data_bytes, int32_t* device_id,
                                      int32_t* dtype_code) {
+  // shared: the role cannot be cleaned up while this call waits, and a release can still run beside it
+  std::shared_lock<std::shared_mutex> lk(g_cons_mu);
   if (!g_consumer.ctrl || !g_consumer.mem) return fail(BIKV_ESTATE, "consumer is not initialised");
   if (!ptr || !shape || !ndim) return fail(BIKV_EINVAL, "null pointer argument");
   bikv_shared_control* c = g_consumer.ctrl;
-  sem_t* s = sem_of(c->sem_start);
-  const int rc = wait_ms(s, timeout_ms);
-  if (rc == -1) {
-    if (errno == ETIMEDOUT) return fail(BIKV_ESTATE, "consumer_receive timed out after %lld ms", (long long)timeout_ms);
-    return fail(BIKV_ESYS, "consumer_receive sem_wait failed: %s", strerror(errno));
-  }
+  const int rc = ring::wait_ms(sem_of(c->sem_start), timeout_ms);
+  if (rc == ring::WAIT_TIMEOUT) return fail(BIKV_ESTATE, "consumer_receive timed out after %lld ms", (long long)timeout_ms);
+  if (rc == ring::WAIT_ERROR) return fail(BIKV_ESYS, "consumer_receive sem_wait failed: %s", strerror(errno));
   if (c->tensor_dim > BIKV_MAX_DIM) return fail(BIKV_ESTATE, "control block holds %zu dimensions", c->tensor_dim);
   *ptr = static_cast<char*>(g_consumer.mem) + c->last_valid_offset;
   *ndim = c->tensor_dim;

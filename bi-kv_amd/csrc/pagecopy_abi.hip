@@ -2,6 +2,8 @@
 // gather/scatter entry points, the run copy and the device->pinned-host staging pipeline.
 // Declarations and the reference call sites each entry point replaces: include/bikv_pagecopy.h.
 #include "../../include/bikv_pagecopy.h"
+#include "host_logic/chunk_planner.h"
+#include "host_logic/host_checks.h"
 #include "pagecopy_internal.h"
 #include "pagecopy_kernels.h"
 
@@ -404,23 +406,8 @@ static int move_pages(int bank, int dir, const bikv_pool* pool, const bikv_page_
 // copy of the caller's device ids before they launch (a debugging aid: it synchronises the stream).
 extern "C" int bikv_find_duplicate(const int64_t* ids, int64_t n, int64_t* dup_out) {
   if (n < 0 || (n > 0 && !ids)) return fail(BIKV_EINVAL, "bad find_duplicate arguments");
-  std::vector<std::pair<int64_t, int64_t>> v((size_t)n);
-  for (int64_t i = 0; i < n; ++i) v[(size_t)i] = {ids[i], i};
-  std::sort(v.begin(), v.end());
-  // report the repeated id whose second occurrence comes first in the caller's order (within a group
-  // of equal ids the positions ascend, because the pairs were sorted)
-  int64_t best = -1, best_first = 0, best_id = 0;
-  for (size_t i = 0; i + 1 < v.size();) {
-    size_t j = i + 1;
-    while (j < v.size() && v[j].first == v[i].first) ++j;
-    if (j - i >= 2 && (best < 0 || v[i + 1].second < best)) {
-      best = v[i + 1].second;
-      best_first = v[i].second;
-      best_id = v[i].first;
-    }
-    i = j;
-  }
-  if (best < 0) return BIKV_OK;
+  int64_t best_id = 0, best_first = 0, best = 0;
+  if (!find_first_duplicate(ids, n, &best_id, &best_first, &best)) return BIKV_OK;
   if (dup_out) *dup_out = best_id;
   return fail(BIKV_EINVAL, "destination id %lld is named more than once (entries %lld and %lld): a scatter's "
                            "destinations must be unique", (long long)best_id, (long long)best_first, (long long)best);
@@ -694,76 +681,6 @@ extern "C" int bikv_stager_destroy(bikv_stager* st) {
 }
 
 namespace bikv {
-
-// One contiguous byte range of the staging image together with the rectangle of
-// (batch pages x planes) that fills it.
-struct Chunk {
-  int64_t first_page, n_pages;  // batch entries
-  int plane_begin, plane_count;
-  int64_t first_slot, n_slots;  // staging slots covered
-};
-
-// Cuts the staging image of a batch into pieces of at most `max_slots` slots, one per call of next().
-// Requests are packed back to back in batch order. Holds no memory of its own.
-class ChunkPlanner {
- public:
-  ChunkPlanner(const int64_t* req_pages, int64_t n_req, int n_planes, int layout, int64_t max_slots)
-      : req_(req_pages), n_req_(n_req), planes_(n_planes), layout_(layout), max_(max_slots) {
-    if (layout_ == BIKV_LAYOUT_PAGE_MAJOR)
-      for (int64_t r = 0; r < n_req_; ++r) total_ += req_[r];
-  }
-
-  bool next(Chunk* out) {
-    if (layout_ == BIKV_LAYOUT_PAGE_MAJOR) {
-      // slot = global_page * n_planes + plane: any run of whole pages is contiguous, across requests
-      if (p_ >= total_) return false;
-      if (max_ >= planes_) {
-        const int64_t per = max_ / planes_;
-        const int64_t n = total_ - p_ < per ? total_ - p_ : per;
-        *out = Chunk{p_, n, 0, planes_, p_ * planes_, n * planes_};
-        p_ += n;
-      } else {
-        // a piece is smaller than one page: cut every page into runs of consecutive planes
-        const int c = planes_ - q_ < (int)max_ ? planes_ - q_ : (int)max_;
-        *out = Chunk{p_, 1, q_, c, p_ * planes_ + q_, c};
-        q_ += c;
-        if (q_ >= planes_) { q_ = 0; ++p_; }
-      }
-      return true;
-    }
-    while (r_ < n_req_ && req_[r_] == 0) ++r_;
-    if (r_ >= n_req_) return false;
-    const int64_t m = req_[r_];
-    if (m <= max_) {
-      int k = (int)(max_ / m);  // whole plane rows per piece
-      if (k > planes_) k = planes_;
-      const int c = planes_ - q_ < k ? planes_ - q_ : k;
-      *out = Chunk{first_page_, m, q_, c, base_slot_ + (int64_t)q_ * m, (int64_t)c * m};
-      q_ += c;
-    } else {
-      const int64_t n = m - j_ < max_ ? m - j_ : max_;
-      *out = Chunk{first_page_ + j_, n, q_, 1, base_slot_ + (int64_t)q_ * m + j_, n};
-      j_ += n;
-      if (j_ >= m) { j_ = 0; ++q_; }
-    }
-    if (q_ >= planes_) {
-      q_ = 0;
-      first_page_ += m;
-      base_slot_ += m * planes_;
-      ++r_;
-    }
-    return true;
-  }
-
- private:
-  const int64_t* req_;
-  int64_t n_req_;
-  int planes_, layout_;
-  int64_t max_;
-  int64_t total_ = 0, p_ = 0;                       // page-major walk
-  int64_t r_ = 0, j_ = 0, first_page_ = 0, base_slot_ = 0;
-  int q_ = 0;
-};
 
 // The lanes a pipeline call runs on: the stager's own, or (allocation-free entry point) the caller's
 // stream with a buffer that already exists.

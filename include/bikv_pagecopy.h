@@ -427,7 +427,11 @@ int bikv_nhd_store_token_major(const bikv_nhd* pool, void* tm, int64_t tm_bytes,
  * creates the shm object and the device ring buffer and stores a 64-byte hipIpcMemHandle_t in
  * `ipc_handle`; a producer in another process maps it, a producer in the SAME process uses the
  * consumer's pointer directly. One producer role and one consumer role per process, as in the
- * reference (ipc_service.cpp:9-17); not thread-safe.
+ * reference (ipc_service.cpp:9-17), whose callers are gRPC thread pools: unlike the reference's, these
+ * entry points may be called from several threads at once. A producer call holds the producer's lock from
+ * its ring window to its publication (the copy included), so concurrent producer calls run one after the
+ * other and every transfer gets a window and a publication of its own; init and cleanup exclude
+ * everything else of their role; bikv_consumer_receive and bikv_consumer_release may run side by side.
  * ------------------------------------------------------------------------------------------ */
 #define BIKV_IPC_HANDLE_SIZE 64
 #define BIKV_MAX_DIM 5

@@ -1,0 +1,192 @@
+// Drives the library's pure host logic under the address and undefined-behaviour sanitizers.
+// Every check aborts with a message on failure; "host_logic ok" on stdout means all passed.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <limits>
+#include <random>
+#include <vector>
+
+#include "chunk_planner.h"
+#include "host_checks.h"
+#include "ring_logic.h"
+
+using namespace bikv;
+
+#define REQUIRE(cond, ...)                                                   \
+  do {                                                                       \
+    if (!(cond)) {                                                           \
+      fprintf(stderr, "%s:%d: %s failed: ", __FILE__, __LINE__, #cond);      \
+      fprintf(stderr, __VA_ARGS__);                                          \
+      fprintf(stderr, "\n");                                                 \
+      abort();                                                               \
+    }                                                                        \
+  } while (0)
+
+// Every slot of the staging image is covered exactly once, in ascending order, by pieces of at most
+// max_slots slots whose (pages x planes) rectangle maps onto exactly the slots they claim.
+static void check_plan(const std::vector<int64_t>& req, int planes, int layout, int64_t max_slots) {
+  int64_t total_pages = 0;
+  for (int64_t m : req) total_pages += m;
+  std::vector<int64_t> req_first(req.size() + 1, 0);
+  for (size_t r = 0; r < req.size(); ++r) req_first[r + 1] = req_first[r] + req[r];
+  ChunkPlanner plan(req.data(), (int64_t)req.size(), planes, layout, max_slots);
+  Chunk c;
+  int64_t next_slot = 0, steps = 0;
+  std::vector<unsigned char> seen((size_t)(total_pages * planes), 0);
+  while (plan.next(&c)) {
+    ++steps;
+    REQUIRE(steps <= total_pages * planes + 1, "planner does not terminate");
+    REQUIRE(c.n_slots >= 1 && c.n_slots <= max_slots, "n_slots %lld max %lld", (long long)c.n_slots, (long long)max_slots);
+    REQUIRE(c.first_slot == next_slot, "pieces not back to back: %lld vs %lld", (long long)c.first_slot, (long long)next_slot);
+    REQUIRE(c.n_slots == c.n_pages * c.plane_count, "rectangle %lld x %d != %lld slots", (long long)c.n_pages, c.plane_count, (long long)c.n_slots);
+    REQUIRE(c.plane_begin >= 0 && c.plane_begin + c.plane_count <= planes && c.plane_count >= 1, "planes");
+    REQUIRE(c.first_page >= 0 && c.first_page + c.n_pages <= total_pages, "pages");
+    // the slots the kernel will compute for this rectangle (slot = base + j + q*m, or page*planes + q)
+    size_t r = 0;
+    while (req_first[r + 1] <= c.first_page) ++r;
+    for (int64_t i = c.first_page; i < c.first_page + c.n_pages; ++i) {
+      if (layout == BIKV_LAYOUT_LAYER_MAJOR) REQUIRE(i < req_first[r + 1], "a piece spans two requests");
+      for (int q = c.plane_begin; q < c.plane_begin + c.plane_count; ++q) {
+        const int64_t slot = layout == BIKV_LAYOUT_PAGE_MAJOR
+                                 ? i * planes + q
+                                 : req_first[r] * planes + (i - req_first[r]) + (int64_t)q * req[r];
+        REQUIRE(slot >= c.first_slot && slot < c.first_slot + c.n_slots, "slot %lld outside its piece", (long long)slot);
+        REQUIRE(!seen[(size_t)slot], "slot %lld covered twice", (long long)slot);
+        seen[(size_t)slot] = 1;
+      }
+    }
+    next_slot += c.n_slots;
+  }
+  REQUIRE(next_slot == total_pages * planes, "image not covered: %lld of %lld", (long long)next_slot, (long long)(total_pages * planes));
+}
+
+static void test_planner() {
+  std::mt19937_64 rng(7);
+  for (int it = 0; it < 3000; ++it) {
+    const int n_req = (int)(rng() % 6);
+    std::vector<int64_t> req((size_t)n_req);
+    for (auto& m : req) m = (int64_t)(rng() % 4 == 0 ? 0 : rng() % 40);
+    const int planes = 1 + (int)(rng() % 9);
+    const int layout = (int)(rng() % 2);
+    const int64_t max_slots = 1 + (int64_t)(rng() % 70);
+    check_plan(req, planes, layout, max_slots);
+  }
+  // extremes: one-slot pieces, a lane buffer far larger than anything, single-page requests with a huge
+  // budget (the rows-per-piece quotient is then enormous)
+  check_plan({5, 1, 3}, 4, BIKV_LAYOUT_LAYER_MAJOR, 1);
+  check_plan({5, 1, 3}, 4, BIKV_LAYOUT_PAGE_MAJOR, 1);
+  check_plan({1, 1, 1}, 3, BIKV_LAYOUT_LAYER_MAJOR, std::numeric_limits<int64_t>::max() / 2);
+  check_plan({7, 2}, 160, BIKV_LAYOUT_PAGE_MAJOR, std::numeric_limits<int64_t>::max() / 2);
+  check_plan({}, 3, BIKV_LAYOUT_LAYER_MAJOR, 8);
+  check_plan({0, 0}, 3, BIKV_LAYOUT_PAGE_MAJOR, 8);
+}
+
+static void test_duplicates() {
+  std::mt19937_64 rng(11);
+  const int64_t lo = std::numeric_limits<int64_t>::min(), hi = std::numeric_limits<int64_t>::max();
+  for (int it = 0; it < 4000; ++it) {
+    const int n = (int)(rng() % 12);
+    std::vector<int64_t> ids((size_t)n);
+    for (auto& x : ids) {
+      const unsigned k = (unsigned)(rng() % 10);
+      x = k == 0 ? lo : k == 1 ? hi : (int64_t)(rng() % 9) - 4;
+    }
+    // brute force: the smallest position that repeats an earlier one
+    int64_t want_second = -1, want_first = -1;
+    for (int j = 1; j < n && want_second < 0; ++j)
+      for (int i = 0; i < j; ++i)
+        if (ids[(size_t)i] == ids[(size_t)j]) { want_second = j; want_first = i; break; }
+    int64_t id = 0, first = 0, second = 0;
+    const bool got = find_first_duplicate(ids.data(), n, &id, &first, &second);
+    REQUIRE(got == (want_second >= 0), "presence");
+    if (got) {
+      REQUIRE(second == want_second, "second occurrence %lld want %lld", (long long)second, (long long)want_second);
+      REQUIRE(ids[(size_t)first] == id && ids[(size_t)second] == id && first < second, "entries");
+      // `first` is the FIRST entry holding that id
+      for (int i = 0; i < first; ++i) REQUIRE(ids[(size_t)i] != id, "first is not the first");
+      (void)want_first;
+    }
+  }
+  int64_t a = 0, b = 0, c = 0;
+  REQUIRE(!find_first_duplicate(nullptr, 0, &a, &b, &c), "empty");
+}
+
+static void test_interleave() {
+  for (size_t n_same = 0; n_same <= 40; ++n_same)
+    for (size_t n_other = 0; n_other <= 40; ++n_other) {
+      const std::vector<bool> o = interleave_order(n_same, n_other);
+      const size_t n = n_same + n_other;
+      REQUIRE(o.size() == n, "size");
+      size_t others = 0;
+      for (size_t k = 0; k < n; ++k) {
+        others += o[k] ? 1 : 0;
+        // every prefix holds the "other" kind in the proportion of the whole, to within one chunk
+        const double ideal = n ? (double)(k + 1) * (double)n_other / (double)n : 0.0;
+        REQUIRE((double)others >= ideal - 1.0 && (double)others <= ideal + 1.0, "prefix %zu of (%zu, %zu): %zu others, ideal %.2f",
+                k, n_same, n_other, others, ideal);
+      }
+      REQUIRE(others == n_other, "count");
+    }
+}
+
+static void test_ring() {
+  bikv_shared_control* c = static_cast<bikv_shared_control*>(malloc(sizeof(bikv_shared_control)));
+  memset(c, 0xEE, sizeof(*c));
+  bikv_shared_control image;
+  memset(&image, 0, sizeof(image));
+  image.buffer_size = 1000;
+  image.device_id = 3;
+  strcpy(image.hostname, "host-a");
+  ring::describe_ring(c, image);
+  REQUIRE(ring::describes_ring(c) == 1000 && c->device_id == 3 && c->current_offset == 0, "describe_ring");
+  ring::Producer p;
+  p.ctrl = c;
+  // the reference's wrap sequence for transfers of 400 bytes in a ring of 1000: 0, 400, 0, 400, 0
+  const int64_t shape[5] = {4, 5, 2, 10, 1};
+  const size_t want[5] = {0, 400, 0, 400, 0};
+  for (int k = 0; k < 5; ++k) {
+    size_t at = 77;
+    REQUIRE(ring::reserve_window(p, 400, &at) == ring::WAIT_OK && at == want[k], "wrap step %d: %zu", k, at);
+    ring::publish_transfer(p, at, 400, shape, 5, 0);
+    REQUIRE(c->last_valid_offset == want[k] && c->current_offset == want[k] + 400 && c->data_size == 400 && c->tensor_dim == 5 &&
+                c->tensor_shape[3] == 10, "publish step %d", k);
+    REQUIRE(ring::wait_ms(ring::sem_of(c->sem_start), 0) == ring::WAIT_OK, "one post per transfer");
+  }
+  REQUIRE(ring::wait_ms(ring::sem_of(c->sem_start), 1) == ring::WAIT_TIMEOUT, "no extra post");
+  // a transfer that exactly fills the rest does not wrap; one byte more does
+  c->current_offset = 600;
+  size_t at = 0;
+  ring::reserve_window(p, 400, &at);
+  REQUIRE(at == 600, "exact fit");
+  c->current_offset = 601;
+  ring::reserve_window(p, 400, &at);
+  REQUIRE(at == 0, "wrap");
+  // back-pressure: a published transfer blocks the publication of the next until it is released, and
+  // a window that overlaps it until then; with a timeout both report WAIT_TIMEOUT and change nothing
+  p.backpressure = true;
+  p.bp_timeout_ms = 20;
+  c->current_offset = 0;
+  ring::reserve_window(p, 600, &at);
+  REQUIRE(at == 0 && ring::wait_slot(p) == ring::WAIT_OK, "first transfer");
+  ring::publish_transfer(p, at, 600, shape, 5, 0);
+  REQUIRE(p.in_flight.size() == 1, "in flight");
+  REQUIRE(ring::reserve_window(p, 300, &at) == ring::WAIT_OK && at == 600, "disjoint window needs no wait");
+  REQUIRE(ring::wait_slot(p) == ring::WAIT_TIMEOUT && p.in_flight.size() == 1, "the slot is taken");
+  REQUIRE(ring::reserve_window(p, 600, &at) == ring::WAIT_TIMEOUT, "overlapping window waits");   // wraps to 0
+  sem_post(ring::sem_of(c->sem_complete));      // the consumer releases
+  REQUIRE(ring::reserve_window(p, 600, &at) == ring::WAIT_OK && at == 0 && p.in_flight.empty(), "released");
+  REQUIRE(ring::wait_slot(p) == ring::WAIT_OK, "slot free");
+  sem_destroy(ring::sem_of(c->sem_start));
+  sem_destroy(ring::sem_of(c->sem_complete));
+  free(c);
+}
+
+int main() {
+  test_planner();
+  test_duplicates();
+  test_interleave();
+  test_ring();
+  printf("host_logic ok\n");
+  return 0;
+}
