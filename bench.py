@@ -54,6 +54,33 @@ MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9948, "scatter": 1.0002},
                           "layout_change": {"load": 1.0029, "store": 1.0035}}
 
 
+# The ratios above describe the kernels as they were when the counters were read: the SHA-256 (first 16 hex
+# digits) of the two kernel sources at that time. A run whose kernel sources differ reports `traffic: null`
+# and says why, so that a change which re-reads data cannot keep printing an old ratio.
+TRAFFIC_MEASURED_AT = "to-be-measured"
+
+
+def kernel_source_digest():
+    import hashlib
+    h = hashlib.sha256()
+    for f in ("pagecopy_kernels.hip", "transpose_kernels.hip"):
+        with open(os.path.join(ROOT, "bi-kv_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def traffic_ratio(workload, kind):
+    """(ratio or None, source text) for `traffic` of the dominant kernel."""
+    r = MEASURED_TRAFFIC_RATIO.get(workload, {}).get(kind)
+    if r is None:
+        return None, None
+    now = kernel_source_digest()
+    if now != TRAFFIC_MEASURED_AT:
+        return None, (f"not reported: the kernel sources (digest {now}) are not the ones the counters under profiles/ were "
+                      f"read from (digest {TRAFFIC_MEASURED_AT})")
+    return r, TRAFFIC_SOURCE
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -443,9 +470,9 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layo
     dominant_is_gather = (s_stat is None) or (float(np.sum(g_ms)) >= float(np.sum(s_ms)))
     kname = "bikv::tile_move_wave_kernel<0=gather>" if dominant_is_gather else "bikv::tile_move_wave_kernel<1=scatter>"
     dom = g_stat if dominant_is_gather else s_stat
-    ratio = MEASURED_TRAFFIC_RATIO.get(name, {}).get("gather" if dominant_is_gather else "scatter")
+    ratio, ratio_src = traffic_ratio(name, "gather" if dominant_is_gather else "scatter")
     if args.pool_pages or layout != "layer_major" or pool_form == "worker":
-        ratio = None                                   # measured on the full-size layer-major workload only
+        ratio, ratio_src = None, None                  # measured on the full-size layer-major workload only
     out = {
         "metric": "paged-KV gather/scatter HBM GB/s (% of MI355X peak) + pages/s, bit-exact",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
@@ -474,7 +501,7 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layo
         "roofline": {"bound": "hbm", "kernel": kname, "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
                      "traffic": (round(ratio * dom["alg_bytes"]) if ratio else None),
-                     "traffic_source": TRAFFIC_SOURCE if ratio else None,
+                     "traffic_source": ratio_src,
                      "alg_bytes_per_launch": dom["alg_bytes"], "avg_launch_ms": dom["avg_ms"]},
         "kernels": {"gather": g_stat, "scatter": s_stat,
                     "plain_copy_2GiB": ({"GBps": round(copy_gbps, 1)} if with_copy else None)},
@@ -513,8 +540,17 @@ def link_yardstick(bk, dev, host, dev_buf, reps=3):
 def run_staging(args, bk, workloads, dev, kept=None):
     """Llama-3-8B shape: every request of the log-normal stream gathered into pinned host memory, and
     scattered back from it, through the staging pipeline. All requests of a pass are enqueued back to back
-    (one wait at the end); a cell is min / median over the passes, next to a plain hipMemcpyAsync of one
-    1 GiB pinned buffer timed immediately before the cell (the host-link yardstick)."""
+    (one wait at the end). The record has three parts, in the order they are measured:
+
+    first_pass  the first pass of a fresh stager in every mode, taken the moment the pool is ready — no
+                warm-up, whatever state the process is in (this benchmark has just freed hundreds of GB of
+                device memory, which the driver scrubs in the background at ~15 GB/s; every hipMemcpyAsync
+                between host and device runs at about half rate until that is done);
+    cells       once a plain hipMemcpyAsync is back at its full rate (the wait is reported), chunk sizes,
+                lane counts and modes, three timed passes each after two untimed ones, each next to a plain
+                hipMemcpyAsync of one 1 GiB pinned buffer timed immediately before it;
+    during_scrub  the same modes measured while the driver is scrubbing 32 GiB that was freed a moment
+                before: which of them depend on the copy engines and which do not."""
     import numpy as np
     import torch
 
@@ -533,11 +569,6 @@ def run_staging(args, bk, workloads, dev, kept=None):
     region = int(max(4 << 30, 2 * sizes.max()))
     host = bk.pinned_empty(region)
     dev_buf = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-    dev_buf.random_(0, 256)
-    # the first DMA into a pinned page is slower than later ones: touch the whole region once
-    for off in range(0, region, dev_buf.numel()):
-        n = min(dev_buf.numel(), region - off)
-        host[off: off + n].copy_(dev_buf[:n])
     # every request gets a window of the pinned region; windows rotate through it, so requests in flight
     # together (neighbours in issue order) never share host bytes
     offs, cur = [], 0
@@ -553,44 +584,46 @@ def run_staging(args, bk, workloads, dev, kept=None):
     total_bytes = int(sizes.sum())
     passes = max(1, args.staging_passes)
     yard = {"d2h": [], "h2d": []}
+    # a prefix of the stream of about 10 GB: what the first-pass and scrub measurements move
+    n_short = int(np.searchsorted(np.cumsum(sizes), 10e9)) + 1
+    short_bytes = int(sizes[:n_short].sum())
+
+    def one_pass(stager, mode, direction, n_req=None, synchronous=False):
+        n_req = len(reqs) if n_req is None else n_req
+        batches = g_batches if direction == "gather" else s_batches
+        t0 = time.perf_counter()
+        for b, off, sz in list(zip(batches, offs, sizes))[:n_req]:
+            win = host[off: off + int(sz)]
+            if synchronous:
+                (stager.gather_to_host if direction == "gather" else stager.scatter_from_host)(pool, b, win, mode)
+            else:
+                (stager.gather_to_host_async if direction == "gather" else stager.scatter_from_host_async)(pool, b, win, mode)
+        if not synchronous:
+            stager.wait()
+        return int(sizes[:n_req].sum()) / (time.perf_counter() - t0) / 1e9
+
+    def small_copy_rate(direction, seconds=0.15):
+        """Rate of back-to-back plain hipMemcpyAsync calls of 64 MiB for about `seconds`: the probe that tells
+        whether the copy engines are at full rate."""
+        n, best, t_end = 64 << 20, 0.0, time.perf_counter() + seconds
+        while True:
+            if direction == "d2h":
+                best = max(best, n / bk.measure_d2h(dev, host[:n], dev_buf[:n], 0) / 1e9)
+            else:
+                best = max(best, n / bk.measure_h2d(dev, dev_buf[:n], host[:n], 0) / 1e9)
+            if time.perf_counter() >= t_end:
+                return best
 
     def cell(stager, mode, direction, synchronous=False):
-        untimed = 2 if stager.n_buffers <= 2 else 4     # a stager with four new lanes takes longer to settle
         d2h, h2d = link_yardstick(bk, dev, host[: dev_buf.numel()], dev_buf)
         yard["d2h"].append(d2h)
         yard["h2d"].append(h2d)
         link = d2h if direction == "gather" else h2d
-        batches = g_batches if direction == "gather" else s_batches
-        rates = []
-        for p in range(passes + untimed):
-            t0 = time.perf_counter()
-            for b, off, sz in zip(batches, offs, sizes):
-                win = host[off: off + int(sz)]
-                if synchronous:
-                    (stager.gather_to_host if direction == "gather" else stager.scatter_from_host)(pool, b, win, mode)
-                else:
-                    (stager.gather_to_host_async if direction == "gather" else stager.scatter_from_host_async)(pool, b, win, mode)
-            if not synchronous:
-                stager.wait()
-            if p >= untimed:
-                rates.append(total_bytes / (time.perf_counter() - t0) / 1e9)
+        rates = [one_pass(stager, mode, direction, synchronous=synchronous) for _ in range(passes + 2)][2:]
         return {"GBps_min": round(min(rates), 2), "GBps_median": round(float(np.median(rates)), 2),
                 "plain_GBps_just_before": round(link, 2),
                 "frac_min": round(min(rates) / link, 4), "frac_median": round(float(np.median(rates)) / link, 4),
                 "passes_GBps": [round(r, 2) for r in rates]}
-
-    def warm_up(stager, seconds):
-        """Untimed passes of the first cell's shape for a fixed time. Now and then a process spends its
-        first 7-15 s of staging at about 35 GB/s (seen with 4 MiB chunks out of the pool; the plain copy
-        timed next to it is at full rate) before it settles for good; the rates seen are kept in the record."""
-        seen, t_start = [], time.perf_counter()
-        while time.perf_counter() - t_start < seconds:
-            t0 = time.perf_counter()
-            for b, off, sz in zip(g_batches, offs, sizes):
-                stager.gather_to_host_async(pool, b, host[off: off + int(sz)], "pipelined")
-            stager.wait()
-            seen.append(round(total_bytes / (time.perf_counter() - t0) / 1e9, 2))
-        return {"seconds": seconds, "passes_GBps": seen}
 
     def verify(stager, mode):
         """Three requests (smallest, median, largest below 1 GiB) staged synchronously and compared, every
@@ -613,6 +646,44 @@ def run_staging(args, bk, workloads, dev, kept=None):
                 if not torch.equal(torch.index_select(pool_t[q], 0, idt2).cpu(), view[q]):
                     raise SystemExit(f"bench: scattered bytes differ ({mode}, request {i}, plane {q})")
 
+    MODES = ("auto", "pipelined_kernel", "pipelined")
+
+    def sweep_modes():
+        """One pass of ~10 GB per mode and direction, each in a stager created for it, with the rate of small
+        plain copies taken right before and after (are the copy engines at full rate?)."""
+        rec = {}
+        for direction, probe in (("gather", "d2h"), ("scatter", "h2d")):
+            for mode in MODES:
+                st = bk.HostStager(dev)
+                before = small_copy_rate(probe, 0.05)
+                r = one_pass(st, mode, direction, n_short)
+                after = small_copy_rate(probe, 0.05)
+                st.close()
+                rec[f"{direction}_{mode}"] = {"GBps": round(r, 2), "plain_64MiB_copies_before_GBps": round(before, 2),
+                                              "plain_64MiB_copies_after_GBps": round(after, 2)}
+        return rec
+
+    # --- 1. first pass of every mode, no warm-up, in whatever state this process is in
+    t_part = time.perf_counter()
+    first = sweep_modes()
+    first["what"] = (f"first pass of a fresh stager per mode (library defaults: 16 MiB x 2 copies per launch x 2 lanes), "
+                     f"{n_short} requests = {short_bytes / 1e9:.1f} GB, no warm-up of any kind; 'plain' = back-to-back "
+                     "hipMemcpyAsync calls of 64 MiB right before / after the pass")
+    log(f"staging first_pass {first}")
+
+    # --- 2. wait until the copy engines are back at full rate (the scrub of what this run freed), then the cells
+    t_wait, settle = time.perf_counter(), []
+    while True:
+        r = small_copy_rate("d2h", 0.2)
+        settle.append(round(r, 1))
+        if (len(settle) >= 3 and min(settle[-3:]) > 50.0) or time.perf_counter() - t_wait > 60.0:
+            break
+    settle_s = time.perf_counter() - t_wait
+    # the first DMA into a pinned page is slower than later ones: the whole region has been touched by now
+    # only if the passes above covered it, so touch it once
+    for off in range(0, region, dev_buf.numel()):
+        n = min(dev_buf.numel(), region - off)
+        host[off: off + n].copy_(dev_buf[:n])
     if args.chunk_mib:
         grid = [(args.chunk_mib, args.buffers, args.per_launch)]
     else:
@@ -624,18 +695,18 @@ def run_staging(args, bk, workloads, dev, kept=None):
         stager = bk.HostStager(dev, chunk_bytes=chunk << 20, n_buffers=lanes, chunks_per_launch=group)
         if (chunk, lanes, group) == grid[0]:
             verify(stager, "pipelined")
-            warm = warm_up(stager, 0 if args.chunk_mib else 20.0)
+            verify(stager, "pipelined_kernel")
         row = {"mode": "pipelined", "chunk_MiB": chunk, "lanes": lanes, "copies_per_launch": group}
         if group == 1 and chunk < 16:
             row["contrast_case"] = "one kernel per small copy: the shape that makes small chunks slow, shown for contrast only"
-        for direction in ("gather", "scatter"):
-            row[direction + "_to_host" if direction == "gather" else "scatter_from_host"] = cell(stager, "pipelined", direction)
+        row["gather_to_host"] = cell(stager, "pipelined", "gather")
+        row["scatter_from_host"] = cell(stager, "pipelined", "scatter")
         log(f"staging {row}")
         cells.append(row)
         stager.close()
     stager = bk.HostStager(dev)          # the library's defaults: 16 MiB x 2 per launch x 2 lanes
     verify(stager, "direct")
-    for mode in ("direct", "auto"):
+    for mode in ("pipelined_kernel", "direct", "auto"):
         row = {"mode": mode, "chunk_MiB": stager.chunk_bytes >> 20, "lanes": stager.n_buffers,
                "copies_per_launch": stager.chunks_per_launch}
         row["gather_to_host"] = cell(stager, mode, "gather")
@@ -648,11 +719,43 @@ def run_staging(args, bk, workloads, dev, kept=None):
                 "scatter_from_host": cell(stager, "auto", "scatter", synchronous=True)}
     stager.close()
     auto = cells[-1]
+
+    # --- 3. the same modes while the driver scrubs device memory that was freed a moment before
+    scrub = None
+    if not args.chunk_mib:
+        scrub_gib = 32
+        free_b = torch.cuda.mem_get_info(dev)[0]
+        if free_b > (scrub_gib + 8) << 30:
+            scrub = {}
+            for direction, probe in (("gather", "d2h"), ("scatter", "h2d")):
+                for mode in MODES:
+                    st = bk.HostStager(dev)
+                    one_pass(st, mode, direction, 2)                     # the stager's streams and buffers exist
+                    x = torch.empty(scrub_gib << 30, dtype=torch.uint8, device=dev)
+                    del x
+                    torch.cuda.empty_cache()                             # hipFree: returns at once, the scrub starts
+                    before = small_copy_rate(probe, 0.05)
+                    r = one_pass(st, mode, direction, n_short)
+                    after = small_copy_rate(probe, 0.05)
+                    st.close()
+                    scrub[f"{direction}_{mode}"] = {"GBps": round(r, 2), "plain_64MiB_copies_before_GBps": round(before, 2),
+                                                    "plain_64MiB_copies_after_GBps": round(after, 2)}
+                    t_w = time.perf_counter()                            # let the scrub finish before the next case
+                    while small_copy_rate(probe, 0.1) < 50.0 and time.perf_counter() - t_w < 20.0:
+                        pass
+            scrub["what"] = (f"one pass of {short_bytes / 1e9:.1f} GB per mode, started right after {scrub_gib} GiB of device memory "
+                             "was allocated and freed (hipFree returns at once; the driver then scrubs the memory in the "
+                             "background for about 2 s, during which plain hipMemcpyAsync runs at ~30 GB/s in both directions)")
+            log(f"staging during_scrub {scrub}")
+
     out = {"workload": f"llama3_8b: {shape.n_pages} pages x {shape.n_planes} planes x {shape.tile_bytes} B, "
                        f"{len(reqs)} requests of {int(sizes.min() // shape.page_bytes)}..{int(sizes.max() // shape.page_bytes)} "
-                       f"pages ({total_bytes / 1e9:.2f} GB per pass), enqueued back to back, {passes} timed passes per cell after two untimed ones (four for a stager with four lanes)",
+                       f"pages ({total_bytes / 1e9:.2f} GB per pass), enqueued back to back, {passes} timed passes per cell after two untimed ones",
            "pool_GB": round(shape.pool_bytes / 1e9, 2),
-           "warm_up_before_the_first_cell": warm,
+           "first_pass": first,
+           "wait_for_full_rate_copies": {"seconds": round(settle_s, 2), "plain_64MiB_d2h_GBps_seen": settle,
+                                         "what": "time from the end of the first passes until back-to-back plain hipMemcpyAsync "
+                                                 "calls held > 50 GB/s three times in a row (60 s at most); nothing is staged meanwhile"},
            "plain_d2h_GBps": {"min": round(min(yard["d2h"]), 2), "median": round(float(np.median(yard["d2h"])), 2),
                               "max": round(max(yard["d2h"]), 2), "samples": len(yard["d2h"])},
            "plain_h2d_GBps": {"min": round(min(yard["h2d"]), 2), "median": round(float(np.median(yard["h2d"])), 2),
@@ -662,13 +765,17 @@ def run_staging(args, bk, workloads, dev, kept=None):
            "frac_of_best_plain_d2h_seen": round(auto["gather_to_host"]["GBps_median"] / max(yard["d2h"]), 4),
            "scatter_from_host_GBps": auto["scatter_from_host"]["GBps_median"],
            "scatter_frac_of_plain_h2d": auto["scatter_from_host"]["frac_median"],
-           "cells": cells, "per_request_blocking_calls": per_call, "bit_exact": True}
+           "cells": cells, "per_request_blocking_calls": per_call, "during_scrub": scrub, "bit_exact": True,
+           "seconds": round(time.perf_counter() - t_part, 1)}
     real = [c for c in cells if "contrast_case" not in c]
     out["min_frac_over_cells"] = {
         "gather_to_host": min(c["gather_to_host"]["frac_min"] for c in real),
         "scatter_from_host": min(c["scatter_from_host"]["frac_min"] for c in real),
         "what": "lowest single pass of any cell, as a fraction of the plain copy timed just before that cell "
                 "(every chunk size, lane count and mode above except the contrast case)"}
+    out["median_frac_over_cells"] = {
+        "gather_to_host": round(float(np.median([c["gather_to_host"]["frac_median"] for c in real])), 4),
+        "scatter_from_host": round(float(np.median([c["scatter_from_host"]["frac_median"] for c in real])), 4)}
     if kept is None:
         pool.close()
         del pool_t
@@ -757,6 +864,72 @@ def run_reference_scenario(args, bk, dev):
     }
 
 
+def run_reference_ipc(dev, transfers=10):
+    """The reference's own scenario through its own operator API, timed the way its script times it
+    (Bi-KV/SharedMemory/CUDA_Shared/test_page_ipc.py:41-102,127-162): producer and consumer roles of
+    `ipc_service` (here in one process), 200 pages x 50 tokens x (128, 2, 28, 2) fp16 = 273.4 MiB per
+    transfer, identity offsets, value 7. One untimed transfer, then `transfers` timed ones: each is one
+    blocking producer_copy_pages call (page copy into the ring, stream sync, publication) followed by one
+    consumer_receive; the producer's and the consumer's "Throughput" are the script's own formulas (MiB of
+    one transfer / mean call time). Beside it the same transfer on the reference's CPU path: torch.index_select
+    of the 200 page rows of a host tensor into a host buffer."""
+    import torch
+    import ipc_service
+
+    page_size, num_pages, head, kvh, layers, kv = 50, 200, 128, 2, 28, 2
+    page_elements = page_size * head * kvh * layers * kv
+    name = f"/bikv_bench_{os.getpid()}"
+    ipc_service.producer_cleanup()
+    ipc_service.consumer_cleanup()
+    ipc_service.consumer_init(0, name, (2 << 30) - 4096)     # the script's ring is 2 GiB; one that size is not exported over IPC
+    ipc_service.producer_init(0, name)
+    try:
+        cache = torch.full((num_pages, page_size, head, kvh, layers, kv), 7, dtype=torch.float16, device=dev)
+        offs = torch.arange(num_pages, dtype=torch.int64, device=dev) * page_elements
+        dims = ipc_service.TensorDims()
+        dims.total_tokens, dims.head_size, dims.num_kv_heads, dims.num_layers, dims.kv_pair = num_pages * page_size, head, kvh, layers, kv
+        torch.cuda.synchronize(dev)
+        prod, cons, result = [], [], None
+        for i in range(transfers + 1):
+            t0 = time.perf_counter()
+            ipc_service.producer_copy_pages(cache, offs, offs, page_size, dims)
+            t1 = time.perf_counter()
+            result = ipc_service.consumer_receive()
+            t2 = time.perf_counter()
+            if tuple(result.shape) != (num_pages * page_size, head, kvh, layers, kv):
+                raise SystemExit(f"bench: reference scenario published shape {tuple(result.shape)}")
+            if i:
+                prod.append(t1 - t0)
+                cons.append(t2 - t1)
+        if not bool((result == 7).all().item()):
+            raise SystemExit("bench: reference scenario data corrupted")
+        mib = cache.numel() * cache.element_size() / (1024 ** 2)
+    finally:
+        ipc_service.producer_cleanup()
+        ipc_service.consumer_cleanup()
+    # CPU twin: the same 200 page rows selected out of a host tensor
+    host = torch.full((num_pages, page_elements), 7, dtype=torch.float16)
+    out = torch.empty_like(host)
+    ids = torch.arange(num_pages, dtype=torch.int64)
+    cpu = []
+    for i in range(transfers + 1):
+        t0 = time.perf_counter()
+        torch.index_select(host, 0, ids, out=out)
+        if i:
+            cpu.append(time.perf_counter() - t0)
+    avg_p, avg_c = sum(prod) / len(prod), sum(cpu) / len(cpu)
+    return {"workload": "reference_200x50 through ipc_service.producer_copy_pages -> ring -> consumer_receive "
+                        "(test_page_ipc.py), one process, 1 untimed + %d timed transfers" % transfers,
+            "MiB_per_transfer": round(mib, 2),
+            "producer_avg_transfer_ms": round(avg_p * 1e3, 4), "producer_MiB_per_s": round(mib / avg_p, 1),
+            "consumer_avg_receive_ms": round(sum(cons) / len(cons) * 1e3, 4),
+            "consumer_MiB_per_s": round(mib * len(cons) / sum(cons), 1),
+            "HBM_GBps_read_plus_written": round(2 * mib * 1024 ** 2 / avg_p / 1e9, 1),
+            "cpu_index_select": {"avg_transfer_ms": round(avg_c * 1e3, 3), "MiB_per_s": round(mib / avg_c, 1),
+                                 "cores": torch.get_num_threads(), "kind": "port"},
+            "bit_exact": True}
+
+
 def run_token_major(args, bk, workloads, dev):
     """The Qwen2-7B request stream in the REFERENCE'S layout: a token-major pool of 131072 pages of
     16 tokens x (128, 4, 28, 2) bf16 = 917 504 bytes each (kvcache.py:38-43 at this shape), one run per
@@ -841,8 +1014,8 @@ def run_token_major(args, bk, workloads, dev):
                     "scatter": {"GBps": round(alg_s / s_ms / 1e6, 1), "avg_ms": round(s_ms, 4), "alg_bytes": alg_s}},
         "roofline": {"bound": "hbm", "kernel": "bikv::copy_runs_wave_kernel", "achieved": round(alg / ms / 1e6, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(alg / ms / 1e6 / HBM_PEAK_GBPS, 4),
-                     "traffic": (int(alg * MEASURED_TRAFFIC_RATIO["qwen2_7b_token_major"]["gather" if slow_g else "scatter"])
-                                 if not args.pool_pages else None),
+                     "traffic": (int(alg * traffic_ratio("qwen2_7b_token_major", "gather" if slow_g else "scatter")[0])
+                                 if not args.pool_pages and traffic_ratio("qwen2_7b_token_major", "gather")[0] else None),
                      "alg_bytes_per_launch": alg, "avg_launch_ms": round(ms, 4)},
     }
 
@@ -937,9 +1110,9 @@ def run_layout_change(args, bk, dev, blocks=None, sort=False, pool_alloc=None):
         "roofline": {"bound": "hbm", "kernel": f"bikv::transpose_pairs_kernel<{1 if slow_is_load else 0}, 2, 512>",
                      "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
-                     "traffic": (int(alg * MEASURED_TRAFFIC_RATIO["layout_change"]["load" if slow_is_load else "store"])
-                                 if at_reference_shape else None),
-                     "traffic_source": TRAFFIC_SOURCE if at_reference_shape else None,
+                     "traffic": (int(alg * traffic_ratio("layout_change", "load" if slow_is_load else "store")[0])
+                                 if at_reference_shape and traffic_ratio("layout_change", "load")[0] else None),
+                     "traffic_source": traffic_ratio("layout_change", "load")[1] if at_reference_shape else None,
                      "alg_bytes_per_launch": alg, "avg_launch_ms": dom["avg_ms"]},
         "kernels": {"load": l_stat, "store": s_stat},
     }
@@ -952,6 +1125,8 @@ def run_layout_change(args, bk, dev, blocks=None, sort=False, pool_alloc=None):
 def emit(out):
     if ALLOC_NOTES:
         out["device_alloc"] = ALLOC_NOTES
+    if "summary" in out:
+        out["summary"] = out.pop("summary")      # keeps it the last key of the line
     print(json.dumps(out), flush=True)
 
 
@@ -1041,10 +1216,85 @@ def main():
                 torch.cuda.empty_cache()
     elif args.workload == "llama3_8b" and not args.no_staging:
         out["staging"] = run_staging(args, bk, workloads, dev)
+    if default_run and not args.no_configs:
+        # the layout change at the reference's own shape (28 layer tensors [10240*16, 2, 2, 128] fp16), about
+        # a quarter of a second of launches, and the reference's scripted scenario through its operator API
+        import copy
+        lc_args = copy.copy(args)
+        lc_args.steps, lc_args.warmup = 200, 5
+        o = run_layout_change(lc_args, bk, dev)
+        out["layout_change"] = {"workload": o["config"]["workload"], "pool_GB": o["config"]["pool_GB"], "value": o["value"],
+                                "pct_of_hbm_peak": o["pct_of_hbm_peak"], "steps": o["steps"], "bit_exact": o["bit_exact"],
+                                "kernels": o["kernels"], "traffic": o["roofline"]["traffic"]}
+        log("the reference's 200 x 50 scenario through ipc_service")
+        out["reference_scenario"] = run_reference_ipc(dev)
     if not args.no_cpu_baseline:
         log("timing the CPU baseline")
         out["cpu_baseline"] = cpu_baseline(shape, wl)
+    if default_run:
+        add_summary(out)
     emit(out)
+
+
+def add_summary(out):
+    """The figures of the whole run, flat and short, under `config` (and once more as the last key of the line):
+    every named configuration's value and per-kernel fraction of 8 TB/s, the torch-allocated headline, the
+    staging record's fractions of the plain copy with its first passes, the layout change and the reference's
+    scenario. Keys are absent for parts that were skipped."""
+    frac = lambda gbps: round(gbps / HBM_PEAK_GBPS, 4)
+    sm = {"headline_value_GBps": out["value"],
+          "headline_gather_frac": frac(out["kernels"]["gather"]["GBps"]),
+          "headline_scatter_frac": frac(out["kernels"]["scatter"]["GBps"]) if out["kernels"]["scatter"] else None}
+    if "other_layout" in out:
+        sm["page_major_value_GBps"] = out["other_layout"]["value"]
+    if "torch_alloc" in out:
+        sm["torch_alloc_value_GBps"] = out["torch_alloc"]["value"]
+        for k, v in out["torch_alloc"]["kernels"].items():
+            if k in ("gather", "scatter"):
+                sm[f"torch_alloc_{k}_frac"] = frac(v["GBps"])
+    for name, c in (out.get("configs") or {}).items():
+        sm[f"{name}_value_GBps"] = c["value"]
+        sm[f"{name}_gather_frac"] = c["gather"]["frac"]
+        if c["scatter"]:
+            sm[f"{name}_scatter_frac"] = c["scatter"]["frac"]
+    st = out.get("staging")
+    if st:
+        sm["staging_host_link_GBps"] = st["host_link_GBps"]
+        sm["staging_plain_d2h_GBps"] = st["plain_d2h_GBps"]["median"]
+        sm["staging_plain_h2d_GBps"] = st["plain_h2d_GBps"]["median"]
+        sm["staging_auto_gather_frac_median"] = st["frac_of_plain_d2h"]
+        sm["staging_auto_scatter_frac_median"] = st["scatter_frac_of_plain_h2d"]
+        sm["staging_gather_frac_min_over_cells"] = st["min_frac_over_cells"]["gather_to_host"]
+        sm["staging_scatter_frac_min_over_cells"] = st["min_frac_over_cells"]["scatter_from_host"]
+        sm["staging_gather_frac_median_over_cells"] = st["median_frac_over_cells"]["gather_to_host"]
+        sm["staging_scatter_frac_median_over_cells"] = st["median_frac_over_cells"]["scatter_from_host"]
+        for k, v in st["first_pass"].items():
+            if isinstance(v, dict):
+                sm[f"staging_first_pass_{k}_GBps"] = v["GBps"]
+        sm["staging_wait_for_full_rate_copies_s"] = st["wait_for_full_rate_copies"]["seconds"]
+        for k, v in (st.get("during_scrub") or {}).items():
+            if isinstance(v, dict):
+                sm[f"staging_during_scrub_{k}_GBps"] = v["GBps"]
+    lc = out.get("layout_change")
+    if lc:
+        sm["layout_change_value_GBps"] = lc["value"]
+        sm["layout_change_load_frac"] = frac(lc["kernels"]["load"]["GBps"])
+        sm["layout_change_store_frac"] = frac(lc["kernels"]["store"]["GBps"])
+    rs = out.get("reference_scenario")
+    if rs:
+        sm["reference_200x50_producer_MiB_per_s"] = rs["producer_MiB_per_s"]
+        sm["reference_200x50_consumer_MiB_per_s"] = rs["consumer_MiB_per_s"]
+        sm["reference_200x50_cpu_index_select_MiB_per_s"] = rs["cpu_index_select"]["MiB_per_s"]
+        sm["reference_200x50_cpu_cores"] = rs["cpu_index_select"]["cores"]
+    for note in ALLOC_NOTES:
+        if note.get("what", "").startswith("qwen2_7b pool") and "seconds" in note:
+            sm["headline_pool_alloc_s"] = note["seconds"]
+            sm["headline_pool_alloc_fillers_GB"] = round(note["n_fillers"] * note["chunk_bytes"] / 1e9, 1)
+            sm["headline_pool_chunks_other_half"] = f"{note['n_other_half']} of {note['n_chunks']}"
+            break
+    for k, v in sm.items():
+        out["config"][k] = v
+    out["summary"] = sm          # emitted last: the end of the line is what a truncated log keeps
 
 
 if __name__ == "__main__":

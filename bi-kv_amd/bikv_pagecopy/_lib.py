@@ -72,7 +72,8 @@ class NHDDesc(C.Structure):
 
 class AllocInfo(C.Structure):
     _fields_ = [("bytes", C.c_int64), ("chunk_bytes", C.c_int64), ("n_chunks", C.c_int32),
-                ("n_other_half", C.c_int32), ("n_fillers", C.c_int32), ("reserved", C.c_int32)]
+                ("n_other_half", C.c_int32), ("n_fillers", C.c_int32), ("n_reprobed", C.c_int32),
+                ("seconds", C.c_double), ("pair_ms_same", C.c_float), ("pair_ms_other", C.c_float)]
 
 
 class StageStats(C.Structure):
@@ -168,6 +169,7 @@ _SIGNATURES = {
     "bikv_h2d_copy": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
                                 C.POINTER(C.c_double)]),
     "bikv_device_alloc": (C.c_int, [C.c_int, C.c_int64, C.c_int32, C.POINTER(C.c_void_p)]),
+    "bikv_device_alloc_bounded": (C.c_int, [C.c_int, C.c_int64, C.c_int32, C.c_int64, C.POINTER(C.c_void_p)]),
     "bikv_device_free": (C.c_int, [C.c_void_p]),
     "bikv_device_alloc_info": (C.c_int, [C.c_void_p, C.POINTER(AllocInfo)]),
     "bikv_host_alloc": (C.c_int, [C.c_int64, C.POINTER(C.c_void_p)]),

@@ -24,7 +24,9 @@ class _Span:
 
 
 class DeviceBuffer:
-    def __init__(self, nbytes: int, device, spread: bool = True):
+    def __init__(self, nbytes: int, device, spread: bool = True, max_filler_bytes: int = None):
+        """`max_filler_bytes` bounds the memory the placement may create and release again on its way to
+        the second half of HBM (None = the library's default, 96 GiB; < 0 = all free memory but 2 GiB)."""
         self.device = torch.device(device)
         if self.device.type != "cuda":
             raise RuntimeError("DeviceBuffer needs a GPU (device must be cuda)")
@@ -32,13 +34,18 @@ class DeviceBuffer:
         self.nbytes = int(nbytes)
         p = C.c_void_p()
         torch.cuda.synchronize(self.device)
-        _lib.check(_lib.load().bikv_device_alloc(idx, self.nbytes, _lib.PLACE_SPREAD if spread else _lib.PLACE_SEQUENTIAL,
-                                                 C.byref(p)))
+        place = _lib.PLACE_SPREAD if spread else _lib.PLACE_SEQUENTIAL
+        if max_filler_bytes is None:
+            _lib.check(_lib.load().bikv_device_alloc(idx, self.nbytes, place, C.byref(p)))
+        else:
+            _lib.check(_lib.load().bikv_device_alloc_bounded(idx, self.nbytes, place, int(max_filler_bytes), C.byref(p)))
         self._ptr = p.value
         info = _lib.AllocInfo()
         _lib.check(_lib.load().bikv_device_alloc_info(p, C.byref(info)))
         self.info = {"bytes": info.bytes, "chunk_bytes": info.chunk_bytes, "n_chunks": info.n_chunks,
-                     "n_other_half": info.n_other_half, "n_fillers": info.n_fillers}
+                     "n_other_half": info.n_other_half, "n_fillers": info.n_fillers, "n_reprobed": info.n_reprobed,
+                     "seconds": round(info.seconds, 3), "pair_ms_same": round(info.pair_ms_same, 4),
+                     "pair_ms_other": round(info.pair_ms_other, 4)}
 
     @property
     def tensor(self) -> torch.Tensor:
@@ -60,7 +67,7 @@ class DeviceBuffer:
             pass
 
 
-def device_empty(nbytes: int, device, spread: bool = True) -> torch.Tensor:
+def device_empty(nbytes: int, device, spread: bool = True, max_filler_bytes: int = None) -> torch.Tensor:
     """A uint8 device tensor of `nbytes` whose memory came from bikv_device_alloc; it is released when the
     last tensor that views it is gone and the collector has run."""
-    return DeviceBuffer(nbytes, device, spread).tensor
+    return DeviceBuffer(nbytes, device, spread, max_filler_bytes).tensor

@@ -90,8 +90,10 @@ class NHDPool:
         return both[0], both[1]
 
     def _call(self, fn, tm: torch.Tensor, block_ids: torch.Tensor, tm_pages: Optional[torch.Tensor]):
-        if not tm.is_cuda or not tm.is_contiguous():
-            raise RuntimeError("token-major buffer must be a contiguous CUDA tensor")
+        if not tm.is_contiguous() or not (tm.is_cuda or tm.is_pinned()):
+            # pinned host memory is mapped into the device's address space: the kernel reads / writes it over
+            # the host link, which is how a transport's host region is filled or drained without a hop
+            raise RuntimeError("token-major buffer must be a contiguous CUDA tensor or pinned host memory")
         if tm.element_size() != self._layers[0].element_size():
             raise RuntimeError("token-major buffer and pool differ in element size")
         if tm_pages is None:

@@ -22,9 +22,16 @@
 #include "pagecopy_internal.h"
 
 #include <algorithm>
+#include <cerrno>
+#include <chrono>
+#include <cstdio>
 #include <map>
 #include <mutex>
 #include <vector>
+#include <fcntl.h>
+#include <sys/file.h>
+#include <sys/stat.h>
+#include <unistd.h>
 
 using namespace bikv;
 
@@ -56,9 +63,13 @@ struct Allocation {
   std::vector<hipMemGenericAllocationHandle_t> handles;   // in mapping order
   int n_other = 0;                                         // chunks classified "other half"
   int n_fillers = 0;                                       // chunks created and released again
+  int n_reprobed = 0;                                      // chunks whose first probe was too close to call
+  double seconds = 0;                                      // wall time of the allocation
+  float pair_ms_same = 0, pair_ms_other = 0;               // slowest / fastest pair probe seen
 };
 
-std::mutex g_mu;
+std::mutex g_mu;                 // guards g_allocs
+std::mutex g_alloc_mu;           // one placement at a time per process
 std::map<void*, Allocation> g_allocs;
 
 size_t pow2_floor(size_t x) {
@@ -67,12 +78,50 @@ size_t pow2_floor(size_t x) {
   return p;
 }
 
+// One placement at a time per GPU across PROCESSES too: Bi-KV runs a cache process and a worker process
+// on each GPU, and two placements at once would disturb each other's probe timings and compete for the
+// filler chunks. An advisory lock on a file named after the GPU's PCI address; the kernel drops it when
+// the process ends, whatever way it ends. Best effort: if the file cannot be opened the placement runs
+// unlocked.
+class DeviceFileLock {
+ public:
+  explicit DeviceFileLock(int device) {
+    char bus[64] = "";
+    if (hipDeviceGetPCIBusId(bus, sizeof(bus), device) != hipSuccess) {
+      (void)hipGetLastError();
+      snprintf(bus, sizeof(bus), "index%d", device);
+    }
+    for (char* c = bus; *c; ++c)
+      if (*c == ':' || *c == '.' || *c == '/') *c = '_';
+    char path[128];
+    snprintf(path, sizeof(path), "/dev/shm/bikv_device_alloc_%s.lock", bus);
+    fd_ = open(path, O_CREAT | O_RDWR, 0666);
+    if (fd_ >= 0) {
+      (void)fchmod(fd_, 0666);
+      int rc;
+      do { rc = flock(fd_, LOCK_EX); } while (rc == -1 && errno == EINTR);
+    }
+  }
+  ~DeviceFileLock() {
+    if (fd_ >= 0) {
+      (void)flock(fd_, LOCK_UN);
+      close(fd_);
+    }
+  }
+  DeviceFileLock(const DeviceFileLock&) = delete;
+  DeviceFileLock& operator=(const DeviceFileLock&) = delete;
+
+ private:
+  int fd_ = -1;
+};
+
 struct Prober {
   hipStream_t stream = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr;
   char* src = nullptr;
   size_t src_bytes = size_t(1) << 30;   // far beyond the caches: the probe's reads come from HBM like a scatter's
   void* window = nullptr;      // two chunks of virtual space: [0] the reference chunk, [1] the candidate
+  bool mapped[2] = {false, false};
   size_t chunk = 0;
   hipMemAccessDesc acc;
 
@@ -89,28 +138,43 @@ struct Prober {
     BIKV_HIP(hipMemAddressReserve(&window, 2 * chunk, 0, nullptr, 0));
     return BIKV_OK;
   }
+  // Whatever is still mapped in the window is unmapped first: releasing the address range, or a handle,
+  // with a live mapping leaks it.
   void destroy() {
+    if (stream) (void)hipStreamSynchronize(stream);
+    for (int slot = 0; slot < 2; ++slot)
+      if (window && mapped[slot]) {
+        (void)hipMemUnmap(static_cast<char*>(window) + (size_t)slot * chunk, chunk);
+        mapped[slot] = false;
+      }
     if (window) (void)hipMemAddressFree(window, 2 * chunk);
     if (src) (void)hipFree(src);
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
     if (stream) (void)hipStreamDestroy(stream);
+    window = nullptr;
+    src = nullptr;
+    e0 = e1 = nullptr;
+    stream = nullptr;
   }
   int map(int slot, hipMemGenericAllocationHandle_t h) {
     char* at = static_cast<char*>(window) + (size_t)slot * chunk;
     BIKV_HIP(hipMemMap(at, chunk, 0, h, 0));
+    mapped[slot] = true;
     BIKV_HIP(hipMemSetAccess(at, chunk, &acc, 1));
     return BIKV_OK;
   }
   int unmap(int slot) {
+    if (!mapped[slot]) return BIKV_OK;
     BIKV_HIP(hipStreamSynchronize(stream));
     BIKV_HIP(hipMemUnmap(static_cast<char*>(window) + (size_t)slot * chunk, chunk));
+    mapped[slot] = false;
     return BIKV_OK;
   }
-  // milliseconds of one probe launch writing ~1 GiB into slot 0 and slot `other` (0 = the reference alone)
-  int time(int other, float* ms) {
+  // milliseconds of one probe launch scattering ~1 GiB into the pair (slot 0, slot 1)
+  int time_pair(float* ms) {
     char* a = static_cast<char*>(window);
-    char* b = a + (size_t)other * chunk;
+    char* b = a + chunk;
     const uint32_t tiles = (uint32_t)(chunk / 16384);
     const uint32_t grid = 1u << 20;                       // 1 Mi workgroups x 1 KiB
     for (int i = 0; i < 2; ++i)
@@ -132,15 +196,26 @@ void release_all(std::vector<hipMemGenericAllocationHandle_t>& v) {
   v.clear();
 }
 
+// A pair that straddles the halves scatters ~19 % faster than a pair inside one half. Every candidate is
+// probed as a PAIR with the first chunk (equal footprint for every probe), and judged against the slowest
+// pair seen so far — pairs inside the first chunk's half. A time inside the band between the two groups is
+// not trusted: the chunk is probed again (twice more at most) and the median decides.
+constexpr float kOtherBelow = 0.92f;     // other half: pair time below 0.92 x the same-half pair time
+constexpr float kBandLo = 0.88f, kBandHi = 0.96f;
+
 }  // namespace
 
-extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, void** out) {
+extern "C" int bikv_device_alloc_bounded(int device, int64_t bytes, int32_t placement, int64_t max_filler_bytes,
+                                         void** out) {
   if (!out) return fail(BIKV_EINVAL, "null out");
   *out = nullptr;
   if (bytes <= 0) return fail(BIKV_EINVAL, "bytes must be positive");
   if (placement != BIKV_PLACE_SPREAD && placement != BIKV_PLACE_SEQUENTIAL)
     return fail(BIKV_EINVAL, "unknown placement %d", placement);
   BIKV_DEVICE(device);
+  const auto t_begin = std::chrono::steady_clock::now();
+  std::lock_guard<std::mutex> process_lock(g_alloc_mu);
+  DeviceFileLock gpu_lock(device);
   hipMemAllocationProp prop = hipMemAllocationProp();
   prop.type = hipMemAllocationTypePinned;
   prop.location.type = hipMemLocationTypeDevice;
@@ -154,6 +229,7 @@ extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, v
   const size_t n = ((size_t)bytes + chunk - 1) / chunk;
   const size_t want_other = placement == BIKV_PLACE_SPREAD ? n / 2 : 0;
   const size_t want_same = n - want_other;
+  const size_t max_fillers = max_filler_bytes < 0 ? ~size_t(0) : (size_t)max_filler_bytes / chunk;
 
   const size_t reserve = size_t(2) << 30;     // never take the last 2 GiB of the device
   {
@@ -164,6 +240,7 @@ extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, v
                   (size_t)bytes, n, chunk, free_now);
   }
   std::vector<hipMemGenericAllocationHandle_t> same, other, fillers;
+  std::vector<float> same_ms;      // pair time of every chunk in `same` (0 for the reference chunk)
   Prober pr;
   int rc = BIKV_OK;
   auto cleanup = [&]() {
@@ -172,16 +249,19 @@ extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, v
     release_all(other);
     release_all(fillers);
   };
-  float t_ref = 0;
   if (placement == BIKV_PLACE_SPREAD && n >= 2) {
     rc = pr.init(device, chunk);
     if (rc) { cleanup(); return rc; }
   }
   // Create chunks until both kinds are complete. Chunks beyond the wanted number of a kind are fillers:
-  // they only push the driver's allocator on towards the other half and are released at the end. A
-  // failed creation (memory exhausted) ends the search with whatever balance was reached.
+  // they only push the driver's allocator on towards the other half and are released at the end. The
+  // search ends with whatever balance was reached when a creation fails (memory exhausted) or the filler
+  // budget is spent.
+  float ref_ms = 0, fastest_ms = 0;
+  int n_reprobed = 0;
   size_t free_b = 0, total_b = 0;
   while (same.size() < want_same || other.size() < want_other) {
+    if (fillers.size() >= max_fillers && (same.size() >= want_same || other.size() >= want_other)) break;
     if (hipMemGetInfo(&free_b, &total_b) != hipSuccess || free_b < chunk + reserve) break;
     hipMemGenericAllocationHandle_t h;
     if (hipMemCreate(&h, chunk, &prop, 0) != hipSuccess) {
@@ -189,44 +269,89 @@ extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, v
       break;
     }
     bool is_other = false;
+    float t_pair = 0;
     if (pr.window) {
       if (same.empty()) {
-        // the first chunk is the reference: time it alone
-        rc = pr.map(0, h);
-        if (!rc) rc = pr.time(0, &t_ref);
+        rc = pr.map(0, h);           // the first chunk is the reference every candidate is paired with
       } else {
-        float t = 0;
         rc = pr.map(1, h);
-        if (!rc) rc = pr.time(1, &t);
-        if (!rc) rc = pr.unmap(1);
-        is_other = !rc && t < 0.92f * t_ref;
+        float t = 0;
+        if (!rc) rc = pr.time_pair(&t);
+        if (!rc && ref_ms > 0 && t > kBandLo * ref_ms && t < kBandHi * ref_ms) {
+          // too close to call: two more probes, the median of the three decides
+          float t2 = 0, t3 = 0;
+          rc = pr.time_pair(&t2);
+          if (!rc) rc = pr.time_pair(&t3);
+          if (!rc) {
+            float v[3] = {t, t2, t3};
+            std::sort(v, v + 3);
+            t = v[1];
+            ++n_reprobed;
+          }
+        }
+        // unmapped whether or not the probes worked: the handle is about to be released or kept for the
+        // final mapping, and neither may happen while the window still maps it
+        const int rc_unmap = pr.unmap(1);
+        if (!rc) rc = rc_unmap;
+        if (!rc) {
+          if (t > ref_ms) ref_ms = t;            // pairs inside one half are the slow ones
+          is_other = t < kOtherBelow * ref_ms;
+          t_pair = t;
+          if (is_other && (fastest_ms == 0 || t < fastest_ms)) fastest_ms = t;
+        }
       }
       if (rc) {
+        (void)pr.unmap(0 + (same.empty() ? 0 : 1));
         (void)hipMemRelease(h);
         break;
       }
     }
     if (is_other) {
       if (other.size() < want_other) other.push_back(h); else fillers.push_back(h);
+    } else if (same.size() < want_same) {
+      same.push_back(h);
+      same_ms.push_back(t_pair);
     } else {
-      if (same.size() < want_same) same.push_back(h); else fillers.push_back(h);
+      fillers.push_back(h);
     }
   }
-  if (pr.window && !same.empty()) (void)pr.unmap(0);
+  if (pr.window) (void)pr.unmap(0);
   if (rc) { cleanup(); return rc; }
-  // what one kind lacks the other makes up (from the fillers), so that the allocation is complete
+  // The reference time only grows during the search: a chunk judged "same" against an early, too small
+  // reference (possible only while no same-half pair had been seen yet) is judged again against the final one.
+  for (size_t i = 1; i < same.size() && i < same_ms.size();) {
+    if (same_ms[i] > 0 && same_ms[i] < kOtherBelow * ref_ms) {
+      other.push_back(same[i]);
+      if (fastest_ms == 0 || same_ms[i] < fastest_ms) fastest_ms = same_ms[i];
+      same.erase(same.begin() + (long)i);
+      same_ms.erase(same_ms.begin() + (long)i);
+    } else {
+      ++i;
+    }
+  }
+  // what one kind lacks the other makes up (from the fillers, else freshly created), so that the
+  // allocation is complete
   while (same.size() + other.size() < n && !fillers.empty()) {
     same.push_back(fillers.back());
     fillers.pop_back();
   }
+  while (same.size() + other.size() < n) {
+    hipMemGenericAllocationHandle_t h;
+    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess || free_b < chunk + reserve ||
+        hipMemCreate(&h, chunk, &prop, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      break;
+    }
+    same.push_back(h);
+  }
   if (same.size() + other.size() < n) {
+    const size_t got = same.size() + other.size();
     cleanup();
-    return fail(BIKV_EHIP, "out of device memory: %zu of %zu chunks of %zu bytes could be created", same.size() + other.size(), n, chunk);
+    return fail(BIKV_EHIP, "out of device memory: %zu of %zu chunks of %zu bytes could be created", got, n, chunk);
   }
   const int n_fillers = (int)fillers.size();
   release_all(fillers);
   pr.destroy();
-  pr = Prober();
 
   // map alternately: position k takes an "other" chunk whenever that keeps the two kinds evenly mixed
   Allocation al;
@@ -235,6 +360,9 @@ extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, v
   al.chunk = chunk;
   al.n_other = (int)other.size();
   al.n_fillers = n_fillers;
+  al.n_reprobed = n_reprobed;
+  al.pair_ms_same = ref_ms;
+  al.pair_ms_other = fastest_ms;
   hipError_t e = hipMemAddressReserve(&al.va, al.bytes, 0, nullptr, 0);
   if (e != hipSuccess) { cleanup(); return fail_hip(e, "hipMemAddressReserve"); }
   const std::vector<bool> order = interleave_order(same.size(), other.size());
@@ -259,12 +387,17 @@ extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, v
   }
   same.clear();
   other.clear();
+  al.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t_begin).count();
   {
     std::lock_guard<std::mutex> lk(g_mu);
     g_allocs[al.va] = al;
   }
   *out = al.va;
   return BIKV_OK;
+}
+
+extern "C" int bikv_device_alloc(int device, int64_t bytes, int32_t placement, void** out) {
+  return bikv_device_alloc_bounded(device, bytes, placement, BIKV_DEFAULT_MAX_FILLER_BYTES, out);
 }
 
 extern "C" int bikv_device_free(void* p) {
@@ -297,6 +430,9 @@ extern "C" int bikv_device_alloc_info(const void* p, bikv_alloc_info* info) {
   info->n_chunks = (int32_t)it->second.handles.size();
   info->n_other_half = it->second.n_other;
   info->n_fillers = it->second.n_fillers;
-  info->reserved = 0;
+  info->n_reprobed = it->second.n_reprobed;
+  info->seconds = it->second.seconds;
+  info->pair_ms_same = it->second.pair_ms_same;
+  info->pair_ms_other = it->second.pair_ms_other;
   return BIKV_OK;
 }

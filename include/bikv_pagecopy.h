@@ -350,23 +350,39 @@ int bikv_h2d_copy(int device, void* dev_dst, const void* host_src, int64_t bytes
  * half (any pool below ~100 GB on an empty GPU) scatters 15-18 % slower than it could, and how a large
  * hipMalloc straddles the boundary changes from one allocation to the next.
  * bikv_device_alloc(BIKV_PLACE_SPREAD) builds the allocation from physical chunks (256 MiB - 1 GiB,
- * hipMemCreate), tells the halves apart with a short timed scatter into pairs of chunks, keeps equal
+ * hipMemCreate), tells the halves apart with a short timed scatter into pairs of chunks (a pair that
+ * straddles the halves runs ~19 % faster; a time too close to call is measured twice more), keeps equal
  * numbers of both kinds and maps them alternately into one virtual range, so that every window of the
  * pool spreads its writes over both halves. To reach the second half it may transiently create (and
- * release again) filler chunks up to the free memory of the device less 2 GiB: call it at start-up,
- * before other large allocations. BIKV_PLACE_SEQUENTIAL maps the chunks in creation order, unprobed.
+ * release again) filler chunks: at most `max_filler_bytes` of them (bikv_device_alloc_bounded; < 0 = as
+ * many as the free memory of the device less 2 GiB allows; bikv_device_alloc uses
+ * BIKV_DEFAULT_MAX_FILLER_BYTES). When the budget does not reach the other half the allocation is
+ * completed with what there is and bikv_device_alloc_info shows the imbalance. Two costs of fillers to
+ * know: they are device memory other tenants of the GPU cannot have for the second or two the placement
+ * takes, and the driver scrubs released memory in the background at ~15 GB/s, during which every
+ * hipMemcpyAsync between host and device runs at about half its rate — so place pools at start-up, before
+ * other large allocations and before traffic starts. Placements are serialised: within a process by a lock,
+ * between the processes that share a GPU (Bi-KV runs a cache process and a worker process per GPU) by an
+ * advisory file lock named after the GPU's PCI address, so that neither disturbs the other's probe timings
+ * nor takes the chunks the other is counting on.
+ * BIKV_PLACE_SEQUENTIAL maps the chunks in creation order, unprobed.
  * The memory behaves like hipMalloc'd memory for kernels and copies; it cannot be exported over HIP IPC.
  * Sizes are rounded up to whole chunks. ------------------------------------------------------------ */
 enum { BIKV_PLACE_SPREAD = 0, BIKV_PLACE_SEQUENTIAL = 1 };
+#define BIKV_DEFAULT_MAX_FILLER_BYTES ((int64_t)96 << 30)
 typedef struct bikv_alloc_info {
   int64_t bytes;          /* mapped size (a whole number of chunks) */
   int64_t chunk_bytes;
   int32_t n_chunks;
   int32_t n_other_half;   /* chunks the probe placed in the other half than the first chunk */
   int32_t n_fillers;      /* chunks created on the way and released again */
-  int32_t reserved;
+  int32_t n_reprobed;     /* chunks whose first probe fell between the two groups and was repeated */
+  double seconds;         /* wall time the placement took, waiting for the locks included */
+  float pair_ms_same;     /* slowest pair probe seen (a pair inside the first chunk's half); 0 = nothing probed */
+  float pair_ms_other;    /* fastest pair probe classified "other half"; 0 = none seen */
 } bikv_alloc_info;
 int bikv_device_alloc(int device, int64_t bytes, int32_t placement, void** out);
+int bikv_device_alloc_bounded(int device, int64_t bytes, int32_t placement, int64_t max_filler_bytes, void** out);
 int bikv_device_free(void* p);
 int bikv_device_alloc_info(const void* p, bikv_alloc_info* info);
 

@@ -518,3 +518,64 @@ def test_packed_transfer_against_committed_digest(ipc, cuda):
     assert total == e["total_tokens"] and tuple(got.shape) == (total,) + dims
     digest = hashlib.sha256(got.cpu().contiguous().view(torch.int16).numpy().tobytes()).hexdigest()
     assert digest == e["received_sha256"]
+
+
+def test_three_producer_threads_share_the_ring_without_losing_a_transfer(ipc, cuda):
+    """The reference's callers are gRPC thread pools over process-global ring state (ipc_service.cpp:9-17).
+    Here three threads call producer_send / producer_copy_pages at once, with back-pressure on, while a
+    fourth receives: every transfer arrives exactly once, whole, and carries its own sender's bytes — no
+    window handed out twice, no publication lost."""
+    import threading
+    print("[case] three producer threads, one ring", flush=True)
+    name = f"/bikv_test_threads_{os.getpid()}"
+    n_threads, per_thread, n = 3, 40, 1 << 14
+    ipc.consumer_init(0, name, 5 * n * 2 // 2)          # 2.5 tensors of n fp16: the ring wraps all the time
+    ipc.producer_init(0, name)
+    errors, seen = [], []
+
+    def consume():
+        try:
+            for _ in range(n_threads * per_thread):
+                t = ipc.consumer_receive(timeout_ms=30000)
+                vals = t.view(torch.int16).cpu()
+                tag = int(vals[0].item())
+                if not bool((vals == tag).all()) or t.numel() != n:
+                    errors.append(f"mixed or short transfer (tag {tag})")
+                seen.append(tag)
+                ipc.consumer_release()
+        except Exception as e:  # noqa: BLE001
+            errors.append(f"consumer: {e}")
+
+    def produce(tid):
+        try:
+            torch.cuda.set_device(cuda)
+            stream = torch.cuda.Stream(device=cuda)
+            d = ipc.TensorDims()
+            d.head_size, d.num_kv_heads, d.num_layers, d.kv_pair = 64, 2, 1, 2
+            page_elems = 16 * 64 * 2 * 1 * 2
+            runs = n // page_elems
+            offs = torch.arange(runs, dtype=torch.int64, device=cuda) * page_elems
+            with torch.cuda.stream(stream):
+                for k in range(per_thread):
+                    tag = tid * per_thread + k + 1
+                    src = torch.full((n,), tag, dtype=torch.int16, device=cuda).view(torch.float16)
+                    if k % 2:
+                        ipc.producer_send(src)
+                    else:
+                        ipc.producer_copy_pages(src, offs, offs, 16, d)
+        except Exception as e:  # noqa: BLE001
+            errors.append(f"producer {tid}: {e}")
+
+    try:
+        ipc.producer_set_backpressure(True, timeout_ms=30000)
+        threads = [threading.Thread(target=consume)] + [threading.Thread(target=produce, args=(t,)) for t in range(n_threads)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(120)
+        assert not any(t.is_alive() for t in threads), "a thread is stuck"
+        assert not errors, errors
+        assert sorted(seen) == list(range(1, n_threads * per_thread + 1))
+    finally:
+        ipc.producer_cleanup()
+        ipc.consumer_cleanup()

@@ -226,3 +226,57 @@ def test_two_process_layered_transfer(oracle, cuda):
         image = oracle.gather_layered_c(src_pool, src, "layer_major")
         oracle.scatter_layered_c(want, dst, image, "layer_major")
     assert results["receiver"][1] == want.tobytes()
+
+
+def _placer(tag, start, out):
+    """One tenant of the GPU: places an 8 GB pool through bikv_device_alloc, writes a page of it, gathers it."""
+    try:
+        _paths()
+        import torch
+        import bikv_pagecopy as bk
+        torch.cuda.init()
+        if not start.wait(120):
+            raise RuntimeError("start signal did not come")
+        t0 = time.time()
+        buf = bk.DeviceBuffer(8 << 30, "cuda:0", spread=True, max_filler_bytes=16 << 30)
+        wall = time.time() - t0
+        n_planes, tile = 4, 16384
+        n_pages = (8 << 30) // (n_planes * tile)
+        pool_t = buf.tensor.view(n_planes, n_pages, tile)
+        ids = np.array([0, n_pages // 2, n_pages - 1], dtype=np.int64)
+        pool_t[:, torch.from_numpy(ids).cuda()] = tag
+        pool = bk.PagedKVPool.from_stacked(pool_t, plane_dims=1)
+        st, _ = pool.gather(pool.make_batch([ids]))
+        pool.check()
+        ok = bool((st == tag).all().item())
+        pool.close()
+        info = dict(buf.info)
+        del pool_t, st
+        buf.free()
+        out.put((tag, "ok" if ok else "gathered bytes differ", info, wall))
+    except Exception as e:  # noqa: BLE001
+        out.put((tag, f"{type(e).__name__}: {e}", None, 0.0))
+
+
+def test_two_processes_place_their_pools_on_one_gpu_at_the_same_time(cuda):
+    """Bi-KV runs a cache process and a worker process per GPU. Two processes call bikv_device_alloc for 8 GB
+    each at the same moment: the placements are serialised by the per-GPU file lock, both complete, both
+    report their bookkeeping, and both pools move pages correctly."""
+    print("[case] two processes place pools at once", flush=True)
+    ctx = mp.get_context("spawn")
+    start, out = ctx.Event(), ctx.Queue()
+    procs = [ctx.Process(target=_placer, args=(tag, start, out)) for tag in (11, 22)]
+    for p in procs:
+        p.start()
+    time.sleep(1.0)
+    start.set()
+    results = [out.get(timeout=300) for _ in procs]
+    for p in procs:
+        p.join(60)
+        assert p.exitcode == 0
+    for tag, status, info, wall in results:
+        assert status == "ok", (tag, status)
+        assert info["bytes"] >= 8 << 30 and info["n_chunks"] * info["chunk_bytes"] == info["bytes"]
+        assert info["n_fillers"] * info["chunk_bytes"] <= 16 << 30
+        assert info["seconds"] > 0 and wall >= info["seconds"] * 0.5
+    print("   placements:", [(r[0], r[2]) for r in results], flush=True)

@@ -779,9 +779,11 @@ def test_device_alloc_builds_a_pool_out_of_chunks_from_both_halves(bk, oracle, c
         info = buf.info
         assert info["bytes"] >= nbytes and info["bytes"] % info["chunk_bytes"] == 0
         assert info["n_chunks"] * info["chunk_bytes"] == info["bytes"] and info["chunk_bytes"] >= 256 << 20
-        assert 0 <= info["n_other_half"] <= info["n_chunks"] // 2
+        assert 0 <= info["n_other_half"] <= info["n_chunks"] and info["seconds"] > 0
         if not spread:
-            assert info["n_other_half"] == 0 and info["n_fillers"] == 0
+            assert info["n_other_half"] == 0 and info["n_fillers"] == 0 and info["pair_ms_same"] == 0
+        else:
+            assert info["pair_ms_same"] > 0       # every candidate was probed as a pair with the first chunk
         t = buf.tensor
         assert t.numel() == nbytes and t.dtype == torch.uint8 and t.device == cuda
         rng = np.random.default_rng(401)
@@ -818,6 +820,12 @@ def test_device_alloc_builds_a_pool_out_of_chunks_from_both_halves(bk, oracle, c
         buf.free()
         with pytest.raises(RuntimeError, match="freed"):
             buf.tensor
+    # a filler budget of zero: the placement keeps what the driver hands out first and creates nothing more
+    buf = bk.DeviceBuffer(nbytes, cuda, spread=True, max_filler_bytes=0)
+    assert buf.info["n_fillers"] == 0 and buf.info["bytes"] >= nbytes
+    buf.tensor[:4096].fill_(7)
+    assert int(buf.tensor[:4096].sum().item()) == 7 * 4096
+    buf.free()
     assert lib.bikv_device_free(C.c_void_p(12345)) == _lib.EINVAL
     p = C.c_void_p()
     assert lib.bikv_device_alloc(0, 0, 0, C.byref(p)) == _lib.EINVAL

@@ -83,3 +83,51 @@ def test_noalloc_gather_limits_and_errors(lib, cuda):
     # an empty batch is a no-op
     eb = small.make_batch([[]])
     assert _call_noalloc(lib, _lib, small, eb, host) == _lib.OK
+
+
+def test_noalloc_gather_allocates_nothing_and_replays_from_a_hip_graph(lib, oracle, cuda):
+    """The two claims of the entry point's contract. (1) Device memory in use is the same before and after
+    a call. (2) A call made while a stream is capturing records kernel nodes only, and the captured graph
+    can be replayed: three replays, with the pool changed by eager work (and the host image cleared) between
+    them, each checked against the oracle for the pool as it is at that moment."""
+    import bikv_pagecopy as bk
+    from bikv_pagecopy import _lib
+    print("[case] allocation-free gather to host: memory use and graph replay", flush=True)
+    assert lib.bikv_init(0) == _lib.OK
+    rng = np.random.default_rng(73)
+    n_planes, n_pages, tile = 4, 30, 1280 * 1024
+    pool_h = rng.integers(0, 256, size=(n_planes, n_pages, tile), dtype=np.uint8)
+    pool_d = torch.from_numpy(pool_h).to(cuda)
+    pool = bk.PagedKVPool.from_stacked(pool_d, plane_dims=1)
+    reqs = [rng.permutation(n_pages)[:9], rng.permutation(n_pages)[:4]]
+    batch = pool.make_batch(reqs)
+    host = bk.pinned_empty(batch.n_slots * tile)
+    torch.cuda.synchronize(cuda)
+    # (1) no allocation: free device memory as the driver reports it, before and after an eager call
+    free_before = torch.cuda.mem_get_info(cuda)[0]
+    stream = C.c_void_p(torch.cuda.current_stream(cuda).cuda_stream)
+    assert _call_noalloc(lib, _lib, pool, batch, host, None, stream) == _lib.OK, lib.bikv_last_error()
+    pool.check()
+    assert torch.cuda.mem_get_info(cuda)[0] == free_before
+    assert host.numpy().tobytes() == oracle.gather_layered_c(pool_h, reqs).tobytes()
+    # (2) capture once, replay three times
+    side = torch.cuda.Stream(device=cuda)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            s = C.c_void_p(torch.cuda.current_stream(cuda).cuda_stream)
+            assert _call_noalloc(lib, _lib, pool, batch, host, None, s) == _lib.OK, lib.bikv_last_error()
+    for rep in range(3):
+        # eager work between replays: new bytes in some of the gathered pages, host image cleared
+        page = int(reqs[0][rep])
+        fresh = rng.integers(0, 256, size=(n_planes, tile), dtype=np.uint8)
+        pool_h[:, page] = fresh
+        pool_d[:, page] = torch.from_numpy(fresh).to(cuda)
+        host.fill_(0xA5)
+        torch.cuda.synchronize(cuda)
+        graph.replay()
+        torch.cuda.synchronize(cuda)
+        assert host.numpy().tobytes() == oracle.gather_layered_c(pool_h, reqs).tobytes(), rep
+    pool.check()
+    del graph
+    pool.close()
