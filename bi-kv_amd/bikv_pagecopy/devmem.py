@@ -44,7 +44,7 @@ class DeviceBuffer:
         _lib.check(_lib.load().bikv_device_alloc_info(p, C.byref(info)))
         self.info = {"bytes": info.bytes, "chunk_bytes": info.chunk_bytes, "n_chunks": info.n_chunks,
                      "n_other_half": info.n_other_half, "n_fillers": info.n_fillers, "n_reprobed": info.n_reprobed,
-                     "seconds": round(info.seconds, 3), "pair_ms_same": round(info.pair_ms_same, 4),
+                     "seconds": round(info.seconds, 6), "pair_ms_same": round(info.pair_ms_same, 4),
                      "pair_ms_other": round(info.pair_ms_other, 4)}
 
     @property

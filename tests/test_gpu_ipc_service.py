@@ -536,8 +536,8 @@ def test_three_producer_threads_share_the_ring_without_losing_a_transfer(ipc, cu
     def consume():
         try:
             for _ in range(n_threads * per_thread):
-                t = ipc.consumer_receive(timeout_ms=30000)
-                vals = t.view(torch.int16).cpu()
+                t = ipc.consumer_receive(timeout_ms=15000)
+                vals = t.reshape(-1).view(torch.int16).cpu()
                 tag = int(vals[0].item())
                 if not bool((vals == tag).all()) or t.numel() != n:
                     errors.append(f"mixed or short transfer (tag {tag})")
@@ -567,7 +567,7 @@ def test_three_producer_threads_share_the_ring_without_losing_a_transfer(ipc, cu
             errors.append(f"producer {tid}: {e}")
 
     try:
-        ipc.producer_set_backpressure(True, timeout_ms=30000)
+        ipc.producer_set_backpressure(True, timeout_ms=15000)
         threads = [threading.Thread(target=consume)] + [threading.Thread(target=produce, args=(t,)) for t in range(n_threads)]
         for t in threads:
             t.start()
