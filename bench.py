@@ -113,6 +113,8 @@ def parse_args():
     ap.add_argument("--wave-block", dest="wave_block", type=int, default=None)
     ap.add_argument("--order", type=int, default=None)
     ap.add_argument("--log2-chunk", dest="log2_chunk", type=int, default=None)
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="any launch knob of bikv_set_tuning, e.g. --tune transpose_kvswap=1 (repeatable)")
     ap.add_argument("--staging-cap-gb", dest="staging_cap_gb", type=float, default=32.0,
                     help="largest staging buffer of one launch; bigger batches take several launches")
     ap.add_argument("--chunk-mib", type=int, default=0, help="staging: measure only this chunk size (0 = the sweep)")
@@ -540,17 +542,16 @@ def link_yardstick(bk, dev, host, dev_buf, reps=3):
 def run_staging(args, bk, workloads, dev, kept=None):
     """Llama-3-8B shape: every request of the log-normal stream gathered into pinned host memory, and
     scattered back from it, through the staging pipeline. All requests of a pass are enqueued back to back
-    (one wait at the end). The record has three parts, in the order they are measured:
+    (one wait at the end). The record has two parts, in the order they are measured:
 
     first_pass  the first pass of a fresh stager in every mode, taken the moment the pool is ready — no
-                warm-up, whatever state the process is in (this benchmark has just freed hundreds of GB of
-                device memory, which the driver scrubs in the background at ~15 GB/s; every hipMemcpyAsync
-                between host and device runs at about half rate until that is done);
-    cells       once a plain hipMemcpyAsync is back at its full rate (the wait is reported), chunk sizes,
-                lane counts and modes, three timed passes each after two untimed ones, each next to a plain
-                hipMemcpyAsync of one 1 GiB pinned buffer timed immediately before it;
-    during_scrub  the same modes measured while the driver is scrubbing 32 GiB that was freed a moment
-                before: which of them depend on the copy engines and which do not."""
+                warm-up of any kind, with the mean rate of plain 64 MiB hipMemcpyAsync calls right before and
+                after it;
+    cells       chunk sizes, lane counts and modes, three timed passes each after two untimed ones, each next
+                to a plain hipMemcpyAsync of one 1 GiB pinned buffer timed immediately before it. Before the
+                first cell the run waits until plain copies hold their full rate (normally no wait at all;
+                the wait is reported): this benchmark has just released hundreds of GB of device memory, and
+                for as long as the driver scrubs released memory every hipMemcpyAsync can run at half rate."""
     import numpy as np
     import torch
 
@@ -603,16 +604,18 @@ def run_staging(args, bk, workloads, dev, kept=None):
         return int(sizes[:n_req].sum()) / (time.perf_counter() - t0) / 1e9
 
     def small_copy_rate(direction, seconds=0.15):
-        """Rate of back-to-back plain hipMemcpyAsync calls of 64 MiB for about `seconds`: the probe that tells
-        whether the copy engines are at full rate."""
-        n, best, t_end = 64 << 20, 0.0, time.perf_counter() + seconds
+        """Mean rate of back-to-back plain hipMemcpyAsync calls of 64 MiB over about `seconds`: the probe that
+        tells whether the copy engines are at full rate."""
+        n, moved, t0 = 64 << 20, 0, time.perf_counter()
+        spent = 0.0
         while True:
             if direction == "d2h":
-                best = max(best, n / bk.measure_d2h(dev, host[:n], dev_buf[:n], 0) / 1e9)
+                spent += bk.measure_d2h(dev, host[:n], dev_buf[:n], 0)
             else:
-                best = max(best, n / bk.measure_h2d(dev, dev_buf[:n], host[:n], 0) / 1e9)
-            if time.perf_counter() >= t_end:
-                return best
+                spent += bk.measure_h2d(dev, dev_buf[:n], host[:n], 0)
+            moved += n
+            if time.perf_counter() - t0 >= seconds:
+                return moved / spent / 1e9
 
     def cell(stager, mode, direction, synchronous=False):
         d2h, h2d = link_yardstick(bk, dev, host[: dev_buf.numel()], dev_buf)
@@ -720,34 +723,6 @@ def run_staging(args, bk, workloads, dev, kept=None):
     stager.close()
     auto = cells[-1]
 
-    # --- 3. the same modes while the driver scrubs device memory that was freed a moment before
-    scrub = None
-    if not args.chunk_mib:
-        scrub_gib = 32
-        free_b = torch.cuda.mem_get_info(dev)[0]
-        if free_b > (scrub_gib + 8) << 30:
-            scrub = {}
-            for direction, probe in (("gather", "d2h"), ("scatter", "h2d")):
-                for mode in MODES:
-                    st = bk.HostStager(dev)
-                    one_pass(st, mode, direction, 2)                     # the stager's streams and buffers exist
-                    x = torch.empty(scrub_gib << 30, dtype=torch.uint8, device=dev)
-                    del x
-                    torch.cuda.empty_cache()                             # hipFree: returns at once, the scrub starts
-                    before = small_copy_rate(probe, 0.05)
-                    r = one_pass(st, mode, direction, n_short)
-                    after = small_copy_rate(probe, 0.05)
-                    st.close()
-                    scrub[f"{direction}_{mode}"] = {"GBps": round(r, 2), "plain_64MiB_copies_before_GBps": round(before, 2),
-                                                    "plain_64MiB_copies_after_GBps": round(after, 2)}
-                    t_w = time.perf_counter()                            # let the scrub finish before the next case
-                    while small_copy_rate(probe, 0.1) < 50.0 and time.perf_counter() - t_w < 20.0:
-                        pass
-            scrub["what"] = (f"one pass of {short_bytes / 1e9:.1f} GB per mode, started right after {scrub_gib} GiB of device memory "
-                             "was allocated and freed (hipFree returns at once; the driver then scrubs the memory in the "
-                             "background for about 2 s, during which plain hipMemcpyAsync runs at ~30 GB/s in both directions)")
-            log(f"staging during_scrub {scrub}")
-
     out = {"workload": f"llama3_8b: {shape.n_pages} pages x {shape.n_planes} planes x {shape.tile_bytes} B, "
                        f"{len(reqs)} requests of {int(sizes.min() // shape.page_bytes)}..{int(sizes.max() // shape.page_bytes)} "
                        f"pages ({total_bytes / 1e9:.2f} GB per pass), enqueued back to back, {passes} timed passes per cell after two untimed ones",
@@ -765,7 +740,7 @@ def run_staging(args, bk, workloads, dev, kept=None):
            "frac_of_best_plain_d2h_seen": round(auto["gather_to_host"]["GBps_median"] / max(yard["d2h"]), 4),
            "scatter_from_host_GBps": auto["scatter_from_host"]["GBps_median"],
            "scatter_frac_of_plain_h2d": auto["scatter_from_host"]["frac_median"],
-           "cells": cells, "per_request_blocking_calls": per_call, "during_scrub": scrub, "bit_exact": True,
+           "cells": cells, "per_request_blocking_calls": per_call, "bit_exact": True,
            "seconds": round(time.perf_counter() - t_part, 1)}
     real = [c for c in cells if "contrast_case" not in c]
     out["min_frac_over_cells"] = {
@@ -773,6 +748,9 @@ def run_staging(args, bk, workloads, dev, kept=None):
         "scatter_from_host": min(c["scatter_from_host"]["frac_min"] for c in real),
         "what": "lowest single pass of any cell, as a fraction of the plain copy timed just before that cell "
                 "(every chunk size, lane count and mode above except the contrast case)"}
+    worst = min(real, key=lambda c: c["gather_to_host"]["frac_min"])
+    out["min_frac_over_cells"]["gather_to_host_worst_cell"] = (f"{worst['mode']} {worst['chunk_MiB']} MiB x {worst['lanes']} lanes x "
+                                                               f"{worst['copies_per_launch']} per launch, passes {worst['gather_to_host']['passes_GBps']}")
     out["median_frac_over_cells"] = {
         "gather_to_host": round(float(np.median([c["gather_to_host"]["frac_median"] for c in real])), 4),
         "scatter_from_host": round(float(np.median([c["scatter_from_host"]["frac_median"] for c in real])), 4)}
@@ -1147,6 +1125,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     knobs = {k: getattr(args, k) for k in ("seg", "unroll", "nontemporal", "wave_block", "order", "log2_chunk") if getattr(args, k) is not None}
+    for kv in args.tune:
+        k, _, v = kv.partition("=")
+        knobs[k.strip()] = int(v)
     if knobs:
         bk.set_tuning(**knobs)
 
@@ -1272,9 +1253,6 @@ def add_summary(out):
             if isinstance(v, dict):
                 sm[f"staging_first_pass_{k}_GBps"] = v["GBps"]
         sm["staging_wait_for_full_rate_copies_s"] = st["wait_for_full_rate_copies"]["seconds"]
-        for k, v in (st.get("during_scrub") or {}).items():
-            if isinstance(v, dict):
-                sm[f"staging_during_scrub_{k}_GBps"] = v["GBps"]
     lc = out.get("layout_change")
     if lc:
         sm["layout_change_value_GBps"] = lc["value"]

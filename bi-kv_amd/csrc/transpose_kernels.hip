@@ -245,6 +245,24 @@ __device__ __forceinline__ void store16(uint64_t p, const u32x4& v, bool sys) {
     __builtin_nontemporal_store(v, (BIKV_GLOBAL u32x4*)p);
 }
 
+// lanes 32-63 of x <-> lanes 0-31 of y, all four dwords. With x = {K of layer A | K of layer B} and
+// y = {V of layer A | V of layer B} (half-waves) this yields {K A | V A} and {K B | V B}, and back: the
+// exchange is its own inverse.
+__device__ __forceinline__ void swap_half_waves(u32x4& x, u32x4& y) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const auto r = __builtin_amdgcn_permlane32_swap(x[i], y[i], false, false);
+    x[i] = r[0];
+    y[i] = r[1];
+  }
+}
+// the 64-bit value lane `src` of this wave holds, as a wave-uniform value
+__device__ __forceinline__ uint64_t from_lane(uint64_t v, int src) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, src);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), src);
+  return ((uint64_t)hi << 32) | lo;
+}
+
 template <int DIR, int ES, int B>
 __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs a) {
   using Unit = typename UnitOf<ES>::T;
@@ -345,22 +363,50 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
     __syncthreads();
     // LDS -> compute rows: 32 bytes of units become one K vector and one V vector
     UWalk o = uwalk_start(tid, dgs, a.m_dgs);                  // (pair, group of d)
-    for (uint32_t base = 0; base < n_cp; base += B) {
-      if (o.outer < Cw) {
-        const uint64_t entry = row_addr[o.outer];
+    if (a.kv_swap) {
+      // K rows and V rows of a (token, layer) are the two halves of ONE contiguous KiB, and a half-wave
+      // covers exactly the K rows of a layer: lanes 0-31 hold {K, V} of layer A, lanes 32-63 of layer B.
+      // Exchanging half-waves turns {K A | K B}, {V A | V B} into {K A | V A}, {K B | V B}: each store
+      // instruction then writes one whole KiB instead of two half-KiB pieces in two layer tensors.
+      const uint32_t lane = tid & 63u;
+      for (uint32_t base = 0; base < n_cp; base += B) {
+        const bool valid = o.outer < Cw;
+        const uint64_t entry = row_addr[valid ? o.outer : 0];
         const uint32_t cp = (uint32_t)(entry >> 48), dg = o.inner;
         const uint32_t s = (cp >> UPV_SHIFT) & sm;
-        const uint32_t flip = (dg >> 2) & 1;                   // lanes 0-3 and 4-7 start on different halves
+        const uint32_t flip = (dg >> 2) & 1;
         const u32x4 lo = lds_vec[cp * gpr + ((2 * dg + flip) ^ s)];
         const u32x4 hi = lds_vec[cp * gpr + ((2 * dg + 1 - flip) ^ s)];
         const u32x4 g0 = flip ? hi : lo, g1 = flip ? lo : hi;
         u32x4 kx, vx;
         split_kv<ES>(g0, g1, kx, vx);
-        const uint64_t ra = (entry & 0xFFFFFFFFFFFFull) + (uint64_t)(dg * 16);
-        store16(ra, kx, sys);
-        store16(ra + kv_bytes, vx, sys);
+        swap_half_waves(kx, vx);                               // kx = {K A | V A}, vx = {K B | V B}
+        const uint64_t ra = entry & 0xFFFFFFFFFFFFull;         // K row of this lane's pair
+        const uint64_t kib_a = from_lane(ra, 0), kib_b = from_lane(ra, 32);   // lane 0 / 32: head 0 of its layer
+        const bool valid_a = __builtin_amdgcn_readlane((int)valid, 0) != 0;
+        const bool valid_b = __builtin_amdgcn_readlane((int)valid, 32) != 0;
+        if (valid_a) store16(kib_a + lane * 16u, kx, sys);
+        if (valid_b) store16(kib_b + lane * 16u, vx, sys);
+        uwalk_step(o, a.q_cp, a.r_cp, dgs);
       }
-      uwalk_step(o, a.q_cp, a.r_cp, dgs);
+    } else {
+      for (uint32_t base = 0; base < n_cp; base += B) {
+        if (o.outer < Cw) {
+          const uint64_t entry = row_addr[o.outer];
+          const uint32_t cp = (uint32_t)(entry >> 48), dg = o.inner;
+          const uint32_t s = (cp >> UPV_SHIFT) & sm;
+          const uint32_t flip = (dg >> 2) & 1;                   // lanes 0-3 and 4-7 start on different halves
+          const u32x4 lo = lds_vec[cp * gpr + ((2 * dg + flip) ^ s)];
+          const u32x4 hi = lds_vec[cp * gpr + ((2 * dg + 1 - flip) ^ s)];
+          const u32x4 g0 = flip ? hi : lo, g1 = flip ? lo : hi;
+          u32x4 kx, vx;
+          split_kv<ES>(g0, g1, kx, vx);
+          const uint64_t ra = (entry & 0xFFFFFFFFFFFFull) + (uint64_t)(dg * 16);
+          store16(ra, kx, sys);
+          store16(ra + kv_bytes, vx, sys);
+        }
+        uwalk_step(o, a.q_cp, a.r_cp, dgs);
+      }
     }
   } else {
     // compute rows -> LDS: a K vector and a V vector interleave into 32 bytes of units
@@ -377,14 +423,26 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
         const uint32_t jj = ou.outer < Cw ? ou.outer : 0;      // a lane past the end re-reads row 0
         const uint64_t entry = row_addr[jj];
         cps[u] = (uint32_t)(entry >> 48);
-        const uint64_t ra = (entry & 0xFFFFFFFFFFFFull) + (uint64_t)(ou.inner * 16);
-        kx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)ra);
-        vx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(ra + kv_bytes));
+        if (a.kv_swap) {
+          // one contiguous KiB per load instruction: the whole wave reads {K | V} of layer A, then of layer B
+          // (see the store side of the other direction); the exchange after the loads gives every lane the
+          // K vector and the V vector of its own pair
+          const uint64_t row = entry & 0xFFFFFFFFFFFFull;
+          const uint64_t kib_a = from_lane(row, 0), kib_b = from_lane(row, 32);
+          const uint32_t lane = tid & 63u;
+          kx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(kib_a + lane * 16u));
+          vx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(kib_b + lane * 16u));
+        } else {
+          const uint64_t ra = (entry & 0xFFFFFFFFFFFFull) + (uint64_t)(ou.inner * 16);
+          kx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)ra);
+          vx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(ra + kv_bytes));
+        }
         uwalk_step(ou, a.q_cp, a.r_cp, dgs);
       }
 #pragma unroll
       for (uint32_t u = 0; u < U; ++u) {
         if (base + u * B >= n_cp) break;
+        if (a.kv_swap) swap_half_waves(kx[u], vx[u]);          // {K A | V A}, {K B | V B} -> {K A | K B}, {V A | V B}
         if (o.outer < Cw) {
           const uint32_t cp = cps[u], dg = o.inner;
           const uint32_t s = (cp >> UPV_SHIFT) & sm;
@@ -480,6 +538,11 @@ hipError_t launch_transpose_pages(int dir, TransposeArgs& a, hipStream_t stream)
       a.m_dgs = magic(dgs);
       a.m_chunks = magic(a.n_chunks);
       a.sys_scope = (uint32_t)tuning().transpose_sc1;
+      // K rows and V rows of a (token, layer) adjacent (the Worker's [tokens, 2, heads, dim] tensors), half a
+      // KiB each, whole token in one tile: half-waves can be exchanged so that every global access of a wave
+      // on the compute side is one contiguous KiB
+      a.kv_swap = (tuning().transpose_kvswap != 0 && a.n_chunks == 1 && n_heads * dgs == 32 &&
+                   a.kv_stride * ES == 512 && (uint32_t)block % 64u == 0) ? 1u : 0u;
       a.q_tm = (uint32_t)block / vpr;
       a.r_tm = (uint32_t)block % vpr;
       a.q_cp = (uint32_t)block / dgs;

@@ -41,6 +41,8 @@ def _make(rng, form, es, P, D, H, L, blocks, n_tm, cuda):
     (4, 3, 128, 4, 16),      # fp32, 128 columns: chunked
     (2, 4, 64, 4, 1),        # a single layer
     (2, 64, 128, 8, 32),     # 64 tokens per block x four column chunks: 256 workgroups per page
+    (4, 3, 64, 2, 5),        # fp32 with half-KiB K rows and an odd layer count: the last wave's upper half-wave has no layer
+    (1, 6, 128, 4, 6),       # 1-byte elements whose K rows are half a KiB (4 heads x 128)
 ])
 @pytest.mark.parametrize("pairs", [1, 0])
 def test_load_and_store_match_oracle(lib, oracle, cuda, form, es, P, D, H, L, pairs):
@@ -93,6 +95,37 @@ def test_word_pair_kernel_at_other_workgroup_sizes(lib, oracle, cuda, block):
         pool.store_token_major(tm_d, torch.from_numpy(ids2).to(cuda), torch.from_numpy(pages2).to(cuda))
         pool.check()
         oracle.transpose_pages_c(layers_h, "block_kv", tm_h, ids2, pages2, "store")
+        assert _to_np(tm_d).tobytes() == tm_h.tobytes()
+    finally:
+        bk.reset_tuning()
+
+
+@pytest.mark.parametrize("kvswap", [1, 0])
+@pytest.mark.parametrize("block", [0, 128, 256, 512, 1024])
+def test_half_wave_exchange_on_the_workers_own_shape(lib, oracle, cuda, block, kvswap):
+    """The Worker's tensors at 2 KV heads x 128 x fp16 (K and V rows of a token adjacent, half a KiB each):
+    the pair kernel reads and writes whole KiB and exchanges half-waves; with the exchange switched off
+    every lane addresses its own rows. Both, at every workgroup size, against the oracle."""
+    import bikv_pagecopy as bk
+    print(f"[case] layout change, half-wave exchange={kvswap}, {block or 'default'} lanes", flush=True)
+    rng = np.random.default_rng(900 + block + kvswap)
+    P, D, H, L, blocks, n_tm = 7, 128, 2, 10, 11, 8
+    tm_h, layers_h, tm_d, layers_d = _make(rng, "token_kv", 2, P, D, H, L, blocks, n_tm, cuda)
+    pool = bk.NHDPool.from_token_kv_layers(layers_d, P)
+    bk.set_tuning(transpose_block=block, transpose_kvswap=kvswap)
+    try:
+        ids = rng.permutation(blocks)[:6].astype(np.int64)
+        pages = rng.permutation(n_tm)[:6].astype(np.int64)
+        pool.load_token_major(tm_d, torch.from_numpy(ids).to(cuda), torch.from_numpy(pages).to(cuda))
+        pool.check()
+        oracle.transpose_pages_c(layers_h, "token_kv", tm_h, ids, pages, "load")
+        for l in range(L):
+            assert _to_np(layers_d[l]).tobytes() == layers_h[l].tobytes(), f"layer {l}"
+        ids2 = rng.permutation(blocks)[:5].astype(np.int64)
+        pages2 = rng.permutation(n_tm)[:5].astype(np.int64)
+        pool.store_token_major(tm_d, torch.from_numpy(ids2).to(cuda), torch.from_numpy(pages2).to(cuda))
+        pool.check()
+        oracle.transpose_pages_c(layers_h, "token_kv", tm_h, ids2, pages2, "store")
         assert _to_np(tm_d).tobytes() == tm_h.tobytes()
     finally:
         bk.reset_tuning()
