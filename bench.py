@@ -2,7 +2,7 @@
 """Benchmark of the KV page-copy hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload qwen2_7b|qwen2_1p5b|llama3_8b|
-                    llama3_70b_fp8|qwen2_7b_token_major|layout_change|staging|reference_200x50]
+                    llama3_70b_fp8|qwen2_7b_token_major|layout_change|staging|staging_trace|reference_200x50]
                     [--pool-form planar|worker] [--pool-alloc spread|stacked|planes] [--layout layer_major|page_major]
 
 Default workload = the configuration the headline target is quoted on: the Qwen2-7B-shaped bf16 pool
@@ -47,17 +47,17 @@ HBM_PEAK_GBPS = 8000.0
 # WRITE_SIZE runs of this file, each scaled by the same counter's reading for the plain-copy
 # calibration launch below (summaries under profiles/). None = not measured for that workload.
 MEASURED_TRAFFIC_RATIO = {"qwen2_7b": {"gather": 0.9948, "scatter": 1.0002},
-                          "qwen2_1p5b": {"gather": 1.001},
+                          "qwen2_1p5b": {"gather": 1.0009},
                           "llama3_8b": {"gather": 0.9967},
                           "llama3_70b_fp8": {"gather": 1.0142, "scatter": 1.0002},
                           "qwen2_7b_token_major": {"gather": 0.9998, "scatter": 1.0002},
-                          "layout_change": {"load": 1.0029, "store": 1.0035}}
+                          "layout_change": {"load": 1.0003, "store": 1.0023}}
 
 
 # The ratios above describe the kernels as they were when the counters were read: the SHA-256 (first 16 hex
 # digits) of the two kernel sources at that time. A run whose kernel sources differ reports `traffic: null`
 # and says why, so that a change which re-reads data cannot keep printing an old ratio.
-TRAFFIC_MEASURED_AT = "to-be-measured"
+TRAFFIC_MEASURED_AT = "7ceba33e6a35aeeb"
 
 
 def kernel_source_digest():
@@ -761,6 +761,115 @@ def run_staging(args, bk, workloads, dev, kept=None):
     return out
 
 
+def trace_summary(steps):
+    """A stager trace (HostStager.trace_read) reduced to what tells where the time of a pass goes: per kind of
+    step the count and duration percentiles; copies by their position behind their lane's last kernel; how much
+    of the pass at least one copy was running, how far the lanes' copy intervals overlap, and the gaps between
+    consecutive steps of a lane."""
+    import numpy as np
+    if not steps:
+        return None
+    span = max(s["end_ms"] for s in steps) - min(s["start_ms"] for s in steps)
+    out = {"steps": len(steps), "span_ms": round(span, 2), "kinds": {}, "copies_by_position_behind_their_kernel": {}}
+    for kind in sorted({s["kind"] for s in steps}):
+        ss = [s for s in steps if s["kind"] == kind]
+        d = np.array([s["end_ms"] - s["start_ms"] for s in ss])
+        b = float(sum(s["bytes"] for s in ss))
+        out["kinds"][kind] = {"n": len(ss), "MiB_per_step": round(b / len(ss) / 2 ** 20, 2), "ms_mean": round(float(d.mean()), 4),
+                              "ms_p10": round(float(np.percentile(d, 10)), 4), "ms_p50": round(float(np.percentile(d, 50)), 4),
+                              "ms_p90": round(float(np.percentile(d, 90)), 4), "ms_max": round(float(d.max()), 4),
+                              "GBps_while_running": round(b / max(float(d.sum()), 1e-9) / 1e6, 1)}
+    lanes = sorted({s["lane"] for s in steps})
+    pos, gaps = {}, {}
+    for lane in lanes:
+        ls = [s for s in steps if s["lane"] == lane]
+        k = 0
+        for s in ls:
+            if s["kind"] == "kernel":
+                k = 0
+            elif s["kind"].startswith("copy"):
+                k += 1
+                pos.setdefault(k, []).append(s["end_ms"] - s["start_ms"])
+        g = np.array([ls[i + 1]["start_ms"] - ls[i]["end_ms"] for i in range(len(ls) - 1)] or [0.0])
+        gaps[f"lane_{lane}"] = {"steps": len(ls), "gap_ms_p50": round(float(np.percentile(g, 50)), 4),
+                                "gap_ms_p90": round(float(np.percentile(g, 90)), 4), "gap_ms_max": round(float(g.max()), 3)}
+    for k in sorted(pos):
+        d = np.array(pos[k])
+        out["copies_by_position_behind_their_kernel"][f"copy_{k}"] = {
+            "n": len(d), "ms_p50": round(float(np.percentile(d, 50)), 4), "ms_p90": round(float(np.percentile(d, 90)), 4)}
+    cs = sorted((s["start_ms"], s["end_ms"]) for s in steps if s["kind"].startswith("copy"))
+    if cs:
+        busy, cur_s, cur_e = 0.0, cs[0][0], cs[0][1]
+        for a_, b_ in cs[1:]:
+            if a_ > cur_e:
+                busy += cur_e - cur_s
+                cur_s, cur_e = a_, b_
+            else:
+                cur_e = max(cur_e, b_)
+        busy += cur_e - cur_s
+        cb = sum(s["bytes"] for s in steps if s["kind"].startswith("copy"))
+        out["copies"] = {"some_copy_running_pct_of_span": round(100 * busy / span, 1),
+                         "GBps_while_some_copy_runs": round(cb / busy / 1e6, 1),
+                         "overlap_factor": round(sum(e - a_ for a_, e in cs) / busy, 2)}
+    out["gaps_between_steps_of_a_lane"] = gaps
+    return out
+
+
+def run_staging_trace(args, bk, workloads, dev):
+    """Where the time of a pipelined pass goes, step by step: the library's own trace (two events around every
+    kernel launch and host copy of a lane, bikv_stager_trace) of the FIRST pass a fresh process makes and of a
+    later one, for the hipMemcpyAsync pipeline and for the copy-kernel pipeline. Llama-3-8B-shaped pool of
+    --pool-pages pages (default 8192 = 34 GB), the first --staging-requests requests (default here: 24, 10 GB
+    per pass), passes back to back."""
+    import numpy as np
+    import torch
+    shape = workloads.SHAPES["llama3_8b"].scaled(args.pool_pages or 8192)
+    wl = workloads.named("llama3_8b", shape)
+    pool_t, _ = make_pool(shape, dev, args.pool_alloc)
+    pool = bk.PagedKVPool.from_planes(pool_t)
+    reqs = wl["gather"][: (args.staging_requests if args.staging_requests != 128 else 24)]
+    sizes = np.array([len(r) * shape.page_bytes for r in reqs], dtype=np.int64)
+    region = int(max(4 << 30, 2 * sizes.max()))
+    host = bk.pinned_empty(region)
+    offs, cur = [], 0
+    for sz in sizes:
+        if cur + sz > region:
+            cur = 0
+        offs.append(cur)
+        cur += int(sz)
+    batches = [pool.make_batch([r], "layer_major") for r in reqs]
+    total = int(sizes.sum())
+    torch.cuda.synchronize(dev)
+    t_ready = time.perf_counter()
+    chunk, lanes, group = (args.chunk_mib or 16), args.buffers, (args.per_launch if args.chunk_mib else 2)
+    record = {"workload": f"llama3_8b x {shape.n_pages} pages, {len(reqs)} requests = {total / 1e9:.1f} GB per pass, "
+                          f"{chunk} MiB x {group} copies per launch x {lanes} lanes", "modes": {}}
+    for mode in ("pipelined", "pipelined_kernel"):
+        st = bk.HostStager(dev, chunk_bytes=chunk << 20, n_buffers=lanes, chunks_per_launch=group)
+        rates, traces = [], {}
+        for p in range(10):
+            traced = p in (0, 8)
+            if traced:
+                st.trace(40000)
+            t0 = time.perf_counter()
+            for b, off, sz in zip(batches, offs, sizes):
+                st.gather_to_host_async(pool, b, host[off: off + int(sz)], mode)
+            st.wait()
+            rates.append(round(total / (time.perf_counter() - t0) / 1e9, 1))
+            if traced:
+                traces[f"pass_{p}"] = dict(trace_summary(st.trace_read()), GBps=rates[-1],
+                                           started_s_after_setup=round(t0 - t_ready, 2))
+                st.trace(0)
+        st.close()
+        dev_buf = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        plain = [round((1 << 30) / bk.measure_d2h(dev, host[: 1 << 30], dev_buf, 0) / 1e9, 1) for _ in range(3)]
+        del dev_buf
+        record["modes"][mode] = {"passes_GBps": rates, "plain_1GiB_d2h_after_GBps": plain, "traces": traces}
+        log(f"staging_trace {mode}: {rates}")
+    pool.close()
+    return record
+
+
 def run_reference_scenario(args, bk, dev):
     """The only workload the reference itself scripts: 200 pages x 50 tokens x 14336 fp16 elements,
     identity offsets, one run copy per transfer (test_page_ipc.py:41-65)."""
@@ -1151,6 +1260,10 @@ def main():
                 out[key] = {"workload": o["config"]["workload"], "pool_GB": o["config"]["pool_GB"], "value": o["value"],
                             "pct_of_hbm_peak": o["pct_of_hbm_peak"], "kernels": o["kernels"]}
         emit(out)
+        return
+    if args.workload == "staging_trace":
+        print(json.dumps({"metric": "pinned-host staging GB/s", "unit": "GB/s", "n_gpus": 1,
+                          "staging_trace": run_staging_trace(args, bk, workloads, dev), "device_alloc": ALLOC_NOTES}), flush=True)
         return
     if args.workload == "staging":
         print(json.dumps({"metric": "pinned-host staging GB/s", "unit": "GB/s", "n_gpus": 1,
