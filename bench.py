@@ -549,9 +549,10 @@ def run_staging(args, bk, workloads, dev, kept=None):
                 after it;
     cells       chunk sizes, lane counts and modes, three timed passes each after two untimed ones, each next
                 to a plain hipMemcpyAsync of one 1 GiB pinned buffer timed immediately before it. Before the
-                first cell the run waits until plain copies hold their full rate (normally no wait at all;
-                the wait is reported): this benchmark has just released hundreds of GB of device memory, and
-                for as long as the driver scrubs released memory every hipMemcpyAsync can run at half rate."""
+                first cell the run repeats short pipelined passes until two in a row are at full rate (the
+                rates seen and the time are reported): this benchmark has just released hundreds of GB of
+                device memory, and for as long as the driver scrubs released memory, copies that land on the
+                copy engine it uses run at half rate."""
     import numpy as np
     import torch
 
@@ -674,13 +675,17 @@ def run_staging(args, bk, workloads, dev, kept=None):
                      "hipMemcpyAsync calls of 64 MiB right before / after the pass")
     log(f"staging first_pass {first}")
 
-    # --- 2. wait until the copy engines are back at full rate (the scrub of what this run freed), then the cells
+    # --- 2. wait until the hipMemcpyAsync lanes are back at full rate (the scrub of what this run released), then
+    # the cells. The probe is the thing itself: short passes of the pipelined mode on a stager of the default
+    # shape (a single plain copy is no probe: in this process it keeps its full rate while the lanes do not).
     t_wait, settle = time.perf_counter(), []
+    probe = bk.HostStager(dev)
+    plain_now = small_copy_rate("d2h", 0.1)
     while True:
-        r = small_copy_rate("d2h", 0.2)
-        settle.append(round(r, 1))
-        if (len(settle) >= 3 and min(settle[-3:]) > 50.0) or time.perf_counter() - t_wait > 60.0:
+        settle.append(round(one_pass(probe, "pipelined", "gather", n_short), 1))
+        if (len(settle) >= 2 and min(settle[-2:]) > 0.93 * plain_now) or time.perf_counter() - t_wait > 60.0:
             break
+    probe.close()
     settle_s = time.perf_counter() - t_wait
     # the first DMA into a pinned page is slower than later ones: the whole region has been touched by now
     # only if the passes above covered it, so touch it once
@@ -728,9 +733,10 @@ def run_staging(args, bk, workloads, dev, kept=None):
                        f"pages ({total_bytes / 1e9:.2f} GB per pass), enqueued back to back, {passes} timed passes per cell after two untimed ones",
            "pool_GB": round(shape.pool_bytes / 1e9, 2),
            "first_pass": first,
-           "wait_for_full_rate_copies": {"seconds": round(settle_s, 2), "plain_64MiB_d2h_GBps_seen": settle,
-                                         "what": "time from the end of the first passes until back-to-back plain hipMemcpyAsync "
-                                                 "calls held > 50 GB/s three times in a row (60 s at most); nothing is staged meanwhile"},
+           "wait_for_full_rate_copies": {"seconds": round(settle_s, 2), "pipelined_pass_GBps_seen": settle,
+                                         "what": f"passes of {short_bytes / 1e9:.1f} GB in the pipelined mode (16 MiB x 2 x 2 lanes) from "
+                                                 "the end of the first passes until two in a row exceed 93 % of a plain copy (60 s at "
+                                                 "most): how long the driver was still scrubbing the device memory this run had released"},
            "plain_d2h_GBps": {"min": round(min(yard["d2h"]), 2), "median": round(float(np.median(yard["d2h"])), 2),
                               "max": round(max(yard["d2h"]), 2), "samples": len(yard["d2h"])},
            "plain_h2d_GBps": {"min": round(min(yard["h2d"]), 2), "median": round(float(np.median(yard["h2d"])), 2),
@@ -844,28 +850,73 @@ def run_staging_trace(args, bk, workloads, dev):
     chunk, lanes, group = (args.chunk_mib or 16), args.buffers, (args.per_launch if args.chunk_mib else 2)
     record = {"workload": f"llama3_8b x {shape.n_pages} pages, {len(reqs)} requests = {total / 1e9:.1f} GB per pass, "
                           f"{chunk} MiB x {group} copies per launch x {lanes} lanes", "modes": {}}
-    for mode in ("pipelined", "pipelined_kernel"):
-        st = bk.HostStager(dev, chunk_bytes=chunk << 20, n_buffers=lanes, chunks_per_launch=group)
+    def run_passes(st, mode, n, traced=()):
         rates, traces = [], {}
-        for p in range(10):
-            traced = p in (0, 8)
-            if traced:
+        for p in range(n):
+            if p in traced:
                 st.trace(40000)
             t0 = time.perf_counter()
             for b, off, sz in zip(batches, offs, sizes):
                 st.gather_to_host_async(pool, b, host[off: off + int(sz)], mode)
             st.wait()
             rates.append(round(total / (time.perf_counter() - t0) / 1e9, 1))
-            if traced:
+            if p in traced:
                 traces[f"pass_{p}"] = dict(trace_summary(st.trace_read()), GBps=rates[-1],
                                            started_s_after_setup=round(t0 - t_ready, 2))
                 st.trace(0)
+        return rates, traces
+
+    dev_buf = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+
+    def plain(seconds=0.15):
+        """mean rate of back-to-back plain hipMemcpyAsync calls of 64 MiB (a fresh stream each)"""
+        n, moved, spent, t0 = dev_buf.numel(), 0, 0.0, time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            spent += bk.measure_d2h(dev, host[:n], dev_buf, 0)
+            moved += n
+        return round(moved / spent / 1e9, 1)
+
+    def fresh():
+        return bk.HostStager(dev, chunk_bytes=chunk << 20, n_buffers=lanes, chunks_per_launch=group)
+
+    # 1. the first thing the process stages, right behind the pool's placement (which released its filler chunks)
+    for mode in ("pipelined", "pipelined_kernel"):
+        st = fresh()
+        rates, traces = run_passes(st, mode, 10, traced=(0, 8))
         st.close()
-        dev_buf = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-        plain = [round((1 << 30) / bk.measure_d2h(dev, host[: 1 << 30], dev_buf, 0) / 1e9, 1) for _ in range(3)]
-        del dev_buf
-        record["modes"][mode] = {"passes_GBps": rates, "plain_1GiB_d2h_after_GBps": plain, "traces": traces}
+        record["modes"][mode] = {"passes_GBps": rates, "plain_64MiB_d2h_after_GBps": plain(), "traces": traces}
         log(f"staging_trace {mode}: {rates}")
+    # 2. nothing released for a while: a fresh stager, first pass traced
+    time.sleep(8.0)
+    st = fresh()
+    rates, traces = run_passes(st, "pipelined", 6, traced=(0,))
+    st.close()
+    record["settled"] = {"what": "a fresh stager 8 s later, nothing released in between", "plain_64MiB_d2h_before_GBps": plain(),
+                         "pipelined_passes_GBps": rates, "traces": traces}
+    log(f"staging_trace settled: {rates}")
+    # 3. 32 GiB of device memory allocated and released (the release returns at once), then a fresh stager at once
+    t_rel = time.perf_counter()
+    bk.DeviceBuffer(32 << 30, dev, spread=False).free()
+    rel_ms = (time.perf_counter() - t_rel) * 1e3
+    before = plain(0.1)
+    st = fresh()
+    rates, traces = run_passes(st, "pipelined", 14, traced=(0,))
+    after = plain()
+    k_rates, _ = run_passes(st, "pipelined_kernel", 3)
+    st.close()
+    bk.DeviceBuffer(32 << 30, dev, spread=False).free()
+    st = fresh()
+    k2_rates, _ = run_passes(st, "pipelined_kernel", 6)
+    d_rates, _ = run_passes(st, "direct", 3)
+    st.close()
+    record["after_release"] = {"what": "32 GiB allocated and released (bikv_device_alloc sequential + bikv_device_free, "
+                                       f"{rel_ms:.0f} ms for both), then a fresh stager at once",
+                               "plain_64MiB_d2h_right_after_the_release_GBps": before, "pipelined_passes_GBps": rates,
+                               "seconds_per_pass": round(total / 1e9 / max(rates[0], 1e-9), 3),
+                               "plain_64MiB_d2h_after_the_passes_GBps": after, "pipelined_kernel_passes_after_GBps": k_rates,
+                               "second_release_then_pipelined_kernel_passes_GBps": k2_rates, "then_direct_passes_GBps": d_rates,
+                               "traces": traces}
+    log(f"staging_trace after release: {rates} | kernel hop right after a second release: {k2_rates}")
     pool.close()
     return record
 
