@@ -239,8 +239,6 @@ extern "C" int bikv_set_tuning(const char* key, int64_t value) {
     t.transpose_block = (int)value;
   } else if (!strcmp(key, "transpose_sc1")) {
     t.transpose_sc1 = value ? 1 : 0;
-  } else if (!strcmp(key, "transpose_ld_sc1")) {
-    t.transpose_ld_sc1 = value ? 1 : 0;
   } else if (!strcmp(key, "transpose_kvswap")) {
     t.transpose_kvswap = value ? 1 : 0;
   } else if (!strcmp(key, "transpose_pairs")) {

@@ -66,7 +66,6 @@ struct Tuning {
   int transpose_block = 0;     // lanes per workgroup of the K/V-pair kernel: 128, 256, 512, 1024;
                                // 0 = chosen per direction (256 for the load, 512 for the store)
   int transpose_sc1 = 1;       // K/V-pair kernel: payload stores are nt with system scope (0 = nt only)
-  int transpose_ld_sc1 = 0;    // K/V-pair kernel: payload loads are nt with system scope (0 = nt only)
   int transpose_kvswap = 0;    // K/V-pair kernel: 1 = whole-KiB compute-side accesses by exchanging half-waves, where
                                // the pool's shape allows; 0 = every lane addresses its own K and V rows (default:
                                // measured, the exchange costs the store 1.7 % and gains the load 0.6 %)
@@ -125,7 +124,6 @@ struct TransposeArgs {
   uint32_t n_heads, m_heads, m_layers, m_vpr, m_dgs, m_chunks;
   uint32_t q_tm, r_tm, q_cp, r_cp;
   uint32_t sys_scope;             // payload stores carry system scope besides nt
-  uint32_t load_sys_scope;        // payload loads carry system scope besides nt
   uint32_t kv_swap;               // pair kernel: K and V rows of a (token, layer) are the halves of one KiB and a
                                   // half-wave covers a layer's K rows: compute-side accesses exchange half-waves
   uint32_t* status;

@@ -271,28 +271,6 @@ __device__ __forceinline__ uint64_t from_lane(uint64_t v, int src) {
   return ((uint64_t)hi << 32) | lo;
 }
 
-// 16-byte payload load: nt, or nt with system scope. The latter is written out as an instruction, which the
-// compiler does not track: the loads of a batch are issued back to back and await_loads() stands between
-// them and the first use of any of their results (its operands tie the results to the wait).
-__device__ __forceinline__ u32x4 load16(uint64_t p, bool sys) {
-  u32x4 v;
-  if (sys)
-    asm volatile("global_load_dwordx4 %0, %1, off sc1 nt" : "=v"(v) : "v"(p) : "memory");
-  else
-    v = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)p);
-  return v;
-}
-template <int N>
-__device__ __forceinline__ void await_loads(u32x4 (&x)[N], bool sys) {
-  if (!sys) return;
-  if constexpr (N == 4)
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]) : : "memory");
-  else
-    asm volatile("s_waitcnt vmcnt(0)"
-                 : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])
-                 : : "memory");
-}
-
 template <int DIR, int ES, int B>
 __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs a) {
   using Unit = typename UnitOf<ES>::T;
@@ -307,7 +285,6 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
 
   const uint32_t tid = threadIdx.x;
   const bool sys = a.sys_scope != 0;
-  const bool lsys = a.load_sys_scope != 0;
   const uint32_t t = udiv_small(blockIdx.x, a.m_chunks);       // token within the page
   const uint32_t chunk = blockIdx.x - t * a.n_chunks;          // column chunk
   const uint64_t i = (uint64_t)blockIdx.y + (uint64_t)blockIdx.z * gridDim.y;
@@ -367,16 +344,15 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
     constexpr uint32_t U = 8;
     UWalk w = uwalk_start(tid, vpr, a.m_vpr);                  // (d, vector within the row piece)
     for (uint32_t base = 0; base < n_tm; base += B * U) {
-      u32x4 x[U] = {};
+      u32x4 x[U];
       UWalk wu = w;
 #pragma unroll
       for (uint32_t u = 0; u < U; ++u) {
         if (base + u * B >= n_tm) break;                       // whole workgroup past the end: nothing to load
         const uint32_t d = wu.outer < D ? wu.outer : 0;        // a lane past the end re-reads row 0
-        x[u] = load16((uint64_t)(tm_tok + (d * tm_row_bytes + wu.inner * 16)), lsys);
+        x[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(tm_tok + (d * tm_row_bytes + wu.inner * 16)));
         uwalk_step(wu, a.q_tm, a.r_tm, vpr);
       }
-      await_loads(x, lsys);
 #pragma unroll
       for (uint32_t u = 0; u < U; ++u) {
         if (base + u * B >= n_tm) break;
@@ -446,7 +422,7 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
     constexpr uint32_t U = 4;
     UWalk o = uwalk_start(tid, dgs, a.m_dgs);
     for (uint32_t base = 0; base < n_cp; base += B * U) {
-      u32x4 kx[U] = {}, vx[U] = {};
+      u32x4 kx[U], vx[U];
       uint32_t cps[U];
       UWalk ou = o;
 #pragma unroll
@@ -462,17 +438,15 @@ __global__ __launch_bounds__(B) void transpose_pairs_kernel(const TransposeArgs 
           const uint64_t row = entry & 0xFFFFFFFFFFFFull;
           const uint64_t kib_a = from_lane(row, 0), kib_b = from_lane(row, 32);
           const uint32_t lane = tid & 63u;
-          kx[u] = load16(kib_a + lane * 16u, lsys);
-          vx[u] = load16(kib_b + lane * 16u, lsys);
+          kx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(kib_a + lane * 16u));
+          vx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(kib_b + lane * 16u));
         } else {
           const uint64_t ra = (entry & 0xFFFFFFFFFFFFull) + (uint64_t)(ou.inner * 16);
-          kx[u] = load16(ra, lsys);
-          vx[u] = load16(ra + kv_bytes, lsys);
+          kx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)ra);
+          vx[u] = __builtin_nontemporal_load((const BIKV_GLOBAL u32x4*)(ra + kv_bytes));
         }
         uwalk_step(ou, a.q_cp, a.r_cp, dgs);
       }
-      await_loads(kx, lsys);
-      await_loads(vx, lsys);
 #pragma unroll
       for (uint32_t u = 0; u < U; ++u) {
         if (base + u * B >= n_cp) break;
@@ -572,7 +546,6 @@ hipError_t launch_transpose_pages(int dir, TransposeArgs& a, hipStream_t stream)
       a.m_dgs = magic(dgs);
       a.m_chunks = magic(a.n_chunks);
       a.sys_scope = (uint32_t)tuning().transpose_sc1;
-      a.load_sys_scope = (uint32_t)tuning().transpose_ld_sc1;
       // K rows and V rows of a (token, layer) adjacent (the Worker's [tokens, 2, heads, dim] tensors), half a
       // KiB each, whole token in one tile: half-waves can be exchanged so that every global access of a wave
       // on the compute side is one contiguous KiB

@@ -79,8 +79,6 @@ int bikv_check_status(int device, void* stream, uint32_t* bits_out);
  * "transpose_pairs" (1 = the K/V-pair kernel, default; 0 = the element-wise kernel), "transpose_block"
  * (its lanes per workgroup: 128, 256, 512, 1024; 0 = default: 256 for the load, 512 for the store) and
  * "transpose_sc1" (1 = its payload stores are nt with system scope, default; 0 = nt only),
- * "transpose_ld_sc1" (1 = its payload loads are nt with system scope as well; 0 = default, nt only: no
- * measurable difference),
  * "transpose_kvswap" (1 = where K and V rows of a token are adjacent halves of one KiB — the Worker's own
  * tensors at 2 KV heads x 128 x fp16 — the pair kernel reads and writes whole KiB on the pool side and
  * exchanges half-waves between lanes; 0 = default: every lane addresses its own rows, which measures 1.7 %

@@ -99,7 +99,7 @@ def test_measure_d2h_runs(lib, cuda):
 
 
 @pytest.mark.parametrize("layout", ["layer_major", "page_major"])
-@pytest.mark.parametrize("mode", ["pipelined", "direct"])
+@pytest.mark.parametrize("mode", ["pipelined", "direct", "pipelined_kernel"])
 def test_scatter_from_host_matches_oracle(lib, oracle, cuda, layout, mode):
     """Pinned staging image -> pool pages, payload and scales, at chunk sizes around the requests."""
     import bikv_pagecopy as bk

@@ -131,39 +131,6 @@ def test_half_wave_exchange_on_the_workers_own_shape(lib, oracle, cuda, block, k
         bk.reset_tuning()
 
 
-@pytest.mark.parametrize("es,P,D,H,L,form", [(2, 16, 128, 2, 28, "token_kv"), (2, 8, 128, 8, 32, "block_kv"),
-                                               (1, 6, 128, 8, 20, "token_kv"), (4, 3, 64, 2, 5, "token_kv")])
-def test_system_scope_loads_move_the_same_bytes(lib, oracle, cuda, es, P, D, H, L, form):
-    """transpose_ld_sc1 = 1: the pair kernel's payload loads are written out as instructions (nt + system
-    scope) and awaited by hand; same result as with compiler-tracked loads, with and without the half-wave
-    exchange."""
-    import bikv_pagecopy as bk
-    print(f"[case] layout change, system-scope loads es={es} P={P} D={D} H={H} L={L} {form}", flush=True)
-    rng = np.random.default_rng(77 + es + H)
-    blocks, n_tm = 9, 7
-    for kvswap in (0, 1):
-        tm_h, layers_h, tm_d, layers_d = _make(rng, form, es, P, D, H, L, blocks, n_tm, cuda)
-        pool = (bk.NHDPool.from_token_kv_layers(layers_d, P) if form == "token_kv" else bk.NHDPool.from_block_kv_layers(layers_d))
-        bk.set_tuning(transpose_ld_sc1=1, transpose_kvswap=kvswap)
-        try:
-            ids = rng.permutation(blocks)[:6].astype(np.int64)
-            pages = rng.permutation(n_tm)[:6].astype(np.int64)
-            pool.load_token_major(tm_d, torch.from_numpy(ids).to(cuda), torch.from_numpy(pages).to(cuda))
-            pool.check()
-            oracle.transpose_pages_c(layers_h, form, tm_h, ids, pages, "load")
-            for l in range(L):
-                assert _to_np(layers_d[l]).tobytes() == layers_h[l].tobytes(), f"layer {l}"
-            ids2 = rng.permutation(blocks)[:5].astype(np.int64)
-            pages2 = rng.permutation(n_tm)[:5].astype(np.int64)
-            pool.store_token_major(tm_d, torch.from_numpy(ids2).to(cuda), torch.from_numpy(pages2).to(cuda))
-            pool.check()
-            oracle.transpose_pages_c(layers_h, form, tm_h, ids2, pages2, "store")
-            assert _to_np(tm_d).tobytes() == tm_h.tobytes()
-        finally:
-            bk.reset_tuning()
-        pool.close()
-
-
 def test_default_tm_pages_is_a_dense_received_buffer(lib, oracle, cuda):
     """A received tensor (tokens,)+token_shape (Worker.py:166-169) is pages 0..n-1 in order."""
     import bikv_pagecopy as bk
