@@ -26,6 +26,12 @@ chunks on 2 and 4 lanes, kernel-direct and automatic modes, both directions, eac
 hipMemcpyAsync of one large pinned buffer timed immediately before it. `--no-configs` / `--no-staging`
 skip those parts.
 
+`roofline.traffic` (HBM bytes per launch of the dominant kernel) is measured at the end of the default run: the
+headline workload is run twice more as a child process under `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE),
+each counter scaled by its reading for the plain 2 GiB copy of the same child (`roofline.traffic_live`). If the
+profiler is missing or a child fails, and with `--no-live-traffic`, the figure is the run's algorithmic bytes
+times the ratio recorded from the same two commands under profiles/ (`traffic_source` says which).
+
 Pools and gather destinations are allocated through the library's bikv_device_alloc, which lays their
 physical chunks alternately in the two halves of HBM (`--pool-alloc torch` / `--staging-alloc torch`
 take torch's allocator instead; the default run times the headline workload once more that way and
@@ -86,6 +92,77 @@ def traffic_ratio(workload, kind):
     return r, TRAFFIC_SOURCE
 
 
+def measure_traffic_live(workload, dominant_kernel, alg_bytes, limit_s=150):
+    """HBM bytes per launch of `dominant_kernel`, measured now: this file is run twice more as a child process
+    under `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE; one counter per run), on the same workload at full size
+    with three timed steps. Each counter's mean per dispatch of the kernel is scaled by what the same counter
+    reads for the plain 2 GiB copy the child also launches. Returns (bytes or None, dict describing the
+    measurement); None whenever anything is missing or out of line, in which case the caller keeps the ratio
+    recorded under profiles/. The parent must hold no large device allocation while the children run."""
+    import csv
+    import glob
+    import shutil
+    import subprocess
+    import tempfile
+    note = {"source": "rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, one child run of this file each, in this run"}
+    if not shutil.which("rocprofv3"):
+        note["skipped"] = "rocprofv3 is not on PATH"
+        return None, note
+    if any("rocprof" in os.environ.get(k, "") for k in ("LD_PRELOAD", "ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB")):
+        note["skipped"] = "this process already runs under a profiler"
+        return None, note
+    csv.field_size_limit(1 << 30)
+    tmp = tempfile.mkdtemp(prefix="bikv_traffic_", dir="/tmp")
+    env = dict(os.environ, TMPDIR="/tmp")
+    means = {}
+    try:
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            d = os.path.join(tmp, counter)
+            cmd = ["timeout", "-s", "KILL", str(limit_s), "rocprofv3", "--pmc", counter, "--output-format", "csv",
+                   "-d", d, "-o", "c", "--", sys.executable, os.path.abspath(__file__), "--workload", workload,
+                   "--steps", "3", "--warmup", "1", "--no-cpu-baseline", "--no-other-layout", "--no-configs",
+                   "--no-staging", "--no-live-traffic"]
+            t0 = time.time()
+            r = subprocess.run(cmd, cwd="/tmp", env=env, stdout=subprocess.PIPE, stderr=subprocess.PIPE)
+            note[f"{counter}_run_s"] = round(time.time() - t0, 1)
+            if r.returncode != 0:
+                note["skipped"] = f"the {counter} run ended with status {r.returncode}"
+                return None, note
+            hits = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+            if not hits:
+                note["skipped"] = f"the {counter} run left no counter file"
+                return None, note
+            per = {}
+            with open(hits[0]) as fh:
+                for row in csv.DictReader(fh):
+                    if row["Counter_Name"] != counter:
+                        continue
+                    k = "copy" if "bikv::copy_runs_wave_kernel" in row["Kernel_Name"] else (
+                        "dominant" if dominant_kernel in row["Kernel_Name"] else None)
+                    if k:
+                        per.setdefault(k, {}).setdefault(row["Dispatch_Id"], 0.0)
+                        per[k][row["Dispatch_Id"]] += float(row["Counter_Value"])
+            if "copy" not in per or "dominant" not in per:
+                note["skipped"] = f"the {counter} run holds no dispatch of the calibration copy or of {dominant_kernel}"
+                return None, note
+            means[counter] = {k: (len(v), sum(v.values()) / len(v)) for k, v in per.items()}
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    kib = (2 << 30) / 1024.0                   # the calibration copy reads 2 GiB and writes 2 GiB
+    fscale = kib / means["FETCH_SIZE"]["copy"][1]
+    wscale = kib / means["WRITE_SIZE"]["copy"][1]
+    fetched = means["FETCH_SIZE"]["dominant"][1] * fscale * 1024
+    written = means["WRITE_SIZE"]["dominant"][1] * wscale * 1024
+    note.update({"kernel": dominant_kernel, "dispatches": means["FETCH_SIZE"]["dominant"][0],
+                 "fetch_scale_from_plain_copy": round(fscale, 5), "write_scale_from_plain_copy": round(wscale, 5),
+                 "fetched_bytes": round(fetched), "written_bytes": round(written),
+                 "ratio_to_algorithmic": round((fetched + written) / alg_bytes, 4)})
+    if not (0.5 < fscale < 4 and 0.5 < wscale < 4 and 0.5 < (fetched + written) / alg_bytes < 3):
+        note["skipped"] = "the counters are out of line with the calibration copy"
+        return None, note
+    return round(fetched + written), note
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -106,6 +183,9 @@ def parse_args():
     ap.add_argument("--staging-alloc", dest="staging_alloc", choices=["torch", "spread", "auto"], default="auto",
                     help="where the dense staging buffers come from: torch, bikv_device_alloc, or auto = the buffer a "
                          "gather WRITES from bikv_device_alloc, the buffer a scatter only reads from torch")
+    ap.add_argument("--no-live-traffic", dest="no_live_traffic", action="store_true",
+                    help="do not run the two rocprofv3 --pmc child processes that measure the dominant kernel's HBM "
+                         "traffic at the end of the default run (roofline.traffic then comes from the recorded ratio)")
     ap.add_argument("--no-configs", dest="no_configs", action="store_true",
                     help="skip the other named configurations (default workload only)")
     ap.add_argument("--no-staging", dest="no_staging", action="store_true",
@@ -1381,6 +1461,25 @@ def main():
     if not args.no_cpu_baseline:
         log("timing the CPU baseline")
         out["cpu_baseline"] = cpu_baseline(shape, wl)
+    if default_run and not args.no_live_traffic:
+        # the dominant kernel's HBM traffic, measured now (every measurement above is finished and its memory freed)
+        import gc
+        gc.collect()
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+        free_b, _ = torch.cuda.mem_get_info()
+        rf = out["roofline"]
+        if free_b < (150 << 30):
+            rf["traffic_live"] = {"skipped": f"only {free_b / 2**30:.0f} GiB of device memory free for the child runs"}
+        else:
+            log("measuring the dominant kernel's HBM traffic (two rocprofv3 --pmc child runs)")
+            dom = "tile_move_wave_kernel<0" if "gather" in rf["kernel"] else "tile_move_wave_kernel<1"
+            live, note = measure_traffic_live(args.workload, dom, rf["alg_bytes_per_launch"])
+            rf["traffic_live"] = note
+            if live is not None:
+                rf["traffic_from_recorded_ratio"] = rf["traffic"]
+                rf["traffic"] = live
+                rf["traffic_source"] = note["source"]
     if default_run:
         add_summary(out)
     emit(out)
