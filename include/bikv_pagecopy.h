@@ -214,7 +214,9 @@ int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* batch,
  * with an HBM buffer of chunks_per_launch * chunk_bytes. Launch k runs on lane k % n_buffers: one
  * gather kernel fills the lane's buffer with the next contiguous piece of the staging image, then one
  * hipMemcpyAsync per chunk_bytes moves it to `host_dst`, all in the lane's stream order, so the copies
- * of one lane overlap the kernel (and queued copies) of the others.
+ * of one lane overlap the kernel (and queued copies) of the others. Two lanes are enough to keep the
+ * link busy; a HIP process has 4 hardware queues by default (GPU_MAX_HW_QUEUES) and its streams are dealt
+ * onto them in turn, so a fourth lane shares a queue with another lane and runs in turn with it.
  *
  * `req_pages` (HOST array, n_requests entries) gives the number of pages of each request; pages of
  * request r occupy batch entries [sum(req_pages[:r]), +req_pages[r]) and, in staging, a contiguous
