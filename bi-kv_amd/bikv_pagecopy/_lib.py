@@ -172,6 +172,8 @@ _SIGNATURES = {
     "bikv_device_alloc_bounded": (C.c_int, [C.c_int, C.c_int64, C.c_int32, C.c_int64, C.POINTER(C.c_void_p)]),
     "bikv_device_free": (C.c_int, [C.c_void_p]),
     "bikv_device_alloc_info": (C.c_int, [C.c_void_p, C.POINTER(AllocInfo)]),
+    "bikv_torch_alloc": (C.c_void_p, [C.c_int64, C.c_int, C.c_void_p]),
+    "bikv_torch_free": (None, [C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
     "bikv_host_alloc": (C.c_int, [C.c_int64, C.POINTER(C.c_void_p)]),
     "bikv_host_free": (C.c_int, [C.c_void_p]),
     "bikv_consumer_init": (C.c_int, [C.c_int, C.c_char_p, C.c_size_t]),

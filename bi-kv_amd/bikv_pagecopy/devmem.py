@@ -7,6 +7,7 @@ scattered into it: the address space behaves as two halves, and random writes co
 alternate between the halves; `.tensor` is a torch view of it (uint8, or reshaped / re-typed by the
 caller) that kernels, torch ops and this library treat like any device tensor.
 """
+import contextlib
 import ctypes as C
 
 import torch
@@ -71,3 +72,44 @@ def device_empty(nbytes: int, device, spread: bool = True, max_filler_bytes: int
     """A uint8 device tensor of `nbytes` whose memory came from bikv_device_alloc; it is released when the
     last tensor that views it is gone and the collector has run."""
     return DeviceBuffer(nbytes, device, spread, max_filler_bytes).tensor
+
+
+_PLACED_POOL = {}
+
+
+def placed_mem_pool(device=None):
+    """A torch.cuda.MemPool (one per device, created on first use) whose segments come from
+    bikv_device_alloc instead of hipMalloc. Every segment is a whole number of chunks of at least 256 MiB
+    and is placed with a timed probe, so the pool is meant for the few large KV allocations of a process,
+    not for its everyday tensors."""
+    idx = None if device is None else torch.device(device).index
+    if idx is None:
+        idx = torch.cuda.current_device()
+    if idx not in _PLACED_POOL:
+        _lib.load()         # fails loudly when the library has not been built
+        alloc = torch.cuda.memory.CUDAPluggableAllocator(_lib.LIB_PATH, "bikv_torch_alloc", "bikv_torch_free")
+        pool = torch.cuda.MemPool(alloc.allocator())
+        # The pool and its allocator live until the process ends and are never torn down: destroying them while
+        # the interpreter finalises releases segments through objects that may already be gone. One extra
+        # reference each keeps their destructors from ever running; the driver reclaims the memory at exit.
+        for obj in (pool, alloc, alloc.allocator()):
+            C.pythonapi.Py_IncRef(C.py_object(obj))
+        _PLACED_POOL[idx] = (pool, alloc)
+    return _PLACED_POOL[idx][0]
+
+
+@contextlib.contextmanager
+def placed_allocations(device=None):
+    """Inside this context torch's allocations on `device` come from bikv_device_alloc, so a caller keeps its
+    own allocation code — the reference's `torch.empty((cache_size,) + token_shape, ...)` of
+    Bi-KV/DistributedStorage/kvcache.py:38-43 or the per-layer `torch.zeros` of Bi-KV/Worker/Worker.py:74-78 —
+    and still gets pools spread over both halves of HBM:
+
+        with bikv_pagecopy.placed_allocations("cuda:0"):
+            self.local_kvcache = [torch.zeros(...) for _ in range(num_layers)]
+
+    Allocate only the pools here: every request torch passes on is rounded up to whole 256 MiB chunks.
+    The memory returns to the pool when its tensors die and to the device when the process ends."""
+    pool = placed_mem_pool(device)
+    with torch.cuda.use_mem_pool(pool, device=device):
+        yield pool

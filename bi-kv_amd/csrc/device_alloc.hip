@@ -22,6 +22,8 @@
 #include "pagecopy_internal.h"
 
 #include <algorithm>
+#include <atomic>
+#include <cstdlib>
 #include <cerrno>
 #include <chrono>
 #include <cstdio>
@@ -418,6 +420,28 @@ extern "C" int bikv_device_free(void* p) {
   if (e != hipSuccess) return fail_hip(e, "hipMemUnmap");
   if (e2 != hipSuccess) return fail_hip(e2, "hipMemAddressFree");
   return BIKV_OK;
+}
+
+// Entry points with the signatures torch.cuda.memory.CUDAPluggableAllocator binds, so that a torch memory pool
+// (torch.cuda.MemPool) can take its segments from bikv_device_alloc and the reference's torch.empty call sites
+// (kvcache.py:38-43, Worker.py:74-78) stay as they are. A null return makes torch report out-of-memory.
+// torch releases what its pools still hold while the process exits, when this library's bookkeeping and the
+// HIP runtime may already be gone; from the first exit handler on, releasing is left to the driver.
+static std::atomic<bool> g_exiting{false};
+static void mark_exiting() { g_exiting.store(true); }
+
+extern "C" void* bikv_torch_alloc(int64_t size, int device, void* /*stream*/) {
+  static std::once_flag once;
+  std::call_once(once, [] { atexit(mark_exiting); });   // registered late, so it runs before any static destructor
+  if (size <= 0 || g_exiting.load()) return nullptr;
+  void* p = nullptr;
+  if (bikv_device_alloc(device, size, BIKV_PLACE_SPREAD, &p) != BIKV_OK) return nullptr;
+  return p;
+}
+
+extern "C" void bikv_torch_free(void* p, size_t /*size*/, int /*device*/, void* /*stream*/) {
+  if (g_exiting.load()) return;
+  (void)bikv_device_free(p);
 }
 
 extern "C" int bikv_device_alloc_info(const void* p, bikv_alloc_info* info) {

@@ -391,6 +391,13 @@ int bikv_device_alloc(int device, int64_t bytes, int32_t placement, void** out);
 int bikv_device_alloc_bounded(int device, int64_t bytes, int32_t placement, int64_t max_filler_bytes, void** out);
 int bikv_device_free(void* p);
 int bikv_device_alloc_info(const void* p, bikv_alloc_info* info);
+/* The same allocator behind the two function signatures torch.cuda.memory.CUDAPluggableAllocator binds
+ * (alloc(size, device, stream) / free(ptr, size, device, stream); BIKV_PLACE_SPREAD, the default filler
+ * budget; null on failure, which torch reports as out of memory). A torch.cuda.MemPool built on them lets
+ * the reference's own torch.empty call sites (kvcache.py:38-43, Worker.py:74-78) produce placed pools;
+ * every segment torch asks for is at least one chunk (256 MiB), so use such a pool for the KV pools only. */
+void* bikv_torch_alloc(int64_t size, int device, void* stream);   /* ssize_t on the caller's side */
+void bikv_torch_free(void* p, size_t size, int device, void* stream);
 
 /* Pinned host memory (hipHostMalloc, mapped + portable). */
 int bikv_host_alloc(int64_t bytes, void** out);

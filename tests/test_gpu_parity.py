@@ -835,6 +835,54 @@ def test_device_alloc_builds_a_pool_out_of_chunks_from_both_halves(bk, oracle, c
     assert b"out of device memory" in lib.bikv_last_error()
 
 
+def test_torch_allocations_inside_placed_allocations_come_from_device_alloc(bk, oracle, cuda, lib):
+    """The reference's own allocation code, unchanged — per-layer torch.zeros([blocks*block, 2, heads, dim]) as in
+    Worker/Worker.py:74-78 — run inside bk.placed_allocations(): torch's memory pool takes each segment from
+    bikv_device_alloc (the library knows the pointers), the tensors behave like any others, and the movers gather
+    from and scatter into them against the oracle. A tensor allocated outside the context is torch's own."""
+    import ctypes as C
+    from bikv_pagecopy import _lib
+    _announce("torch memory pool on bikv_device_alloc")
+    P, H, D, L, blocks = 16, 2, 128, 3, 40000          # 3 layers of 312.5 MiB: each its own segment of two chunks
+    with bk.placed_allocations(cuda):
+        layers_d = [torch.zeros(blocks * P, 2, H, D, dtype=torch.float16, device=cuda) for _ in range(L)]
+    outside = torch.zeros(blocks * P, 2, H, D, dtype=torch.float16, device=cuda)
+    info = _lib.AllocInfo()
+    for t in layers_d:
+        assert lib.bikv_device_alloc_info(C.c_void_p(t.data_ptr()), C.byref(info)) == _lib.OK, lib.bikv_last_error()
+        assert info.bytes >= t.numel() * 2 and info.n_chunks >= 2 and info.chunk_bytes >= 256 << 20
+        assert int(t.abs().sum().item()) == 0
+    assert lib.bikv_device_alloc_info(C.c_void_p(outside.data_ptr()), C.byref(info)) == _lib.EINVAL
+    rng = np.random.default_rng(977)
+    used = np.unique(np.concatenate([rng.integers(0, blocks, size=60), [0, blocks - 1, (256 << 20) // (P * 2 * H * D * 2)]]))
+    rows_h = rng.integers(0, 65536, size=(L, len(used), P, 2, H, D), dtype=np.uint16)
+    for l in range(L):
+        v = layers_d[l].view(torch.int16).view(blocks, P, 2, H, D)
+        v[torch.from_numpy(used).to(cuda)] = torch.from_numpy(rows_h[l].view(np.int16)).to(cuda)
+    pool = bk.PagedKVPool.from_token_kv_layers(layers_d, P)
+    # the oracle works on the used blocks only, renumbered
+    small = [rows_h[l].reshape(len(used) * P, 2, H, D) for l in range(L)]
+    planes_h = oracle.planes_of_token_kv_layers(small, P).view(np.uint8)
+    pick = rng.permutation(len(used))
+    reqs_small = [pick[:25], pick[25:31], np.array([0, 0])]
+    reqs = [used[r] for r in reqs_small]
+    batch = pool.make_batch(reqs, "layer_major")
+    st, _ = pool.gather(batch)
+    pool.check()
+    assert _to_np(st).tobytes() == oracle.gather_layered_c(planes_h, reqs_small, "layer_major").tobytes()
+    fresh = np.setdiff1d(np.arange(blocks), used)[rng.permutation(blocks - len(used))[:33]]
+    sb = pool.make_batch([fresh[:25], fresh[25:31], fresh[31:33]], "layer_major", check_unique=True)
+    pool.scatter(sb, st)
+    pool.check()
+    moved = np.concatenate(reqs)
+    for l in range(L):
+        v = layers_d[l].view(torch.int16).view(blocks, P, 2, H, D)
+        assert torch.equal(v[torch.from_numpy(fresh).to(cuda)], v[torch.from_numpy(moved).to(cuda)]), f"layer {l}"
+    pool.close()
+    del layers_d, v, st
+    torch.cuda.synchronize(cuda)
+
+
 # ---- several host threads -----------------------------------------------------------------------
 def test_four_host_threads_move_pages_through_one_pool(bk, oracle, cuda):
     """The reference's callers are thread pools (20 gRPC workers per process, config.yml:53,60). Four host
