@@ -1262,6 +1262,10 @@ def run_layout_change(args, bk, dev, blocks=None, sort=False, pool_alloc=None):
     if pool_alloc == "spread":
         arena = spread_empty(bk, L * blocks * P * 2 * H * D * 2, dev, "layer tensors")
         layers = list(arena.view(torch.float16).view(L, blocks * P, 2, H, D).unbind(0))
+    elif pool_alloc == "placed_torch":
+        # the reference's own allocation code (one torch tensor per layer), inside the library's torch memory pool
+        with bk.placed_allocations(dev):
+            layers = [torch.empty((blocks * P, 2, H, D), dtype=torch.float16, device=dev) for _ in range(L)]
     else:
         layers = [torch.empty((blocks * P, 2, H, D), dtype=torch.float16, device=dev) for _ in range(L)]
     for t in layers:
@@ -1269,7 +1273,7 @@ def run_layout_change(args, bk, dev, blocks=None, sort=False, pool_alloc=None):
     pool = bk.NHDPool.from_token_kv_layers(layers, P)
     tm = torch.empty((n_pages, P, D, H, L, 2), dtype=torch.float16, device=dev)
     fill_random_bytes(tm)
-    if pool_alloc == "spread" and args.staging_alloc in ("auto", "spread"):   # the written image, like a gather's
+    if pool_alloc in ("spread", "placed_torch") and args.staging_alloc in ("auto", "spread"):   # the written image, like a gather's
         tm_out = spread_empty(bk, tm.numel() * 2, dev, "token-major image written by the store").view(torch.float16).view(tm.shape)
     else:
         tm_out = torch.empty_like(tm)
@@ -1326,7 +1330,8 @@ def run_layout_change(args, bk, dev, blocks=None, sort=False, pool_alloc=None):
                                f"{n_pages} pages of {P} tokens loaded then stored per step, random blocks"
                                f"{'; the load walks them in ascending block order' if sort else ''}",
                    "pool_GB": round(L * blocks * P * 2 * H * D * 2 / 1e9, 2),
-                   "pool_alloc": "bikv_device_alloc (chunks alternating between the halves of HBM)" if pool_alloc == "spread" else "torch"},
+                   "pool_alloc": {"spread": "bikv_device_alloc (chunks alternating between the halves of HBM)",
+                                  "placed_torch": "28 torch.empty calls inside bikv_pagecopy.placed_allocations()"}.get(pool_alloc, "torch")},
         "timed_region_s": round(wall, 3),
         "pct_of_hbm_peak": round(100 * 2 * alg / (wall / args.steps) / 1e9 / HBM_PEAK_GBPS, 2),
         "pages_per_s": round(2 * n_pages / (wall / args.steps), 1), "bit_exact": True,
@@ -1391,6 +1396,7 @@ def main():
         out = run_layout_change(args, bk, dev)
         if not args.pool_pages:
             for key, kw in (("torch_alloc", dict(pool_alloc="stacked")), ("torch_alloc_sorted_load", dict(pool_alloc="stacked", sort=True)),
+                            ("torch_alloc_inside_placed_allocations", dict(pool_alloc="placed_torch")),
                             ("pool_163840_blocks", dict(blocks=163840))):
                 o = run_layout_change(args, bk, dev, **kw)
                 out[key] = {"workload": o["config"]["workload"], "pool_GB": o["config"]["pool_GB"], "value": o["value"],

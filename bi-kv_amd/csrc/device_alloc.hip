@@ -18,6 +18,7 @@
 // half) and maps them alternately into one virtual range (hipMemAddressReserve / hipMemMap). Every
 // window of such a pool, however small, then spreads its writes over both halves.
 #include "../../include/bikv_pagecopy.h"
+#include "host_logic/arena_logic.h"
 #include "host_logic/host_checks.h"
 #include "pagecopy_internal.h"
 
@@ -424,7 +425,21 @@ extern "C" int bikv_device_free(void* p) {
 
 // Entry points with the signatures torch.cuda.memory.CUDAPluggableAllocator binds, so that a torch memory pool
 // (torch.cuda.MemPool) can take its segments from bikv_device_alloc and the reference's torch.empty call sites
-// (kvcache.py:38-43, Worker.py:74-78) stay as they are. A null return makes torch report out-of-memory.
+// (kvcache.py:38-43, Worker.py:74-78) stay as they are. Segments of up to 1 GiB are carved, one after the other,
+// out of placed arenas of 2 GiB (host_logic/arena_logic.h), so that a pool made of many tensors smaller than a
+// chunk still alternates between the halves; larger ones are placements of their own. A null return makes
+// torch report out-of-memory.
+constexpr int64_t kTorchArenaBytes = int64_t(2) << 30;
+static void* torch_backend_alloc(int device, int64_t bytes) {
+  void* p = nullptr;
+  return bikv_device_alloc(device, bytes, BIKV_PLACE_SPREAD, &p) == BIKV_OK ? p : nullptr;
+}
+static void torch_backend_free(void* base) { (void)bikv_device_free(base); }
+static arena::Book& torch_book() {
+  static arena::Book* book = new arena::Book(kTorchArenaBytes, torch_backend_alloc, torch_backend_free);   // never destroyed
+  return *book;
+}
+
 // torch releases what its pools still hold while the process exits, when this library's bookkeeping and the
 // HIP runtime may already be gone; from the first exit handler on, releasing is left to the driver.
 static std::atomic<bool> g_exiting{false};
@@ -434,21 +449,23 @@ extern "C" void* bikv_torch_alloc(int64_t size, int device, void* /*stream*/) {
   static std::once_flag once;
   std::call_once(once, [] { atexit(mark_exiting); });   // registered late, so it runs before any static destructor
   if (size <= 0 || g_exiting.load()) return nullptr;
-  void* p = nullptr;
-  if (bikv_device_alloc(device, size, BIKV_PLACE_SPREAD, &p) != BIKV_OK) return nullptr;
-  return p;
+  return torch_book().take(device, size);
 }
 
 extern "C" void bikv_torch_free(void* p, size_t /*size*/, int /*device*/, void* /*stream*/) {
   if (g_exiting.load()) return;
-  (void)bikv_device_free(p);
+  (void)torch_book().give(p);
 }
 
 extern "C" int bikv_device_alloc_info(const void* p, bikv_alloc_info* info) {
   if (!p || !info) return fail(BIKV_EINVAL, "null argument");
   std::lock_guard<std::mutex> lk(g_mu);
-  auto it = g_allocs.find(const_cast<void*>(p));
-  if (it == g_allocs.end()) return fail(BIKV_EINVAL, "pointer was not returned by bikv_device_alloc");
+  // any address inside an allocation names it (tensors carved out of an arena start past its base)
+  auto it = g_allocs.upper_bound(const_cast<void*>(p));
+  if (it == g_allocs.begin()) return fail(BIKV_EINVAL, "address is not inside memory from bikv_device_alloc");
+  --it;
+  if (static_cast<const char*>(p) >= static_cast<const char*>(it->first) + it->second.bytes)
+    return fail(BIKV_EINVAL, "address is not inside memory from bikv_device_alloc");
   info->bytes = (int64_t)it->second.bytes;
   info->chunk_bytes = (int64_t)it->second.chunk;
   info->n_chunks = (int32_t)it->second.handles.size();

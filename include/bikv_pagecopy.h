@@ -395,7 +395,10 @@ int bikv_device_alloc_info(const void* p, bikv_alloc_info* info);
  * (alloc(size, device, stream) / free(ptr, size, device, stream); BIKV_PLACE_SPREAD, the default filler
  * budget; null on failure, which torch reports as out of memory). A torch.cuda.MemPool built on them lets
  * the reference's own torch.empty call sites (kvcache.py:38-43, Worker.py:74-78) produce placed pools;
- * every segment torch asks for is at least one chunk (256 MiB), so use such a pool for the KV pools only. */
+ * segments of up to 1 GiB are carved one after the other out of placed arenas of 2 GiB (so a pool made of
+ * many tensors smaller than a chunk still alternates between the halves), larger ones are placements of
+ * their own; use such a pool for the KV pools only. bikv_device_alloc_info accepts any address inside a
+ * placed allocation. */
 void* bikv_torch_alloc(int64_t size, int device, void* stream);   /* ssize_t on the caller's side */
 void bikv_torch_free(void* p, size_t size, int device, void* stream);
 

@@ -4,9 +4,12 @@
 #include <cstdlib>
 #include <cstring>
 #include <limits>
+#include <map>
 #include <random>
 #include <vector>
+#include <sys/mman.h>
 
+#include "arena_logic.h"
 #include "chunk_planner.h"
 #include "host_checks.h"
 #include "ring_logic.h"
@@ -182,7 +185,104 @@ static void test_ring() {
   free(c);
 }
 
+// The arena bookkeeping behind the torch allocator hooks, over a malloc backend: blocks never overlap, stay
+// inside what the backend handed out, follow each other in memory in allocation order, big requests get
+// allocations of their own, and everything the backend gave is returned once the last block is gone.
+static std::map<void*, int64_t> g_backend;      // base -> bytes, what the backend currently has out
+static int g_backend_fail_after = -1;
+static void* backend_alloc(int /*device*/, int64_t bytes) {
+  if (g_backend_fail_after == 0) return nullptr;
+  if (g_backend_fail_after > 0) --g_backend_fail_after;
+  // address space only: the bookkeeping compares addresses and never touches the memory
+  void* p = mmap(nullptr, (size_t)bytes, PROT_NONE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+  REQUIRE(p != MAP_FAILED, "mmap of %lld bytes of address space", (long long)bytes);
+  g_backend[p] = bytes;
+  return p;
+}
+static void backend_drop(void* base) {
+  munmap(base, (size_t)g_backend[base]);
+  g_backend.erase(base);
+}
+static void backend_free(void* base) {
+  REQUIRE(g_backend.count(base) == 1, "release of %p, which the backend did not hand out", base);
+  backend_drop(base);
+}
+static void backend_drop_all() {
+  while (!g_backend.empty()) backend_drop(g_backend.begin()->first);
+}
+static void test_arena() {
+  const int64_t A = int64_t(2) << 30;
+  {
+    arena::Book book(A, backend_alloc, backend_free);
+    std::vector<void*> p;
+    for (int i = 0; i < 28; ++i) p.push_back(book.take(0, int64_t(160) << 20));       // the Worker's 28 layer tensors
+    for (void* q : p) REQUIRE(q != nullptr, "take failed");
+    REQUIRE(book.live_arenas() == 3 && g_backend.size() == 3, "28 x 160 MiB fill three arenas of 2 GiB, got %zu", book.live_arenas());
+    for (int i = 1; i < 12; ++i)
+      REQUIRE((char*)p[(size_t)i] - (char*)p[(size_t)i - 1] == (int64_t(160) << 20), "blocks of one arena are neighbours");
+    void* big = book.take(0, (int64_t(1) << 30) + 1);
+    REQUIRE(big && g_backend.size() == 4, "a request above half an arena is an allocation of its own");
+    void* other_dev = book.take(1, int64_t(2) << 20);
+    REQUIRE(other_dev && g_backend.size() == 5, "another device gets its own arena");
+    REQUIRE(!book.give((char*)p[0] + 4096), "an address inside a block is not a block");
+    for (int i = 0; i < 12; ++i) REQUIRE(book.give(p[(size_t)i]), "give");
+    REQUIRE(g_backend.size() == 4, "an older arena is released with its last block");
+    REQUIRE(!book.give(p[0]), "a block is given back once");
+    for (int i = 12; i < 28; ++i) REQUIRE(book.give(p[(size_t)i]), "give");
+    REQUIRE(book.give(big) && book.give(other_dev), "give");
+    REQUIRE(book.live_blocks() == 0, "no block left");
+    // the newest arena of each device is rewound and kept
+    REQUIRE(g_backend.size() == 2 && book.live_arenas() == 2, "kept arenas: %zu", g_backend.size());
+    void* again = book.take(0, int64_t(4) << 20);
+    REQUIRE(again && g_backend.size() == 2, "a kept arena serves the next request");
+    REQUIRE(book.give(again), "give");
+    backend_drop_all();
+  }
+  {
+    // random traffic: blocks are disjoint and inside a backend allocation
+    arena::Book book(A, backend_alloc, backend_free);
+    std::mt19937_64 rng(7);
+    std::map<char*, int64_t> live;
+    for (int step = 0; step < 4000; ++step) {
+      if (live.empty() || rng() % 3) {
+        const int64_t sz = (int64_t)(rng() % 700 + 1) << 20;
+        char* q = (char*)book.take(0, sz);
+        REQUIRE(q != nullptr, "take");
+        const int64_t r = arena::round_up(sz, arena::kAlign);
+        bool inside = false;
+        for (auto& b : g_backend) inside |= q >= (char*)b.first && q + r <= (char*)b.first + b.second;
+        REQUIRE(inside, "block outside every backend allocation");
+        auto nx = live.lower_bound(q);
+        REQUIRE(nx == live.end() || q + r <= nx->first, "block overlaps its successor");
+        if (nx != live.begin()) { --nx; REQUIRE(nx->first + nx->second <= q, "block overlaps its predecessor"); }
+        live[q] = r;
+      } else {
+        auto it = live.begin();
+        std::advance(it, (long)(rng() % live.size()));
+        REQUIRE(book.give(it->first), "give");
+        live.erase(it);
+      }
+    }
+    for (auto& b : live) REQUIRE(book.give(b.first), "give");
+    REQUIRE(book.live_blocks() == 0 && g_backend.size() <= 1, "all but the kept arena returned");
+    backend_drop_all();
+  }
+  {
+    // the backend running dry: take reports it and leaves nothing behind
+    arena::Book book(A, backend_alloc, backend_free);
+    g_backend_fail_after = 1;
+    void* a = book.take(0, int64_t(900) << 20);
+    void* b = book.take(0, int64_t(900) << 20);
+    void* c = book.take(0, int64_t(900) << 20);     // needs a second arena: refused
+    REQUIRE(a && b && !c && book.live_blocks() == 2, "out of memory is reported");
+    g_backend_fail_after = -1;
+    REQUIRE(book.give(a) && book.give(b), "give");
+    backend_drop_all();
+  }
+}
+
 int main() {
+  test_arena();
   test_planner();
   test_duplicates();
   test_interleave();

@@ -843,16 +843,24 @@ def test_torch_allocations_inside_placed_allocations_come_from_device_alloc(bk, 
     import ctypes as C
     from bikv_pagecopy import _lib
     _announce("torch memory pool on bikv_device_alloc")
-    P, H, D, L, blocks = 16, 2, 128, 3, 40000          # 3 layers of 312.5 MiB: each its own segment of two chunks
+    P, H, D, L, blocks = 16, 2, 128, 3, 40000          # 3 layers of 312.5 MiB
     with bk.placed_allocations(cuda):
         layers_d = [torch.zeros(blocks * P, 2, H, D, dtype=torch.float16, device=cuda) for _ in range(L)]
+        big = torch.empty((1 << 30) + (64 << 20), dtype=torch.uint8, device=cuda)       # above half an arena: on its own
     outside = torch.zeros(blocks * P, 2, H, D, dtype=torch.float16, device=cuda)
     info = _lib.AllocInfo()
     for t in layers_d:
+        # any address inside a placed allocation names it; the three layers were carved out of one 2 GiB arena,
+        # one after the other
         assert lib.bikv_device_alloc_info(C.c_void_p(t.data_ptr()), C.byref(info)) == _lib.OK, lib.bikv_last_error()
-        assert info.bytes >= t.numel() * 2 and info.n_chunks >= 2 and info.chunk_bytes >= 256 << 20
+        assert info.bytes == 2 << 30 and info.n_chunks >= 2 and info.chunk_bytes >= 256 << 20
         assert int(t.abs().sum().item()) == 0
+    seg = -(-layers_d[0].numel() * 2 // (2 << 20)) * (2 << 20)
+    assert [t.data_ptr() - layers_d[0].data_ptr() for t in layers_d] == [0, seg, 2 * seg]
+    assert lib.bikv_device_alloc_info(C.c_void_p(big.data_ptr()), C.byref(info)) == _lib.OK and info.bytes >= big.numel()
+    assert not (layers_d[0].data_ptr() <= big.data_ptr() < layers_d[0].data_ptr() + (2 << 30))
     assert lib.bikv_device_alloc_info(C.c_void_p(outside.data_ptr()), C.byref(info)) == _lib.EINVAL
+    del big
     rng = np.random.default_rng(977)
     used = np.unique(np.concatenate([rng.integers(0, blocks, size=60), [0, blocks - 1, (256 << 20) // (P * 2 * H * D * 2)]]))
     rows_h = rng.integers(0, 65536, size=(L, len(used), P, 2, H, D), dtype=np.uint16)
