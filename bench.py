@@ -92,6 +92,44 @@ def traffic_ratio(workload, kind):
     return r, TRAFFIC_SOURCE
 
 
+def counter_means(csv_path, counter, dominant_kernel):
+    """Mean per dispatch of `counter` in a rocprofv3 counter_collection.csv, for the plain-copy calibration
+    kernel ("copy") and for the kernels whose name contains `dominant_kernel` ("dominant"): {key: (dispatches,
+    mean)}. A dispatch's rows (one per counter instance) are summed."""
+    import csv
+    csv.field_size_limit(1 << 30)
+    per = {}
+    with open(csv_path) as fh:
+        for row in csv.DictReader(fh):
+            if row["Counter_Name"] != counter:
+                continue
+            k = "copy" if "bikv::copy_runs_wave_kernel" in row["Kernel_Name"] else (
+                "dominant" if dominant_kernel in row["Kernel_Name"] else None)
+            if k:
+                per.setdefault(k, {}).setdefault(row["Dispatch_Id"], 0.0)
+                per[k][row["Dispatch_Id"]] += float(row["Counter_Value"])
+    return {k: (len(v), sum(v.values()) / len(v)) for k, v in per.items()}
+
+
+def traffic_from_counters(fetch, write, alg_bytes, copy_bytes=2 << 30):
+    """HBM bytes per launch of the dominant kernel from the two counters' means (counter_means): FETCH_SIZE and
+    WRITE_SIZE count KiB in units that differ between the two, so each is scaled by what it reads for the plain
+    copy of `copy_bytes` each way. Returns (bytes or None, details)."""
+    kib = copy_bytes / 1024.0
+    fscale = kib / fetch["copy"][1]
+    wscale = kib / write["copy"][1]
+    fetched = fetch["dominant"][1] * fscale * 1024
+    written = write["dominant"][1] * wscale * 1024
+    note = {"dispatches": fetch["dominant"][0],
+            "fetch_scale_from_plain_copy": round(fscale, 5), "write_scale_from_plain_copy": round(wscale, 5),
+            "fetched_bytes": round(fetched), "written_bytes": round(written),
+            "ratio_to_algorithmic": round((fetched + written) / alg_bytes, 4)}
+    if not (0.5 < fscale < 4 and 0.5 < wscale < 4 and 0.5 < (fetched + written) / alg_bytes < 3):
+        note["skipped"] = "the counters are out of line with the calibration copy"
+        return None, note
+    return round(fetched + written), note
+
+
 def measure_traffic_live(workload, dominant_kernel, alg_bytes, limit_s=150):
     """HBM bytes per launch of `dominant_kernel`, measured now: this file is run twice more as a child process
     under `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE; one counter per run), on the same workload at full size
@@ -99,19 +137,18 @@ def measure_traffic_live(workload, dominant_kernel, alg_bytes, limit_s=150):
     reads for the plain 2 GiB copy the child also launches. Returns (bytes or None, dict describing the
     measurement); None whenever anything is missing or out of line, in which case the caller keeps the ratio
     recorded under profiles/. The parent must hold no large device allocation while the children run."""
-    import csv
     import glob
     import shutil
     import subprocess
     import tempfile
-    note = {"source": "rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, one child run of this file each, in this run"}
+    note = {"source": "rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, one child run of this file each, in this run",
+            "kernel": dominant_kernel}
     if not shutil.which("rocprofv3"):
         note["skipped"] = "rocprofv3 is not on PATH"
         return None, note
     if any("rocprof" in os.environ.get(k, "") for k in ("LD_PRELOAD", "ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB")):
         note["skipped"] = "this process already runs under a profiler"
         return None, note
-    csv.field_size_limit(1 << 30)
     tmp = tempfile.mkdtemp(prefix="bikv_traffic_", dir="/tmp")
     env = dict(os.environ, TMPDIR="/tmp")
     means = {}
@@ -132,35 +169,15 @@ def measure_traffic_live(workload, dominant_kernel, alg_bytes, limit_s=150):
             if not hits:
                 note["skipped"] = f"the {counter} run left no counter file"
                 return None, note
-            per = {}
-            with open(hits[0]) as fh:
-                for row in csv.DictReader(fh):
-                    if row["Counter_Name"] != counter:
-                        continue
-                    k = "copy" if "bikv::copy_runs_wave_kernel" in row["Kernel_Name"] else (
-                        "dominant" if dominant_kernel in row["Kernel_Name"] else None)
-                    if k:
-                        per.setdefault(k, {}).setdefault(row["Dispatch_Id"], 0.0)
-                        per[k][row["Dispatch_Id"]] += float(row["Counter_Value"])
-            if "copy" not in per or "dominant" not in per:
+            means[counter] = counter_means(hits[0], counter, dominant_kernel)
+            if "copy" not in means[counter] or "dominant" not in means[counter]:
                 note["skipped"] = f"the {counter} run holds no dispatch of the calibration copy or of {dominant_kernel}"
                 return None, note
-            means[counter] = {k: (len(v), sum(v.values()) / len(v)) for k, v in per.items()}
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
-    kib = (2 << 30) / 1024.0                   # the calibration copy reads 2 GiB and writes 2 GiB
-    fscale = kib / means["FETCH_SIZE"]["copy"][1]
-    wscale = kib / means["WRITE_SIZE"]["copy"][1]
-    fetched = means["FETCH_SIZE"]["dominant"][1] * fscale * 1024
-    written = means["WRITE_SIZE"]["dominant"][1] * wscale * 1024
-    note.update({"kernel": dominant_kernel, "dispatches": means["FETCH_SIZE"]["dominant"][0],
-                 "fetch_scale_from_plain_copy": round(fscale, 5), "write_scale_from_plain_copy": round(wscale, 5),
-                 "fetched_bytes": round(fetched), "written_bytes": round(written),
-                 "ratio_to_algorithmic": round((fetched + written) / alg_bytes, 4)})
-    if not (0.5 < fscale < 4 and 0.5 < wscale < 4 and 0.5 < (fetched + written) / alg_bytes < 3):
-        note["skipped"] = "the counters are out of line with the calibration copy"
-        return None, note
-    return round(fetched + written), note
+    live, details = traffic_from_counters(means["FETCH_SIZE"], means["WRITE_SIZE"], alg_bytes)
+    note.update(details)
+    return live, note
 
 
 def parse_args():

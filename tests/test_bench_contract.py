@@ -63,3 +63,39 @@ def test_summary_block_is_flat_complete_and_last():
     with contextlib.redirect_stdout(buf):
         bench.emit(out)
     assert list(json.loads(buf.getvalue()).keys())[-1] == "summary"
+
+
+def test_live_traffic_is_computed_from_the_two_counters_and_their_calibration(tmp_path):
+    """The figures `roofline.traffic` is made of when the run measures them itself: per-dispatch means of each
+    counter for the dominant kernel, each scaled by the same counter's reading for the plain 2 GiB copy. The
+    counter files here are written by hand in rocprofv3's column layout: FETCH_SIZE counting half the KiB a
+    kernel fetches (as on MI355X), WRITE_SIZE all of them, two instances per dispatch, other kernels in between."""
+    import bench
+    head = '"Correlation_Id","Dispatch_Id","Kernel_Name","Counter_Name","Counter_Value"\n'
+    kib = (2 << 30) // 1024
+    alg = 2 * 3 * (1 << 30)                                            # the kernel reads 3 GiB and writes 3 GiB
+    def rows(counter, copy_val, dom_val):
+        out, did = [], 0
+        for name, val, n in (("void bikv::copy_runs_wave_kernel<true, true, 64, true>(bikv::RunArgs)", copy_val, 3),
+                             ("void at::native::vectorized_elementwise_kernel<4>(int)", 12345.0, 2),
+                             ("void bikv::tile_move_wave_kernel<0, 2, 64>(bikv::MoveArgs)", dom_val, 4),
+                             ("void bikv::tile_move_wave_kernel<1, 2, 64>(bikv::MoveArgs)", 7.0, 4)):
+            for _ in range(n):
+                did += 1
+                for inst in range(2):                                   # two rows of one dispatch add up
+                    out.append(f'{did},{did},"{name}","{counter}",{val / 2}\n')
+                out.append(f'{did},{did},"{name}","SOME_OTHER_COUNTER",1.0\n')
+        return head + "".join(out)
+    f, w = tmp_path / "f.csv", tmp_path / "w.csv"
+    f.write_text(rows("FETCH_SIZE", kib / 2, 3 * (1 << 20) / 2 * 1.01))   # 1 % more fetched than the algorithm needs
+    w.write_text(rows("WRITE_SIZE", kib, 3 * (1 << 20)))
+    fm = bench.counter_means(str(f), "FETCH_SIZE", "tile_move_wave_kernel<0")
+    wm = bench.counter_means(str(w), "WRITE_SIZE", "tile_move_wave_kernel<0")
+    assert fm["copy"][0] == 3 and fm["dominant"][0] == 4 and abs(fm["copy"][1] - kib / 2) < 1e-6
+    live, note = bench.traffic_from_counters(fm, wm, alg)
+    assert abs(note["fetch_scale_from_plain_copy"] - 2.0) < 1e-9 and abs(note["write_scale_from_plain_copy"] - 1.0) < 1e-9
+    assert note["written_bytes"] == 3 << 30 and abs(note["fetched_bytes"] - 1.01 * (3 << 30)) < 2
+    assert live == note["fetched_bytes"] + note["written_bytes"] and note["ratio_to_algorithmic"] == 1.005
+    # counters that make no sense against the calibration are not reported
+    bad, note = bench.traffic_from_counters({"copy": (3, kib * 100.0), "dominant": fm["dominant"]}, wm, alg)
+    assert bad is None and "skipped" in note
