@@ -203,7 +203,6 @@ void release_all(std::vector<hipMemGenericAllocationHandle_t>& v) {
 // probed as a PAIR with the first chunk (equal footprint for every probe), and judged against the slowest
 // pair seen so far — pairs inside the first chunk's half. A time inside the band between the two groups is
 // not trusted: the chunk is probed again (twice more at most) and the median decides.
-constexpr float kOtherBelow = 0.92f;     // other half: pair time below 0.92 x the same-half pair time
 constexpr float kBandLo = 0.88f, kBandHi = 0.96f;
 
 }  // namespace
@@ -242,12 +241,19 @@ extern "C" int bikv_device_alloc_bounded(int device, int64_t bytes, int32_t plac
       return fail(BIKV_EHIP, "out of device memory: %zu bytes asked for (%zu chunks of %zu), %zu free, 2 GiB kept back",
                   (size_t)bytes, n, chunk, free_now);
   }
+  // Every chunk created, with the time of its pair probe against the first one (0 for the first chunk itself,
+  // and for everything when nothing is probed). A chunk's kind is judged against the SLOWEST pair seen — pairs
+  // inside the first chunk's half are the slow ones — and that reference only grows during the search, so kinds
+  // are always derived from the times, never stored: a chunk that looked "same" while only fast pairs had been
+  // seen (the driver handing out the other half first) turns into "other" as soon as a slow pair shows up.
+  std::vector<hipMemGenericAllocationHandle_t> all;     // every chunk created, in creation order
+  std::vector<float> pair_ms;                           // ... and the time of its pair probe
   std::vector<hipMemGenericAllocationHandle_t> same, other, fillers;
-  std::vector<float> same_ms;      // pair time of every chunk in `same` (0 for the reference chunk)
   Prober pr;
   int rc = BIKV_OK;
   auto cleanup = [&]() {
     pr.destroy();
+    release_all(all);
     release_all(same);
     release_all(other);
     release_all(fillers);
@@ -256,29 +262,29 @@ extern "C" int bikv_device_alloc_bounded(int device, int64_t bytes, int32_t plac
     rc = pr.init(device, chunk);
     if (rc) { cleanup(); return rc; }
   }
+  float ref_ms = 0;
   // Create chunks until both kinds are complete. Chunks beyond the wanted number of a kind are fillers:
   // they only push the driver's allocator on towards the other half and are released at the end. The
   // search ends with whatever balance was reached when a creation fails (memory exhausted) or the filler
   // budget is spent.
-  float ref_ms = 0, fastest_ms = 0;
   int n_reprobed = 0;
   size_t free_b = 0, total_b = 0;
-  while (same.size() < want_same || other.size() < want_other) {
-    if (fillers.size() >= max_fillers && (same.size() >= want_same || other.size() >= want_other)) break;
+  for (;;) {
+    const size_t n_other_now = count_other_chunks(pair_ms, ref_ms), n_same_now = all.size() - n_other_now;
+    if (n_same_now >= want_same && n_other_now >= want_other) break;
+    if (all.size() >= n && all.size() - n >= max_fillers) break;
     if (hipMemGetInfo(&free_b, &total_b) != hipSuccess || free_b < chunk + reserve) break;
     hipMemGenericAllocationHandle_t h;
     if (hipMemCreate(&h, chunk, &prop, 0) != hipSuccess) {
       (void)hipGetLastError();
       break;
     }
-    bool is_other = false;
-    float t_pair = 0;
+    float t = 0;
     if (pr.window) {
-      if (same.empty()) {
+      if (all.empty()) {
         rc = pr.map(0, h);           // the first chunk is the reference every candidate is paired with
       } else {
         rc = pr.map(1, h);
-        float t = 0;
         if (!rc) rc = pr.time_pair(&t);
         if (!rc && ref_ms > 0 && t > kBandLo * ref_ms && t < kBandHi * ref_ms) {
           // too close to call: two more probes, the median of the three decides
@@ -296,47 +302,29 @@ extern "C" int bikv_device_alloc_bounded(int device, int64_t bytes, int32_t plac
         // final mapping, and neither may happen while the window still maps it
         const int rc_unmap = pr.unmap(1);
         if (!rc) rc = rc_unmap;
-        if (!rc) {
-          if (t > ref_ms) ref_ms = t;            // pairs inside one half are the slow ones
-          is_other = t < kOtherBelow * ref_ms;
-          t_pair = t;
-          if (is_other && (fastest_ms == 0 || t < fastest_ms)) fastest_ms = t;
-        }
       }
       if (rc) {
-        (void)pr.unmap(0 + (same.empty() ? 0 : 1));
+        (void)pr.unmap(all.empty() ? 0 : 1);
         (void)hipMemRelease(h);
         break;
       }
+      if (t > ref_ms) ref_ms = t;                // pairs inside one half are the slow ones
     }
-    if (is_other) {
-      if (other.size() < want_other) other.push_back(h); else fillers.push_back(h);
-    } else if (same.size() < want_same) {
-      same.push_back(h);
-      same_ms.push_back(t_pair);
-    } else {
-      fillers.push_back(h);
-    }
+    all.push_back(h);
+    pair_ms.push_back(t);
   }
   if (pr.window) (void)pr.unmap(0);
   if (rc) { cleanup(); return rc; }
-  // The reference time only grows during the search: a chunk judged "same" against an early, too small
-  // reference (possible only while no same-half pair had been seen yet) is judged again against the final one.
-  for (size_t i = 1; i < same.size() && i < same_ms.size();) {
-    if (same_ms[i] > 0 && same_ms[i] < kOtherBelow * ref_ms) {
-      other.push_back(same[i]);
-      if (fastest_ms == 0 || same_ms[i] < fastest_ms) fastest_ms = same_ms[i];
-      same.erase(same.begin() + (long)i);
-      same_ms.erase(same_ms.begin() + (long)i);
-    } else {
-      ++i;
+  // Hand the chunks out by their final kinds (deal_chunks): the wanted number of each, what one kind lacks made
+  // up from the other's surplus (then from freshly created chunks), everything else released as fillers.
+  float fastest_ms = 0;
+  {
+    const std::vector<int> use = deal_chunks(pair_ms, ref_ms, want_same, want_other);
+    for (size_t i = 0; i < all.size(); ++i) {
+      if (chunk_is_other(pair_ms[i], ref_ms) && (fastest_ms == 0 || pair_ms[i] < fastest_ms)) fastest_ms = pair_ms[i];
+      (use[i] == CHUNK_OTHER ? other : use[i] == CHUNK_SAME ? same : fillers).push_back(all[i]);
     }
-  }
-  // what one kind lacks the other makes up (from the fillers, else freshly created), so that the
-  // allocation is complete
-  while (same.size() + other.size() < n && !fillers.empty()) {
-    same.push_back(fillers.back());
-    fillers.pop_back();
+    all.clear();
   }
   while (same.size() + other.size() < n) {
     hipMemGenericAllocationHandle_t h;

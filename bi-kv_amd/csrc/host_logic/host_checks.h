@@ -50,4 +50,45 @@ inline std::vector<bool> interleave_order(size_t n_same, size_t n_other) {
   return out;
 }
 
+// How bikv_device_alloc tells the two kinds of physical chunks apart and deals them out. Every chunk but the
+// first is probed as a pair with the first; a pair that straddles the two halves of HBM is faster than a pair
+// inside one half. The yardstick is the SLOWEST pair seen (`ref_ms`), which only grows while chunks are being
+// created: kinds are therefore derived from the times whenever they are needed and never stored, so that
+// chunks met before the first slow pair — the driver handing out the OTHER half first — are not stuck with the
+// kind they seemed to have then.
+constexpr float kOtherBelow = 0.92f;     // other half: pair time below 0.92 x the slowest pair time
+
+inline bool chunk_is_other(float pair_ms, float ref_ms) { return pair_ms > 0 && pair_ms < kOtherBelow * ref_ms; }
+
+inline size_t count_other_chunks(const std::vector<float>& pair_ms, float ref_ms) {
+  size_t k = 0;
+  for (float t : pair_ms) k += chunk_is_other(t, ref_ms) ? 1 : 0;
+  return k;
+}
+
+enum ChunkUse : int { CHUNK_SAME = 0, CHUNK_OTHER = 1, CHUNK_FILLER = 2 };
+
+// Deals the created chunks out for an allocation of n = want_same + want_other chunks: the wanted number of
+// each kind; what one kind lacks is made up from the other's surplus; the rest are fillers (released by the
+// caller). Fewer than n chunks in all: every chunk is used.
+inline std::vector<int> deal_chunks(const std::vector<float>& pair_ms, float ref_ms, size_t want_same, size_t want_other) {
+  std::vector<int> use(pair_ms.size(), CHUNK_FILLER);
+  size_t n_same = 0, n_other = 0;
+  for (size_t i = 0; i < pair_ms.size(); ++i) {
+    if (chunk_is_other(pair_ms[i], ref_ms)) {
+      if (n_other < want_other) { use[i] = CHUNK_OTHER; ++n_other; }
+    } else if (n_same < want_same) {
+      use[i] = CHUNK_SAME;
+      ++n_same;
+    }
+  }
+  const size_t n = want_same + want_other;
+  for (size_t i = 0; i < pair_ms.size() && n_same + n_other < n; ++i) {
+    if (use[i] != CHUNK_FILLER) continue;
+    if (chunk_is_other(pair_ms[i], ref_ms)) { use[i] = CHUNK_OTHER; ++n_other; }
+    else { use[i] = CHUNK_SAME; ++n_same; }
+  }
+  return use;
+}
+
 }  // namespace bikv

@@ -281,8 +281,102 @@ static void test_arena() {
   }
 }
 
+// The allocator's search for chunks of both kinds, replayed on the CPU with scripted halves: chunk k lies in
+// half halves[k] (the first chunk is the reference), a pair inside one half probes slow, a straddling pair
+// fast. The search creates chunks until it has want_same + want_other of the right kinds (or the script / the
+// filler budget ends) and deals them out. Whatever order the driver hands the halves out in, the result must
+// hold the wanted number of each kind whenever the script contains them.
+struct Dealt { size_t same_in_ref_half, same_in_other_half, other_in_ref_half, other_in_other_half, fillers, created; };
+static Dealt search_and_deal(const std::vector<int>& halves, size_t n, size_t max_fillers, std::mt19937_64& rng) {
+  const size_t want_other = n / 2, want_same = n - want_other;
+  std::vector<float> pair_ms;
+  float ref_ms = 0;
+  size_t k = 0;
+  for (;;) {
+    const size_t n_other = count_other_chunks(pair_ms, ref_ms), n_same = pair_ms.size() - n_other;
+    if (n_same >= want_same && n_other >= want_other) break;
+    if (pair_ms.size() >= n && pair_ms.size() - n >= max_fillers) break;
+    if (k >= halves.size()) break;                                   // "out of memory"
+    float t = 0;
+    if (k > 0) t = (halves[k] == halves[0] ? 0.382f : 0.319f) * (1.0f + 0.01f * (float)((int)(rng() % 5) - 2));
+    if (t > ref_ms) ref_ms = t;
+    pair_ms.push_back(t);
+    ++k;
+  }
+  const std::vector<int> use = deal_chunks(pair_ms, ref_ms, want_same, want_other);
+  Dealt d = {0, 0, 0, 0, 0, pair_ms.size()};
+  for (size_t i = 0; i < use.size(); ++i) {
+    const bool in_ref_half = halves[i] == halves[0];
+    if (use[i] == CHUNK_SAME) (in_ref_half ? d.same_in_ref_half : d.same_in_other_half)++;
+    else if (use[i] == CHUNK_OTHER) (in_ref_half ? d.other_in_ref_half : d.other_in_other_half)++;
+    else d.fillers++;
+  }
+  return d;
+}
+static void test_deal() {
+  std::mt19937_64 rng(11);
+  auto script = [](std::initializer_list<std::pair<int, int>> runs) {
+    std::vector<int> h;
+    for (auto& r : runs) h.insert(h.end(), (size_t)r.second, r.first);
+    return h;
+  };
+  // the usual order: the reference's half first, then the other
+  Dealt d = search_and_deal(script({{0, 40}, {1, 40}}), 18, 384, rng);
+  REQUIRE(d.same_in_ref_half == 9 && d.other_in_other_half == 9 && d.same_in_other_half == 0 && d.other_in_ref_half == 0,
+          "usual order: %zu/%zu", d.same_in_ref_half, d.other_in_other_half);
+  REQUIRE(d.fillers == 31 && d.created == 49, "fillers %zu created %zu", d.fillers, d.created);
+  // the reference is the last free chunk of its half: sixty chunks of the other half come first (all fast pairs,
+  // nothing to compare them with yet), then the reference's half again
+  d = search_and_deal(script({{0, 1}, {1, 60}, {0, 30}}), 18, 384, rng);
+  REQUIRE(d.same_in_ref_half == 9 && d.other_in_other_half == 9 && d.same_in_other_half == 0 && d.other_in_ref_half == 0,
+          "other half first: same %zu (+%zu misplaced), other %zu (+%zu misplaced)", d.same_in_ref_half, d.same_in_other_half,
+          d.other_in_other_half, d.other_in_ref_half);
+  // alternating halves: no fillers at all
+  {
+    std::vector<int> h;
+    for (int i = 0; i < 40; ++i) h.push_back(i & 1);
+    d = search_and_deal(h, 18, 384, rng);
+    REQUIRE(d.same_in_ref_half == 9 && d.other_in_other_half == 9 && d.fillers == 0, "alternating: fillers %zu", d.fillers);
+  }
+  // a filler budget that does not reach the other half: complete, all of one kind, nothing labelled "other"
+  d = search_and_deal(script({{0, 100}, {1, 40}}), 18, 10, rng);
+  REQUIRE(d.created == 28 && d.same_in_ref_half == 18 && d.other_in_other_half + d.other_in_ref_half == 0 && d.fillers == 10,
+          "budget: created %zu same %zu fillers %zu", d.created, d.same_in_ref_half, d.fillers);
+  // memory runs out with too few chunks of the reference's half: the other kind makes up the difference
+  d = search_and_deal(script({{0, 3}, {1, 40}}), 18, 384, rng);
+  REQUIRE(d.same_in_ref_half == 3 && d.other_in_other_half + d.same_in_other_half == 15 && d.fillers == 25,
+          "short half: same %zu other %zu fillers %zu", d.same_in_ref_half, d.other_in_other_half, d.fillers);
+  // an odd count and a single chunk
+  d = search_and_deal(script({{0, 10}, {1, 10}}), 7, 384, rng);
+  REQUIRE(d.same_in_ref_half == 4 && d.other_in_other_half == 3, "odd count");
+  d = search_and_deal(script({{0, 10}}), 1, 384, rng);
+  REQUIRE(d.same_in_ref_half == 1 && d.created == 1 && d.fillers == 0, "single chunk");
+  // random scripts: never more than wanted of a kind, every wanted chunk present when the script has it
+  for (int trial = 0; trial < 300; ++trial) {
+    std::vector<int> h;
+    const size_t len = 20 + rng() % 200;
+    int cur = 0;
+    while (h.size() < len) {
+      const size_t run = 1 + rng() % 40;
+      h.insert(h.end(), run, cur);
+      cur ^= 1;
+    }
+    const size_t n = 2 + rng() % 18;
+    size_t have_ref = 0, have_other = 0;
+    for (int x : h) (x == h[0] ? have_ref : have_other)++;
+    d = search_and_deal(h, n, ~size_t(0), rng);
+    const size_t want_other = n / 2, want_same = n - want_other;
+    REQUIRE(d.same_in_ref_half + d.same_in_other_half + d.other_in_ref_half + d.other_in_other_half == std::min(n, h.size()), "complete");
+    REQUIRE(d.other_in_ref_half == 0, "a chunk of the reference's half is never labelled other");
+    if (have_ref >= want_same && have_other >= want_other)
+      REQUIRE(d.same_in_ref_half == want_same && d.other_in_other_half == want_other,
+              "trial %d: same %zu of %zu, other %zu of %zu", trial, d.same_in_ref_half, want_same, d.other_in_other_half, want_other);
+  }
+}
+
 int main() {
   test_arena();
+  test_deal();
   test_planner();
   test_duplicates();
   test_interleave();
