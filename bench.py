@@ -429,10 +429,12 @@ TRAFFIC_SOURCE = "profiles/<kernel>_<workload>.md (rocprofv3 --pmc FETCH_SIZE an
 
 
 def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layout=None, steps=None,
-                       warmup=None, target_s=None, keep_pool=False, pool_form=None):
+                       warmup=None, target_s=None, keep_pool=False, pool_form=None, reuse=None):
     """One named configuration at full size: pool resident in HBM, one launch per direction (more when the
     staging image would exceed --staging-cap-gb), `steps` timed steps (or as many as fill `target_s`
-    seconds). Returns (json fragment, shape, workload, kept) — kept = (pool_t, pool) when keep_pool."""
+    seconds). Returns (json fragment, shape, workload, kept) — kept = (pool_t, pool) when keep_pool. `reuse` =
+    the kept pool of an earlier call on the same shape (planar, no scale class), taken over instead of
+    allocating the same pool once more."""
     import numpy as np
     import torch
 
@@ -446,8 +448,14 @@ def run_gather_scatter(args, bk, workloads, dev, with_copy=True, name=None, layo
     wl = workloads.named(name, shape)
     log(f"{name}: pool {shape.pool_bytes / 1e9:.2f} GB, tile {shape.tile_bytes} B x {shape.n_planes} planes, layout {layout}")
     pool_form = pool_form or args.pool_form
-    pool_t, scale_t = make_pool(shape, dev, args.pool_alloc, pool_form)
-    if pool_form == "worker":                       # second value = the per-layer tensors, not scale planes
+    if reuse is not None:
+        pool_t, pool = reuse
+        scale_t = None
+    else:
+        pool_t, scale_t = make_pool(shape, dev, args.pool_alloc, pool_form)
+    if reuse is not None:
+        pass
+    elif pool_form == "worker":                       # second value = the per-layer tensors, not scale planes
         pool, scale_t = bk.PagedKVPool.from_token_kv_layers(scale_t, shape.page_tokens), None
     else:
         pool = bk.PagedKVPool.from_planes(pool_t, scale_t)
@@ -1435,14 +1443,18 @@ def main():
         print(json.dumps({"metric": "pinned-host staging GB/s", "unit": "GB/s", "n_gpus": 1,
                           "staging": run_staging(args, bk, workloads, dev)}), flush=True)
         return
-    out, shape, wl, _ = run_gather_scatter(args, bk, workloads, dev)
+    same_pool_again = not args.no_other_layout and args.pool_form == "planar" and not workloads.SHAPES[args.workload].scales
+    out, shape, wl, kept = run_gather_scatter(args, bk, workloads, dev, keep_pool=same_pool_again)
     if knobs:
         out["config"]["tuning"] = knobs
     if not args.no_other_layout:
-        # the same request stream with the other staging image (reported next to the headline number)
+        # the same request stream with the other staging image (reported next to the headline number), on
+        # the same pool where that is possible
         alt_layout = "page_major" if args.layout == "layer_major" else "layer_major"
         log(f"same workload, staging layout {alt_layout}")
-        o2, _, _, _ = run_gather_scatter(args, bk, workloads, dev, with_copy=False, layout=alt_layout, target_s=0.6, warmup=3)
+        o2, _, _, _ = run_gather_scatter(args, bk, workloads, dev, with_copy=False, layout=alt_layout, target_s=0.6, warmup=3,
+                                         reuse=kept)
+        kept = None
         out["other_layout"] = {"layout": alt_layout, "value": o2["value"], "pct_of_hbm_peak": o2["pct_of_hbm_peak"],
                                "steps": o2["steps"], "kernels": {k: v for k, v in o2["kernels"].items() if v}}
     default_run = args.workload == "qwen2_7b" and not args.pool_pages
