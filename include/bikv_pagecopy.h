@@ -215,8 +215,9 @@ int bikv_scatter_pages(const bikv_pool* pool, const bikv_page_batch* batch,
  * gather kernel fills the lane's buffer with the next contiguous piece of the staging image, then one
  * hipMemcpyAsync per chunk_bytes moves it to `host_dst`, all in the lane's stream order, so the copies
  * of one lane overlap the kernel (and queued copies) of the others. Two lanes are enough to keep the
- * link busy; a HIP process has 4 hardware queues by default (GPU_MAX_HW_QUEUES) and its streams are dealt
- * onto them in turn, so a fourth lane shares a queue with another lane and runs in turn with it.
+ * link busy and are the steady choice: hipMemcpyAsync on three or four streams at once has whole passes at
+ * two thirds of the link's rate, and a HIP process has 4 hardware queues by default (GPU_MAX_HW_QUEUES), its
+ * streams dealt onto them in turn, so a fourth lane shares a queue with another lane.
  *
  * `req_pages` (HOST array, n_requests entries) gives the number of pages of each request; pages of
  * request r occupy batch entries [sum(req_pages[:r]), +req_pages[r]) and, in staging, a contiguous
