@@ -8,7 +8,11 @@
 #include <cstring>
 #include <thread>
 #include <vector>
+#include <map>
+#include <mutex>
+#include <sys/mman.h>
 
+#include "arena_logic.h"
 #include "ring_logic.h"
 
 using namespace bikv;
@@ -18,7 +22,83 @@ static void die(const char* what) {
   abort();
 }
 
+// The arena bookkeeping behind the torch allocator hooks, driven from four threads at once over a backend
+// that hands out address space only: every block a thread holds lies inside a live backend allocation and
+// overlaps no block of any other thread (each thread stamps its block's first and last byte address into a
+// shared map under its own lock and checks for intruders).
+static std::mutex g_backend_mu;
+static std::map<char*, int64_t> g_backend_live;
+static void* arena_backend_alloc(int, int64_t bytes) {
+  void* p = mmap(nullptr, (size_t)bytes, PROT_NONE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+  if (p == MAP_FAILED) die("mmap");
+  std::lock_guard<std::mutex> lk(g_backend_mu);
+  g_backend_live[(char*)p] = bytes;
+  return p;
+}
+static void arena_backend_free(void* base) {
+  int64_t bytes;
+  {
+    std::lock_guard<std::mutex> lk(g_backend_mu);
+    auto it = g_backend_live.find((char*)base);
+    if (it == g_backend_live.end()) die("release of memory the backend did not hand out");
+    bytes = it->second;
+    g_backend_live.erase(it);
+  }
+  munmap(base, (size_t)bytes);
+}
+static void arena_threads() {
+  bikv::arena::Book book(int64_t(2) << 30, arena_backend_alloc, arena_backend_free);
+  std::mutex held_mu;
+  std::map<char*, int64_t> held;                 // every block currently held by any thread
+  std::vector<std::thread> threads;
+  for (int t = 0; t < 4; ++t)
+    threads.emplace_back([&, t] {
+      uint64_t x = 88172645463325252ull + (uint64_t)t * 977;
+      auto rnd = [&] { x ^= x << 13; x ^= x >> 7; x ^= x << 17; return x; };
+      std::vector<std::pair<char*, int64_t>> mine;
+      for (int step = 0; step < 600; ++step) {
+        if (mine.empty() || rnd() % 3) {
+          const int64_t sz = (int64_t)(rnd() % 1300 + 1) << 20;          // some above half an arena
+          char* q = (char*)book.take((int)(rnd() % 2), sz);
+          if (!q) die("take failed");
+          const int64_t r = bikv::arena::round_up(sz, bikv::arena::kAlign);
+          {
+            std::lock_guard<std::mutex> lk(g_backend_mu);
+            auto it = g_backend_live.upper_bound(q);
+            if (it == g_backend_live.begin()) die("block below every backend allocation");
+            --it;
+            if (q + r > it->first + it->second) die("block sticks out of its backend allocation");
+          }
+          {
+            std::lock_guard<std::mutex> lk(held_mu);
+            auto nx = held.lower_bound(q);
+            if (nx != held.end() && q + r > nx->first) die("block overlaps another thread's block");
+            if (nx != held.begin()) { --nx; if (nx->first + nx->second > q) die("block overlaps another thread's block"); }
+            held[q] = r;
+          }
+          mine.emplace_back(q, r);
+        } else {
+          const size_t k = (size_t)(rnd() % mine.size());
+          { std::lock_guard<std::mutex> lk(held_mu); held.erase(mine[k].first); }
+          if (!book.give(mine[k].first)) die("give refused a live block");
+          mine.erase(mine.begin() + (long)k);
+        }
+      }
+      for (auto& b : mine) {
+        { std::lock_guard<std::mutex> lk(held_mu); held.erase(b.first); }
+        if (!book.give(b.first)) die("give refused a live block");
+      }
+    });
+  for (auto& th : threads) th.join();
+  if (book.live_blocks() != 0) die("blocks left behind");
+  std::lock_guard<std::mutex> lk(g_backend_mu);
+  if (g_backend_live.size() > 2) die("more than the two kept arenas (one per device) left with the backend");
+  for (auto& b : g_backend_live) munmap(b.first, (size_t)b.second);
+  g_backend_live.clear();
+}
+
 int main() {
+  arena_threads();
   const int kProducers = 3, kPerProducer = 400;
   const size_t kRing = 4096;
   bikv_shared_control* c = static_cast<bikv_shared_control*>(malloc(sizeof(bikv_shared_control)));
