@@ -1537,6 +1537,10 @@ def add_summary(out):
     sm = {"headline_value_GBps": out["value"],
           "headline_gather_frac": frac(out["kernels"]["gather"]["GBps"]),
           "headline_scatter_frac": frac(out["kernels"]["scatter"]["GBps"]) if out["kernels"]["scatter"] else None}
+    rf = out.get("roofline") or {}
+    if rf.get("traffic"):
+        sm["headline_traffic_over_algorithmic"] = round(rf["traffic"] / rf["alg_bytes_per_launch"], 4)
+        sm["headline_traffic_measured_in_this_run"] = "traffic_from_recorded_ratio" in rf
     if "other_layout" in out:
         sm["page_major_value_GBps"] = out["other_layout"]["value"]
     if "torch_alloc" in out:
