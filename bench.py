@@ -130,7 +130,7 @@ def traffic_from_counters(fetch, write, alg_bytes, copy_bytes=2 << 30):
     return round(fetched + written), note
 
 
-def measure_traffic_live(workload, dominant_kernel, alg_bytes, limit_s=150):
+def measure_traffic_live(workload, dominant_kernel, alg_bytes, limit_s=60):
     """HBM bytes per launch of `dominant_kernel`, measured now: this file is run twice more as a child process
     under `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE; one counter per run), on the same workload at full size
     with three timed steps. Each counter's mean per dispatch of the kernel is scaled by what the same counter
